@@ -1,0 +1,304 @@
+"""ctypes front end of the C oracle (oracle/vi_oracle.c) plus a pure-Python-int
+restatement of the same definitions.
+
+TEST INFRASTRUCTURE ONLY.  Two independent statements of every algorithm live here
+so that each can pin the other:
+
+  * `C.*`  -- the compiled scalar C restatement (fast enough for 2^16..2^26 sizes)
+  * `py_*` -- arbitrary-precision Python, written straight from the mathematical
+              definition (a*b % p, the DFT sum, the Lagrange closed form, the
+              sumcheck sum), usable only at toy sizes.
+
+Reference lines each function follows are cited in vi_oracle.c; the `py_*`
+functions cite theirs below.
+"""
+import ctypes
+import os
+import subprocess
+from ctypes import POINTER, c_double, c_int, c_size_t, c_uint64, c_uint8, c_void_p
+
+import numpy as np
+
+P = (1 << 64) - (1 << 32) + 1          # prover/protocol.py:27
+G = 7                                   # prover/protocol.py:28
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libvi_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile the C oracle in place (gcc, a second or two)."""
+    if force or not os.path.exists(_SO):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libvi_oracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_SO)
+        u64p, u8p, ip = POINTER(c_uint64), POINTER(c_uint8), POINTER(c_int)
+        for name in ("vo_add", "vo_sub", "vo_mul", "vo_pow"):
+            getattr(L, name).restype = c_uint64
+            getattr(L, name).argtypes = [c_uint64, c_uint64]
+        L.vo_inv.restype = c_uint64
+        L.vo_inv.argtypes = [c_uint64]
+        L.vo_root_of_unity.restype = c_uint64
+        L.vo_root_of_unity.argtypes = [c_uint64]
+        L.vo_binop_vec.argtypes = [c_int, u64p, u64p, u64p, c_size_t]
+        L.vo_ntt.argtypes = [u64p, c_size_t, c_int]
+        L.vo_ntt_rows.argtypes = [u64p, c_size_t, c_size_t, c_int]
+        L.vo_dft_naive.argtypes = [u64p, u64p, c_size_t, c_int]
+        L.vo_coset_lde_rows.argtypes = [u64p, c_size_t, c_size_t, c_size_t, c_size_t,
+                                        c_size_t, c_uint64, u64p]
+        L.vo_lagrange.restype = c_uint64
+        L.vo_lagrange.argtypes = [c_uint64, c_uint64, c_uint64]
+        L.vo_lde_dense_row.argtypes = [u64p, c_size_t, c_size_t, c_size_t, c_uint64, u64p]
+        L.vo_fold.argtypes = [u64p, c_size_t, c_uint64, u64p]
+        L.vo_sumcheck_prove.restype = c_int
+        L.vo_sumcheck_prove.argtypes = [POINTER(c_void_p), c_int, c_size_t, ip, ip, u64p,
+                                        c_int, u64p, u64p, u64p, u64p]
+        L.vo_kquant_to_field.restype = c_int
+        L.vo_kquant_to_field.argtypes = [c_int, u8p, c_size_t, c_double, u64p]
+        L.vo_num_threads.restype = c_int
+        _lib = L
+    return _lib
+
+
+def _p64(a: np.ndarray):
+    assert a.dtype == np.uint64 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(POINTER(c_uint64))
+
+
+def num_threads() -> int:
+    return int(lib().vo_num_threads())
+
+
+# ---------------------------------------------------------------- C oracle ----
+def binop(op: str, a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=np.uint64)
+    b = np.ascontiguousarray(b, dtype=np.uint64)
+    out = np.empty_like(a)
+    lib().vo_binop_vec({"add": 0, "sub": 1, "mul": 2}[op], _p64(a), _p64(b), _p64(out), a.size)
+    return out
+
+
+def ntt(a: np.ndarray, inverse: bool = False) -> np.ndarray:
+    out = np.array(a, dtype=np.uint64, copy=True)
+    lib().vo_ntt(_p64(out), out.size, int(inverse))
+    return out
+
+
+def ntt_rows(rows: np.ndarray, inverse: bool = False) -> np.ndarray:
+    out = np.array(rows, dtype=np.uint64, copy=True, order="C")
+    m, n = out.shape
+    lib().vo_ntt_rows(_p64(out), m, n, int(inverse))
+    return out
+
+
+def dft_naive(a: np.ndarray, inverse: bool = False) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=np.uint64)
+    out = np.empty_like(a)
+    lib().vo_dft_naive(_p64(a), _p64(out), a.size, int(inverse))
+    return out
+
+
+def coset_lde_rows(msgs: np.ndarray, K: int, N: int, shift: int = G) -> np.ndarray:
+    msgs = np.ascontiguousarray(msgs, dtype=np.uint64)
+    m, w = msgs.shape
+    out = np.empty((m, N), dtype=np.uint64)
+    lib().vo_coset_lde_rows(_p64(msgs), m, w, w, K, N, shift, _p64(out))
+    return out
+
+
+def lde_dense_row(msg: np.ndarray, K: int, N: int, shift: int = G) -> np.ndarray:
+    msg = np.ascontiguousarray(msg, dtype=np.uint64)
+    out = np.empty(N, dtype=np.uint64)
+    lib().vo_lde_dense_row(_p64(msg), msg.size, K, N, shift, _p64(out))
+    return out
+
+
+def fold(f: np.ndarray, r: int) -> np.ndarray:
+    f = np.ascontiguousarray(f, dtype=np.uint64)
+    out = np.empty(f.size // 2, dtype=np.uint64)
+    lib().vo_fold(_p64(f), f.size, r % P, _p64(out))
+    return out
+
+
+def sumcheck_prove(tables, terms, coins):
+    """tables: list of uint64 arrays of equal power-of-two length.
+    terms: list of (coeff, [table indices]).  coins: list of ints (one per round).
+    Returns (claim, samples[v][deg+1], finals[n_tables])."""
+    tabs = [np.ascontiguousarray(t, dtype=np.uint64) for t in tables]
+    size = tabs[0].size
+    v = size.bit_length() - 1
+    ptrs = (c_void_p * len(tabs))(*[t.ctypes.data for t in tabs])
+    off, idx = [0], []
+    for _, fs in terms:
+        idx.extend(fs)
+        off.append(len(idx))
+    deg = max(len(fs) for _, fs in terms)
+    off_a = (c_int * len(off))(*off)
+    idx_a = (c_int * max(len(idx), 1))(*idx)
+    co = np.array([c % P for c, _ in terms], dtype=np.uint64)
+    cn = np.array([c % P for c in coins[:v]] + [0] * max(0, 1 - v), dtype=np.uint64)
+    claim = c_uint64(0)
+    samples = np.zeros(max(v, 1) * (deg + 1), dtype=np.uint64)
+    finals = np.zeros(len(tabs), dtype=np.uint64)
+    lib().vo_sumcheck_prove(ptrs, len(tabs), size, off_a, idx_a, _p64(co), len(terms),
+                            _p64(cn), ctypes.byref(claim), _p64(samples), _p64(finals))
+    return (int(claim.value),
+            [[int(x) for x in samples[r * (deg + 1):(r + 1) * (deg + 1)]] for r in range(v)],
+            [int(x) for x in finals])
+
+
+QTYPE_ID = {"Q4_K": 4, "Q5_K": 5, "Q6_K": 6}
+BLOCK_BYTES = {"Q4_K": 144, "Q5_K": 176, "Q6_K": 210}
+
+
+def kquant_to_field(raw: np.ndarray, qtype: str, S: float) -> np.ndarray:
+    raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1)
+    nb = raw.size // BLOCK_BYTES[qtype]
+    assert nb * BLOCK_BYTES[qtype] == raw.size
+    out = np.empty(nb * 256, dtype=np.uint64)
+    rc = lib().vo_kquant_to_field(QTYPE_ID[qtype], raw.ctypes.data_as(POINTER(c_uint8)), nb,
+                                  float(S), _p64(out))
+    assert rc == 0
+    return out
+
+
+# ------------------------------------------------- pure-Python definitions ----
+def py_root(n: int) -> int:
+    """prover/ref/goldilocks_ref.py:45-49"""
+    assert (P - 1) % n == 0
+    return pow(G, (P - 1) // n, P)
+
+
+def py_dft(a, inverse: bool = False):
+    """X[k] = sum_j a[j] w^(jk)  (inverse: w^-1 and a 1/n factor)."""
+    n = len(a)
+    w = py_root(n)
+    if inverse:
+        w = pow(w, -1, P)
+    out = []
+    for k in range(n):
+        wk = pow(w, k, P)
+        acc, cur = 0, 1
+        for x in a:
+            acc += int(x) * cur
+            cur = cur * wk % P
+        out.append(acc % P)
+    if inverse:
+        ni = pow(n, -1, P)
+        out = [x * ni % P for x in out]
+    return out
+
+
+def py_lagrange(K: int, c: int, eta: int) -> int:
+    """prover/protocol.py:75-84"""
+    zc = pow(py_root(K), c, P)
+    return zc * (pow(eta, K, P) - 1) % P * pow(K * (eta - zc) % P, -1, P) % P
+
+
+def py_lde_dense(msg, K: int, N: int, shift: int = G):
+    """prover/protocol.py:86-93 with eta_j = shift * w_N^j (protocol.py:56-58)."""
+    wn = py_root(N)
+    out = []
+    for j in range(N):
+        eta = shift * pow(wn, j, P) % P
+        acc = 0
+        for c, v in enumerate(msg):
+            if v:
+                acc += int(v) * py_lagrange(K, c, eta)
+        out.append(acc % P)
+    return out
+
+
+def py_sumcheck(tables, terms, coins):
+    """Brute-force statement of layergkr/sumcheck.py:153-226 on Python ints.
+    Same argument/return shapes as `sumcheck_prove`."""
+    cur = [[int(x) % P for x in t] for t in tables]
+    size = len(cur[0])
+    deg = max(len(fs) for _, fs in terms)
+    claim = 0
+    for i in range(size):
+        for c, fs in terms:
+            prod = c % P
+            for j in fs:
+                prod = prod * cur[j][i] % P
+            claim += prod
+    claim %= P
+    samples, rnd = [], 0
+    while len(cur[0]) > 1:
+        half = len(cur[0]) // 2
+        row = []
+        for x in range(deg + 1):
+            acc = 0
+            for c, fs in terms:
+                for i in range(half):
+                    prod = c % P
+                    for j in fs:
+                        f = cur[j]
+                        prod = prod * ((f[i] + x * (f[half + i] - f[i])) % P) % P
+                    acc += prod
+            row.append(acc % P)
+        samples.append(row)
+        r = coins[rnd] % P
+        cur = [[(f[i] + r * (f[half + i] - f[i])) % P for i in range(half)] for f in cur]
+        rnd += 1
+    return claim, samples, [f[0] for f in cur]
+
+
+def py_mle_eval(values, point):
+    """layergkr/sumcheck.py:40-48"""
+    cur = [int(v) % P for v in values]
+    for r in point:
+        half = len(cur) // 2
+        cur = [(cur[i] + r * (cur[half + i] - cur[i])) % P for i in range(half)]
+    return cur[0] % P
+
+
+def np_kquant_to_field(raw: np.ndarray, qtype: str, S: float) -> np.ndarray:
+    """Vectorised numpy-float32 restatement of prover/kquant_cuda.py:42-111,
+    independent of the C one (array ops instead of a per-weight loop)."""
+    bb = BLOCK_BYTES[qtype]
+    blk = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, bb)
+    nb = blk.shape[0]
+    e = np.arange(256)
+    if qtype == "Q6_K":
+        ql, qh = blk[:, 0:128], blk[:, 128:192]
+        sc = blk[:, 192:208].view(np.int8)
+        d = blk[:, 208:210].copy().view(np.float16).astype(np.float32)          # (nb,1)
+        lo = (ql[:, (e >> 7) * 64 + (e & 63)] >> (4 * ((e >> 6) & 1))) & 0xF
+        hi = (qh[:, (e >> 7) * 32 + (e & 31)] >> (2 * ((e >> 5) & 3))) & 3
+        q = (lo | (hi << 4)).astype(np.int8).astype(np.int32) - 32
+        v = (d * sc[:, e >> 4].astype(np.float32)) * q.astype(np.float32)
+    else:
+        d = blk[:, 0:2].copy().view(np.float16).astype(np.float32)
+        dmin = blk[:, 2:4].copy().view(np.float16).astype(np.float32)
+        s12 = blk[:, 4:16].astype(np.uint32)
+        sc = np.empty((nb, 8), dtype=np.uint32)
+        mn = np.empty((nb, 8), dtype=np.uint32)
+        sc[:, :4] = s12[:, 0:4] & 0x3F
+        mn[:, :4] = s12[:, 4:8] & 0x3F
+        sc[:, 4:] = (s12[:, 8:12] & 0x0F) | ((s12[:, 0:4] >> 2) & 0x30)
+        mn[:, 4:] = (s12[:, 8:12] >> 4) | ((s12[:, 4:8] >> 2) & 0x30)
+        qs = blk[:, 16:144] if qtype == "Q4_K" else blk[:, 48:176]
+        q = ((qs[:, (e >> 6) * 32 + (e & 31)] >> (4 * ((e >> 5) & 1))) & 0xF).astype(np.int32)
+        if qtype == "Q5_K":
+            qhb = blk[:, 16:48]
+            q = q | (((qhb[:, e & 31] >> (e >> 5)) & 1).astype(np.int32) << 4)
+        scf = sc[:, e >> 5].astype(np.float32)
+        mnf = mn[:, e >> 5].astype(np.float32)
+        v = (d * scf) * q.astype(np.float32) - (dmin * mnf)
+    assert v.dtype == np.float32
+    x = np.rint(v.astype(np.float64) * np.float64(S)).astype(np.int64).reshape(-1)
+    out = x.astype(np.uint64)
+    neg = x < 0
+    out[neg] = np.uint64(P) - (-x[neg]).astype(np.uint64)
+    return out

@@ -1,0 +1,414 @@
+/*
+ * CPU oracle for the Goldilocks hot path -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load
+ * this library, and only as the checker / the timed CPU baseline.  Nothing in the
+ * shipped package may call into it.
+ *
+ * Every function restates, in plain scalar C, the algorithm of a reference file
+ * (cited per function as path:line under the upstream tree).  The restatement is
+ * deliberately the slow textbook form; independent pins (closed forms, brute
+ * force, invariants) live in tests/test_oracle_*.py.
+ *
+ * Parity status (what pins each function):
+ *   vo_add/vo_sub/vo_mul/vo_pow/vo_inv  pinned: Python big-int (a op b) % p, edge set
+ *   vo_ntt / vo_ntt_rows                pinned: O(n^2) DFT definition, golden n=1024 vector
+ *   vo_dft_naive                        pinned: is the definition (checked vs Python ints)
+ *   vo_coset_lde_rows                   pinned: Lagrange closed form (vo_lde_dense_row) + Python ints
+ *   vo_lde_dense_row / vo_lagrange      pinned: Python big-int evaluation of the closed form
+ *   vo_sumcheck_prove                   pinned: brute-force definition in Python ints, verifier identities
+ *   vo_kquant_to_field                  pinned against the reference kernel's byte map by an independent
+ *                                       numpy restatement and closed-form cases; agreement with the
+ *                                       third-party gguf-py 0.19.0 dequantiser is PARITY UNPINNED
+ *                                       (package and model file are not available offline).
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <stdlib.h>
+#include <string.h>
+#include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef uint64_t u64;
+typedef unsigned __int128 u128;
+
+#define GL_P   0xFFFFFFFF00000001ULL
+#define GL_EPS 0xFFFFFFFFULL
+
+/* ---- field: follows prover/kernels/goldilocks.cuh:28-81 ------------------- */
+
+/* goldilocks.cuh:28-48 -- (hi:lo) -> canonical residue via 2^64 = 2^32-1, 2^96 = -1 */
+static inline u64 reduce128(u64 lo, u64 hi) {
+    u64 top = hi >> 32, bot = hi & GL_EPS;
+    u64 t0 = lo - top;
+    if (lo < top) t0 -= GL_EPS;
+    u64 t1 = bot * GL_EPS;
+    u64 r = t0 + t1;
+    if (r < t0) r += GL_EPS;
+    if (r >= GL_P) r -= GL_P;
+    return r;
+}
+
+/* goldilocks.cuh:50-56 */
+u64 vo_add(u64 a, u64 b) {
+    u64 s = a + b;
+    if (s < a) s += GL_EPS;
+    if (s >= GL_P) s -= GL_P;
+    return s;
+}
+
+/* goldilocks.cuh:58-64 */
+u64 vo_sub(u64 a, u64 b) {
+    u64 d = a - b;
+    if (a < b) d -= GL_EPS;
+    return d;
+}
+
+/* goldilocks.cuh:66-70 */
+u64 vo_mul(u64 a, u64 b) {
+    u128 w = (u128)a * b;
+    return reduce128((u64)w, (u64)(w >> 64));
+}
+
+/* goldilocks.cuh:73-81 */
+u64 vo_pow(u64 base, u64 e) {
+    u64 r = 1;
+    while (e) {
+        if (e & 1) r = vo_mul(r, base);
+        base = vo_mul(base, base);
+        e >>= 1;
+    }
+    return r;
+}
+
+/* prover/protocol.py:34 -- Fermat inverse */
+u64 vo_inv(u64 a) { return vo_pow(a, GL_P - 2); }
+
+/* prover/ref/goldilocks_ref.py:45-49 -- primitive n-th root 7^((p-1)/n) */
+u64 vo_root_of_unity(u64 n) { return vo_pow(7, (GL_P - 1) / n); }
+
+void vo_binop_vec(int op, const u64 *a, const u64 *b, u64 *out, size_t n) {
+    for (size_t i = 0; i < n; ++i)
+        out[i] = op == 0 ? vo_add(a[i], b[i]) : op == 1 ? vo_sub(a[i], b[i]) : vo_mul(a[i], b[i]);
+}
+
+/* ---- NTT: follows prover/ref/goldilocks_ref.py:52-90 ---------------------- */
+
+/* in-place natural-order transform: X[k] = sum_j a[j] w^(jk), w = 7^((p-1)/n);
+ * the inverse uses w^-1 and multiplies by n^-1 (goldilocks_ref.py:71-90). */
+void vo_ntt(u64 *a, size_t n, int inverse) {
+    if (n < 2) return;
+    /* bit-reversal permutation, goldilocks_ref.py:60-69 */
+    for (size_t i = 1, j = 0; i < n; ++i) {
+        size_t bit = n >> 1;
+        for (; j & bit; bit >>= 1) j ^= bit;
+        j ^= bit;
+        if (i < j) { u64 t = a[i]; a[i] = a[j]; a[j] = t; }
+    }
+    u64 w_n = vo_root_of_unity(n);
+    for (size_t len = 2; len <= n; len <<= 1) {
+        u64 w_len = vo_pow(w_n, n / len);
+        if (inverse) w_len = vo_inv(w_len);
+        size_t half = len >> 1;
+        for (size_t i = 0; i < n; i += len) {
+            u64 w = 1;
+            for (size_t k = 0; k < half; ++k) {
+                u64 u = a[i + k], v = vo_mul(a[i + k + half], w);
+                a[i + k] = vo_add(u, v);
+                a[i + k + half] = vo_sub(u, v);
+                w = vo_mul(w, w_len);
+            }
+        }
+    }
+    if (inverse) {
+        u64 n_inv = vo_inv((u64)n % GL_P);
+        for (size_t i = 0; i < n; ++i) a[i] = vo_mul(a[i], n_inv);
+    }
+}
+
+/* same transform with the per-level twiddles tabulated once (used for the timed
+ * CPU baseline; identical arithmetic, identical results) */
+static void ntt_tab(u64 *a, size_t n, const u64 *tw /* w^k, k < n/2 */, u64 n_inv, int inverse) {
+    for (size_t i = 1, j = 0; i < n; ++i) {
+        size_t bit = n >> 1;
+        for (; j & bit; bit >>= 1) j ^= bit;
+        j ^= bit;
+        if (i < j) { u64 t = a[i]; a[i] = a[j]; a[j] = t; }
+    }
+    for (size_t len = 2; len <= n; len <<= 1) {
+        size_t half = len >> 1, step = n / len;
+        for (size_t i = 0; i < n; i += len)
+            for (size_t k = 0; k < half; ++k) {
+                u64 u = a[i + k], v = vo_mul(a[i + k + half], tw[k * step]);
+                a[i + k] = vo_add(u, v);
+                a[i + k + half] = vo_sub(u, v);
+            }
+    }
+    if (inverse)
+        for (size_t i = 0; i < n; ++i) a[i] = vo_mul(a[i], n_inv);
+}
+
+static u64 *make_twiddles(size_t n, int inverse) {
+    size_t h = n / 2 ? n / 2 : 1;
+    u64 *tw = (u64 *)malloc(h * sizeof(u64));
+    u64 w = vo_root_of_unity(n);
+    if (inverse) w = vo_inv(w);
+    u64 c = 1;
+    for (size_t k = 0; k < h; ++k) { tw[k] = c; c = vo_mul(c, w); }
+    return tw;
+}
+
+/* batched rows, prover/cuda_primitives.py:388-409 semantics (each row independently) */
+void vo_ntt_rows(u64 *a, size_t m, size_t n, int inverse) {
+    if (n < 2) return;
+    u64 *tw = make_twiddles(n, inverse);
+    u64 n_inv = vo_inv((u64)n % GL_P);
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < (long)m; ++r) ntt_tab(a + (size_t)r * n, n, tw, n_inv, inverse);
+    free(tw);
+}
+
+/* the definition itself, O(n^2) */
+void vo_dft_naive(const u64 *in, u64 *out, size_t n, int inverse) {
+    u64 w = vo_root_of_unity(n);
+    if (inverse) w = vo_inv(w);
+    u64 n_inv = vo_inv((u64)n % GL_P);
+    #pragma omp parallel for schedule(static)
+    for (long k = 0; k < (long)n; ++k) {
+        u64 wk = vo_pow(w, (u64)k), cur = 1, acc = 0;
+        for (size_t j = 0; j < n; ++j) {
+            acc = vo_add(acc, vo_mul(in[j], cur));
+            cur = vo_mul(cur, wk);
+        }
+        out[k] = inverse ? vo_mul(acc, n_inv) : acc;
+    }
+}
+
+/* ---- coset LDE ------------------------------------------------------------ */
+
+/* layergkr/gpu.py:141-203 (and prover/core.py:721-743): per row, values at w_K^c
+ * (slots [w,K) zero) -> iNTT_K -> times shift^i -> zero-extend to N -> NTT_N.
+ * `in` has m rows of w values with row pitch in_stride; out is (m, N) dense. */
+void vo_coset_lde_rows(const u64 *in, size_t m, size_t w, size_t in_stride,
+                       size_t K, size_t N, u64 shift, u64 *out) {
+    u64 *twi = make_twiddles(K, 1), *twf = make_twiddles(N, 0);
+    u64 k_inv = vo_inv((u64)K % GL_P);
+    u64 *gp = (u64 *)malloc(K * sizeof(u64));      /* gpu.py:128-138 */
+    u64 c = 1;
+    for (size_t i = 0; i < K; ++i) { gp[i] = c; c = vo_mul(c, shift); }
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < (long)m; ++r) {
+        u64 *row = out + (size_t)r * N;
+        memset(row, 0, N * sizeof(u64));
+        memcpy(row, in + (size_t)r * in_stride, w * sizeof(u64));
+        if (K >= 2) ntt_tab(row, K, twi, k_inv, 1);
+        for (size_t i = 0; i < K; ++i) row[i] = vo_mul(row[i], gp[i]);
+        if (N >= 2) ntt_tab(row, N, twf, 0, 0);
+    }
+    free(twi); free(twf); free(gp);
+}
+
+/* prover/protocol.py:75-84 -- L_c(eta) = zeta_c (eta^K - 1) / (K (eta - zeta_c)) */
+u64 vo_lagrange(u64 K, u64 c, u64 eta) {
+    u64 zc = vo_pow(vo_root_of_unity(K), c);
+    u64 num = vo_mul(zc, vo_sub(vo_pow(eta, K), 1));
+    u64 den = vo_mul(K % GL_P, vo_sub(eta, zc));
+    return vo_mul(num, vo_inv(den));
+}
+
+/* prover/protocol.py:86-93 + layergkr/rs.py:110-132: cw[j] = sum_c msg[c] L_c(eta_j),
+ * eta_j = shift * w_N^j (protocol.py:56-58).  O(w*N) field inversions: toy sizes only. */
+void vo_lde_dense_row(const u64 *msg, size_t w, size_t K, size_t N, u64 shift, u64 *out) {
+    u64 wn = vo_root_of_unity(N);
+    #pragma omp parallel for schedule(static)
+    for (long j = 0; j < (long)N; ++j) {
+        u64 eta = vo_mul(shift, vo_pow(wn, (u64)j)), acc = 0;
+        for (size_t c = 0; c < w; ++c)
+            if (msg[c]) acc = vo_add(acc, vo_mul(msg[c], vo_lagrange(K, c, eta)));
+        out[j] = acc;
+    }
+}
+
+/* ---- sumcheck: follows layergkr/sumcheck.py:153-226 ----------------------- */
+
+/* sumcheck.py:51-54 -- out[i] = f[i] + r (f[h+i] - f[i]), variable order MSB first */
+void vo_fold(const u64 *f, size_t len, u64 r, u64 *out) {
+    size_t h = len / 2;
+    #pragma omp parallel for schedule(static)
+    for (long i = 0; i < (long)h; ++i)
+        out[i] = vo_add(f[i], vo_mul(r, vo_sub(f[h + i], f[i])));
+}
+
+/* Sum-of-products sumcheck prover.
+ *   tables      n_tables pointers to tables of `size` = 2^v canonical values
+ *   term_off    n_terms+1 offsets into factor_idx; factors of term k are
+ *               tables[factor_idx[term_off[k] .. term_off[k+1])]
+ *   coeffs      n_terms coefficients
+ *   coins       v challenges (already reduced mod p), one per round
+ *   out_claim   sum over the cube (sumcheck.py:180-189), without any mask
+ *   out_samples v*(deg+1) values S_rnd(x), x = 0..deg (sumcheck.py:194-205)
+ *   out_final   n_tables fully folded values (each table folded by every challenge)
+ * The tables are copied; the caller's data is left untouched.  Returns deg. */
+int vo_sumcheck_prove(const u64 *const *tables, int n_tables, size_t size,
+                      const int *term_off, const int *factor_idx, const u64 *coeffs,
+                      int n_terms, const u64 *coins,
+                      u64 *out_claim, u64 *out_samples, u64 *out_final) {
+    int deg = 0;
+    for (int k = 0; k < n_terms; ++k) {
+        int nf = term_off[k + 1] - term_off[k];
+        if (nf > deg) deg = nf;
+    }
+    u64 **cur = (u64 **)malloc(sizeof(u64 *) * (size_t)n_tables);
+    for (int t = 0; t < n_tables; ++t) {
+        cur[t] = (u64 *)malloc(size * sizeof(u64));
+        memcpy(cur[t], tables[t], size * sizeof(u64));
+    }
+    /* claim */
+    u64 claim = 0;
+    #pragma omp parallel
+    {
+        u64 part = 0;
+        #pragma omp for schedule(static) nowait
+        for (long i = 0; i < (long)size; ++i)
+            for (int k = 0; k < n_terms; ++k) {
+                u64 prod = coeffs[k];
+                for (int j = term_off[k]; j < term_off[k + 1]; ++j)
+                    prod = vo_mul(prod, cur[factor_idx[j]][i]);
+                part = vo_add(part, prod);
+            }
+        #pragma omp critical
+        claim = vo_add(claim, part);
+    }
+    *out_claim = claim;
+
+    size_t len = size;
+    int rnd = 0;
+    while (len > 1) {
+        size_t half = len / 2;
+        for (int x = 0; x <= deg; ++x) {
+            u64 acc = 0;
+            #pragma omp parallel
+            {
+                u64 part = 0;
+                #pragma omp for schedule(static) nowait
+                for (long i = 0; i < (long)half; ++i)
+                    for (int k = 0; k < n_terms; ++k) {
+                        u64 prod = coeffs[k];
+                        for (int j = term_off[k]; j < term_off[k + 1]; ++j) {
+                            const u64 *f = cur[factor_idx[j]];
+                            u64 fx = vo_add(f[i], vo_mul((u64)x, vo_sub(f[half + i], f[i])));
+                            prod = vo_mul(prod, fx);
+                        }
+                        part = vo_add(part, prod);
+                    }
+                #pragma omp critical
+                acc = vo_add(acc, part);
+            }
+            out_samples[(size_t)rnd * (size_t)(deg + 1) + (size_t)x] = acc;
+        }
+        u64 r = coins[rnd];
+        for (int t = 0; t < n_tables; ++t) {
+            u64 *f = cur[t];
+            #pragma omp parallel for schedule(static)
+            for (long i = 0; i < (long)half; ++i)
+                f[i] = vo_add(f[i], vo_mul(r, vo_sub(f[half + i], f[i])));
+        }
+        len = half;
+        ++rnd;
+    }
+    for (int t = 0; t < n_tables; ++t) {
+        if (out_final) out_final[t] = cur[t][0];
+        free(cur[t]);
+    }
+    free(cur);
+    return deg;
+}
+
+/* ---- K-quant -> field: follows prover/kquant_cuda.py:42-111 ---------------- */
+
+/* IEEE binary16 -> binary32, exact (subnormals included) */
+static float half_to_float(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1Fu, m = h & 0x3FFu, bits;
+    if (e == 0) {
+        if (m == 0) bits = sign;
+        else {
+            int sh = 0;
+            while (!(m & 0x400u)) { m <<= 1; ++sh; }
+            bits = sign | ((uint32_t)(113 - sh) << 23) | ((m & 0x3FFu) << 13);
+        }
+    } else if (e == 31) bits = sign | 0x7F800000u | (m << 13);
+    else bits = sign | ((e + 112u) << 23) | (m << 13);
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* kquant_cuda.py:42-45 -- round-half-even of double(v)*S, negatives as p - |x| */
+static u64 to_field(float v, double S) {
+    long long ll = llrint((double)v * S);      /* default rounding mode: nearest-even */
+    return ll >= 0 ? (u64)ll : GL_P - (u64)(-ll);
+}
+
+/* kquant_cuda.py:48-58 */
+static void scale_min(const uint8_t *sc12, int s, uint32_t *sc, uint32_t *mn) {
+    if (s < 4) {
+        *sc = sc12[s] & 0x3F;
+        *mn = sc12[s + 4] & 0x3F;
+    } else {
+        int j = s - 4;
+        *sc = (sc12[8 + j] & 0x0F) | ((sc12[j] >> 2) & 0x30);
+        *mn = (sc12[8 + j] >> 4) | ((sc12[j + 4] >> 2) & 0x30);
+    }
+}
+
+static uint16_t rd16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+
+/* qtype: 4 = Q4_K (144 B), 5 = Q5_K (176 B), 6 = Q6_K (210 B); 256 weights per block.
+ * Compile with -ffp-contract=off: the fp32 expression is mul, mul, mul, sub with each
+ * result rounded (kquant_cuda.py:161-163). */
+int vo_kquant_to_field(int qtype, const uint8_t *raw, size_t n_blocks, double S, u64 *out) {
+    size_t bb = qtype == 4 ? 144 : qtype == 5 ? 176 : qtype == 6 ? 210 : 0;
+    if (!bb) return -1;
+    #pragma omp parallel for schedule(static)
+    for (long b = 0; b < (long)n_blocks; ++b) {
+        const uint8_t *p = raw + (size_t)b * bb;
+        u64 *o = out + (size_t)b * 256;
+        for (int e = 0; e < 256; ++e) {
+            volatile float v;
+            if (qtype == 6) {                                  /* kquant_cuda.py:95-111 */
+                const uint8_t *ql = p, *qh = p + 128;
+                const int8_t *sc = (const int8_t *)(p + 192);
+                float d = half_to_float(rd16(p + 208));
+                int lo = (ql[(e >> 7) * 64 + (e & 63)] >> (4 * ((e >> 6) & 1))) & 0xF;
+                int hi = (qh[(e >> 7) * 32 + (e & 31)] >> (2 * ((e >> 5) & 3))) & 3;
+                int q = (int)(int8_t)(lo | (hi << 4)) - 32;
+                volatile float t = d * (float)sc[e >> 4];
+                v = t * (float)q;
+            } else {                                           /* :60-74 and :76-93 */
+                float d = half_to_float(rd16(p)), dmin = half_to_float(rd16(p + 2));
+                uint32_t sc, mn;
+                scale_min(p + 4, e >> 5, &sc, &mn);
+                const uint8_t *qs = p + (qtype == 4 ? 16 : 48);
+                int q = (qs[(e >> 6) * 32 + (e & 31)] >> (4 * ((e >> 5) & 1))) & 0xF;
+                if (qtype == 5) q |= ((p[16 + (e & 31)] >> (e >> 5)) & 1) << 4;
+                volatile float t0 = d * (float)sc;
+                volatile float t1 = t0 * (float)q;
+                volatile float t2 = dmin * (float)mn;
+                v = t1 - t2;
+            }
+            o[e] = to_field(v, S);
+        }
+    }
+    return 0;
+}
+
+int vo_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
