@@ -1,0 +1,132 @@
+/*
+ * libverinf_hip -- C ABI of the MI355X (gfx950) Goldilocks prover kernels.
+ *
+ * Every entry point takes plain device pointers, sizes and a hipStream_t (passed
+ * as void*; NULL = the null stream), launches asynchronously on that stream and
+ * returns 0, or a negative VI_E* code after recording a message readable through
+ * vi_last_error().  Nothing throws across the boundary.  Unless stated otherwise
+ * an entry point allocates no device memory: scratch is passed in as a workspace
+ * whose size the matching *_workspace_bytes() query returns.  Twiddle tables are
+ * the exception: they are built once per (length, direction, device) on first use
+ * and cached for the life of the process, like the reference's NTT contexts.
+ *
+ * All field elements are uint64 words, canonical in [0, p), p = 2^64 - 2^32 + 1.
+ * "reference" below = JamesPetrie/VerInf; each entry point names the interface it
+ * replaces.
+ */
+#ifndef VERINF_HIP_H
+#define VERINF_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VI_OK 0
+#define VI_EINVAL (-1)   /* bad argument (shape, size, null pointer)   */
+#define VI_EHIP (-2)     /* a HIP runtime call failed                  */
+#define VI_ENOMEM (-3)   /* workspace too small                        */
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *vi_last_error(void);
+/* Library version, "major.minor". */
+const char *vi_version(void);
+
+/* ---- elementwise field ops --------------------------------------------------
+ * Replaces gl_mul / gl_add / gl_sub (prover/cuda_primitives.py:208-271, 1086-1088):
+ * out[i] = a[i] op b[i].  op: 0 add, 1 sub, 2 mul.  out may alias a or b. */
+int vi_gl_binop(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream);
+
+/* Same with a broadcast right operand: out[i] = a[i] op b[i % period].  Serves the
+ * coset twist gl_mul(coeffs, gamma^l expanded) of prover/core.py:736-739 and
+ * layergkr/gpu.py:198 without materialising the expanded operand. */
+int vi_gl_binop_bcast(int op, const uint64_t *a, const uint64_t *b, int64_t period, uint64_t *out,
+                      int64_t n, void *stream);
+
+/* Replaces gl_neg (cuda_primitives.py:272-280; gl_extras.cuh:22-28) and
+ * gl_pow / gl_inv / gl_inv_batched (cuda_primitives.py:281-303, 1089-1101):
+ * op 0: out = -a;  op 1: out = a^arg;  op 2: out = a^(p-2) (arg ignored). */
+int vi_gl_unop(int op, const uint64_t *a, uint64_t arg, uint64_t *out, int64_t n, void *stream);
+
+/* Replaces gl_axpy (cuda_primitives.py:282-288, 1104-1106; gl_extras.cuh:33-41):
+ * y[i] += alpha * x[i], in place. */
+int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *stream);
+
+/* Replaces layergkr/gpu.py:326-338 gl_sum: out[0] = sum of a[0..n) in the field.
+ * ws: vi_gl_sum_workspace_bytes(n) bytes of device scratch. */
+size_t vi_gl_sum_workspace_bytes(int64_t n);
+int vi_gl_sum(const uint64_t *a, int64_t n, uint64_t *out, void *ws, size_t ws_bytes, void *stream);
+
+/* ---- NTT ---------------------------------------------------------------------
+ * Replaces ntt_forward / ntt_inverse / ntt_forward_batched / ntt_inverse_batched
+ * (prover/cuda_primitives.py:347-409, 1111-1114; prover/kernels/ntt.cuh:667-770):
+ * in-place natural-order transform of each of the m contiguous rows of length n
+ * (a power of two >= 2): X[k] = sum_j x[j] w^(jk), w = 7^((p-1)/n); the inverse
+ * uses w^-1 and multiplies by n^-1.  Rows of more than 4096 elements need
+ * vi_ntt_workspace_bytes(m, n) bytes of scratch (0 otherwise). */
+size_t vi_ntt_workspace_bytes(int64_t m, int64_t n);
+int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, size_t ws_bytes,
+                   void *stream);
+
+/* ---- coset low-degree extension ------------------------------------------------
+ * Replaces the host recipe layergkr/gpu.py:141-203 (encode_batch_ntt) and
+ * prover/core.py:721-743 (_coset_encode_codewords after ntt_inverse_batched,
+ * core.py:798):  row r of `in` holds `width` <= K values of a polynomial at
+ * w_K^c (slots [width, K) read as zero);  row r of `out` receives its N values at
+ * shift * w_N^j.  K, N powers of two, 2 <= K <= N.  `in` rows are in_stride
+ * elements apart, `out` rows out_stride >= N.  in and out must not overlap.
+ * The workspace may be smaller than vi_coset_lde_workspace_bytes(m, K, N): rows
+ * are then processed in chunks; vi_coset_lde_min_workspace_bytes(K, N) is the
+ * least that is accepted (one row). */
+size_t vi_coset_lde_workspace_bytes(int64_t m, int64_t K, int64_t N);
+size_t vi_coset_lde_min_workspace_bytes(int64_t K, int64_t N);
+int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
+                 int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, void *ws,
+                 size_t ws_bytes, void *stream);
+
+/* ---- K-quant super-blocks -> field ---------------------------------------------
+ * Replaces q4k_to_field / q5k_to_field / q6k_to_field behind kquant_to_field
+ * (prover/kquant_cuda.py:60-139, 170-177): raw holds n_blocks super-blocks of
+ * 144 / 176 / 210 bytes (qtype 4 / 5 / 6); out receives n_blocks*256 field
+ * elements, round-half-even(double(fp32 dequant) * S), negatives as p - |x|. */
+int vi_kquant_to_field(int qtype, const uint8_t *raw, int64_t n_blocks, double S, uint64_t *out,
+                       void *stream);
+
+/* ---- multilinear sumcheck --------------------------------------------------------
+ * Replace the per-round torch composition of layergkr/gpu.py:341-410 (fold_t,
+ * gl_sum, prove_terms_gpu) with fused kernels.
+ *
+ * A problem is n_tables tables of `len` = 2*half values and n_terms terms; term k
+ * has coefficient coeffs[k] and factors tables[factor_idx[term_off[k] ..
+ * term_off[k+1])].  deg = the largest factor count.  For x = 0..deg
+ *   S(x) = sum_k coeffs[k] * sum_{i<half} prod_j (f_j[i] + x (f_j[half+i] - f_j[i])).
+ *
+ * The descriptor arrays (tables, term_off, factor_idx, coeffs) are HOST memory;
+ * they are passed to the kernel by value (limits: VI_SC_MAX_TABLES, VI_SC_MAX_TERMS,
+ * VI_SC_MAX_FACTORS).  out_samples: deg+1 device words.  ws: device scratch of
+ * vi_sumcheck_workspace_bytes() bytes. */
+#define VI_SC_MAX_TABLES 32
+#define VI_SC_MAX_TERMS 32
+#define VI_SC_MAX_FACTORS 64
+size_t vi_sumcheck_workspace_bytes(void);
+
+/* samples of the current round (sumcheck.py:194-205 / gpu.py:384-394) */
+int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
+                     const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                     uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream);
+
+/* fold every table by r (sumcheck.py:51-54 / gpu.py:341-347): dst[t][i] = src[t][i] +
+ * r (src[t][half+i] - src[t][i]), i < half; and, when half >= 2, also return the
+ * NEXT round's samples computed from the folded tables in the same pass.
+ * dst[t] may equal src[t] (fold in place).  out_samples may be NULL (fold only). */
+int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
+                          int64_t half, uint64_t r, const int *term_off, const int *factor_idx,
+                          const uint64_t *coeffs, int n_terms, uint64_t *out_samples, void *ws,
+                          size_t ws_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VERINF_HIP_H */

@@ -1,0 +1,83 @@
+// CPU build of the NTT / LDE pass logic (verinf_amd/csrc/ntt_pass.hpp, ntt_plan.hpp).
+// Runs every workgroup phase as a plain loop over thread ids, so the index maps,
+// twiddle tables and pass sequencing of the HIP kernels can be checked against the
+// oracle without a GPU.
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../verinf_amd/csrc/ntt_plan.hpp"
+
+using namespace ntt;
+
+namespace {
+
+struct Owned {
+    HostTables H;
+    std::vector<u64> twl;
+    Tables T;
+};
+
+Owned *make_owned(int logn, int inv) {
+    Owned *o = new Owned();
+    o->H = make_tables(logn, inv);
+    o->twl = make_twl(inv);
+    o->T.sp = o->H.sp;
+    o->T.logn = logn;
+    for (int q = 0; q < 3; ++q) o->T.tw[q] = o->H.tw[q].empty() ? nullptr : o->H.tw[q].data();
+    o->T.twl = o->twl.data();
+    o->T.scale = o->H.scale;
+    return o;
+}
+
+void run_pass(const PassArgs &A) {
+    i64 tiles = pass_tiles(A);
+    std::vector<u64> lds(LDS_WORDS);
+    std::vector<u64> regs((size_t)NTHREADS * EPT);
+    int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
+    for (i64 tile = 0; tile < tiles; ++tile) {
+        for (int tid = 0; tid < NTHREADS; ++tid)
+            ph_load(A, tile, tid, *reinterpret_cast<u64(*)[EPT]>(&regs[(size_t)tid * EPT]));
+        for (int t = 0; t < n_loop; ++t) {
+            for (int tid = 0; tid < NTHREADS; ++tid)
+                ph_stage(A, tile, tid, t, *reinterpret_cast<const u64(*)[EPT]>(&regs[(size_t)tid * EPT]), lds.data());
+            for (int s = 0; s < A.a; ++s)
+                for (int tid = 0; tid < NTHREADS; ++tid) ph_level(A, tid, s, lds.data());
+            for (int tid = 0; tid < NTHREADS; ++tid) ph_store(A, tile, tid, t, lds.data());
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
+u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
+u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }
+u64 emu_mul_pow2(u64 x, unsigned s) { return gl::mul_pow2(x, s); }
+
+int emu_ntt_batched(u64 *buf, long m, int logn, int inverse) {
+    Owned *o = make_owned(logn, inverse);
+    std::vector<u64> ws(o->T.sp.p > 1 ? (size_t)m << logn : 1);
+    std::vector<PassArgs> passes;
+    build_ntt_passes(o->T, buf, ws.data(), m, passes);
+    for (auto &A : passes) run_pass(A);
+    delete o;
+    return (int)passes.size();
+}
+
+int emu_coset_lde(const u64 *in, long m, long w, long in_stride, int logK, int logN, u64 shift,
+                  u64 *out) {
+    Owned *oi = make_owned(logK, 1), *of = make_owned(logK, 0);
+    std::vector<u64> pre = make_coset_pre(logK, logN, shift);
+    std::vector<u64> ws((size_t)lde_ws_elems(logK, logN, m));
+    std::vector<PassArgs> passes;
+    build_lde_passes(oi->T, of->T, pre.data(), logN, in, w, in_stride, out, (i64)1 << logN, ws.data(), m,
+                     passes);
+    for (auto &A : passes) run_pass(A);
+    delete oi;
+    delete of;
+    return (int)passes.size();
+}
+}

@@ -1,0 +1,137 @@
+"""No-GPU checks: the C-ABI library loads and exports every declared symbol, argument
+validation answers without touching a device, and the host-side logic of the
+package (domains, Lagrange form, verifier, mask algebra) is right."""
+import ctypes
+import os
+import random
+import re
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+P = O.P
+
+
+@pytest.fixture(scope="module")
+def L():
+    from verinf_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from verinf_amd.build import build
+        build()
+    return _lib.lib()
+
+
+def test_library_exports_every_declared_symbol(L):
+    hdr = open(os.path.join(ROOT, "include", "verinf_hip.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    names = sorted(set(re.findall(r"\b(vi_[a-z0-9_]+)\s*\(", hdr)))
+    assert len(names) >= 17
+    from verinf_amd import _lib
+    assert sorted(_lib.EXPORTS) == names
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), n
+    assert L.vi_version() == b"0.1"
+
+
+def test_size_queries_and_argument_validation_without_a_device(L):
+    assert L.vi_ntt_workspace_bytes(4, 1 << 12) == 0
+    assert L.vi_ntt_workspace_bytes(4, 1 << 16) == 4 * (1 << 16) * 8
+    assert L.vi_ntt_workspace_bytes(4, 12) == 0
+    one = L.vi_coset_lde_min_workspace_bytes(1 << 16, 1 << 18)
+    assert one == (1 << 16) * 8 * 5
+    assert L.vi_coset_lde_min_workspace_bytes(1 << 10, 1 << 12) == (1 << 10) * 8
+    assert L.vi_coset_lde_workspace_bytes(1024, 1 << 16, 1 << 18) % one == 0
+    assert L.vi_coset_lde_min_workspace_bytes(24, 96) == 0
+    assert L.vi_sumcheck_workspace_bytes() > 0
+    # bad arguments are refused before any HIP call
+    assert L.vi_gl_binop(7, None, None, None, 4, None) == -1 and b"op" in L.vi_last_error()
+    assert L.vi_ntt_batched(None, 1, 12, 0, None, 0, None) == -1 and b"power of 2" in L.vi_last_error()
+    assert L.vi_coset_lde(None, 1, 8, 8, 8, 4, 7, None, 4, None, 0, None) == -1
+    assert L.vi_coset_lde(None, 1, 9, 9, 8, 32, 7, None, 32, None, 0, None) == -1
+    assert L.vi_kquant_to_field(8, None, 1, 4096.0, None, None) == -1 and b"qtype" in L.vi_last_error()
+    assert L.vi_gl_binop(0, None, None, None, 0, None) == 0
+    assert L.vi_ntt_batched(None, 0, 16, 0, None, 0, None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from verinf_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libverinf_hip.so")
+    with pytest.raises(_lib.VerinfHipError):
+        _lib.lib()
+
+
+def test_no_gpu_means_an_error_not_a_cpu_path():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from verinf_amd.layergkr import gpu, rs, sumcheck
+    cfg = rs.Config(ELL=16, K_DEG=32, N_LIG=64, T_QUERIES=4)
+    with pytest.raises(RuntimeError):
+        gpu.encode_batch_ntt(cfg, [[1, 2, 3]])
+    with pytest.raises(RuntimeError):
+        rs.Commit.from_messages(cfg, [[1, 2, 3]])
+    with pytest.raises(RuntimeError):
+        sumcheck.prove([[1, 2], [3, 4]], lambda i: 5)
+    with pytest.raises(RuntimeError):
+        gpu.prove_terms_gpu([(1, [[1, 2], [3, 4]])], lambda i: 5, P)
+
+
+def test_product_package_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "verinf_amd")
+    pat = re.compile(r"^\s*(from|import)\s+oracle\b|#include.*oracle|vi_oracle|libvi_oracle", re.M)
+    for dp, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                assert not pat.search(open(os.path.join(dp, f)).read()), (dp, f)
+
+
+def test_protocol_domains_and_lagrange_form():
+    from verinf_amd.prover import protocol as pr
+    cfg = pr.Config(ELL=16, K_DEG=32, N_LIG=64, T_QUERIES=4)
+    assert pow(cfg.W_K, 32, P) == 1 and pow(cfg.W_K, 16, P) == P - 1
+    assert cfg.eta(0) == 7 and cfg.zeta(1) == cfg.W_K
+    r = random.Random(3)
+    msg = [r.randrange(P) for _ in range(16)]
+    want = O.lde_dense_row(np.array(msg, dtype=np.uint64), 32, 64, 7)
+    for j in (0, 1, 17, 63):
+        assert pr.eval_zeta_form(cfg, msg, cfg.eta(j)) == int(want[j])
+    assert pr.lagrange(cfg, 5, cfg.eta(9)) == O.py_lagrange(32, 5, cfg.eta(9))
+    assert pr.poly_eval([1, 2, 3], 5) == 1 + 10 + 75 and pr.inv(7) * 7 % P == 1
+
+
+def test_host_verifier_accepts_oracle_proofs_and_rejects_tampering():
+    from verinf_amd.layergkr import sumcheck as sc
+    r = random.Random(4)
+    n = 32
+    tabs = [[r.randrange(P) for _ in range(n)] for _ in range(3)]
+    terms_idx = [(3, [0, 1, 2]), (P - 1, [1]), (9, [2, 2])]
+    coins = [r.randrange(P) for _ in range(5)]
+    claim, samples, _ = O.py_sumcheck(tabs, terms_idx, coins)
+    terms = [(c, [tabs[i] for i in fs]) for c, fs in terms_idx]
+    pf = sc.SumcheckProof(claim=claim, round_polys=[list(enumerate(s)) for s in samples],
+                          challenges=list(coins), final_point=list(coins))
+    ok, why = sc.verify_terms(pf, terms, lambda i: coins[i])
+    assert ok, why
+    pf.round_polys[2][1] = (1, (pf.round_polys[2][1][1] + 1) % P)
+    assert not sc.verify_terms(pf, terms, lambda i: coins[i])[0]
+    assert sc.mle_eval(tabs[0], coins) == O.py_mle_eval(tabs[0], coins)
+    assert sc._fold([1, 2, 3, 4], 5) == [11, 12]
+    for d in (1, 2, 3, 4):
+        mu = r.randrange(P)
+        u = [r.randrange(P) for _ in range(d)]
+        h = sc.mask_poly_coeffs(mu, u)
+        assert (sc.poly_eval_coeffs(h, 0) + sc.poly_eval_coeffs(h, 1)) % P == mu
+        assert sc.solve_tape_for_target(mu, h) == u
+        bad = list(h)
+        bad[0] = (bad[0] + 1) % P
+        assert sc.solve_tape_for_target(mu, bad) is None
+    assert sc.masked_product_ok(3, 4, 5, 6, 7)
+    tp = sc.MaskTape([1, 2, 3])
+    assert tp.take(2) == [1, 2]
+    with pytest.raises(RuntimeError):
+        tp.take(2)

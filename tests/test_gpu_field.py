@@ -1,0 +1,116 @@
+"""GPU parity: elementwise field ops through the C ABI vs the oracle (bit-exact)."""
+import json
+import os
+import random
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+from oracle import oracle as O  # noqa: E402
+from tests.gpu_util import P, rand_field, to_dev, to_np, unhex  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def cp():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from verinf_amd.prover import cuda_primitives
+    return cuda_primitives
+
+
+def test_golden_field_vectors(cp, golden_dir):
+    vec = json.load(open(os.path.join(golden_dir, "field_vectors.json")))
+    a, b = to_dev(unhex([v["a"] for v in vec])), to_dev(unhex([v["b"] for v in vec]))
+    assert np.array_equal(to_np(cp.gl_add(a, b)), unhex([v["add"] for v in vec]))
+    assert np.array_equal(to_np(cp.gl_sub(a, b)), unhex([v["sub"] for v in vec]))
+    assert np.array_equal(to_np(cp.gl_mul(a, b)), unhex([v["mul"] for v in vec]))
+
+
+@pytest.mark.parametrize("n", [1, 2, 257, 4096, 1000003])
+def test_binops_match_oracle(cp, n):
+    a, b = rand_field(n, 1), rand_field(n, 2)
+    da, db = to_dev(a), to_dev(b)
+    for name, fn in (("add", cp.gl_add), ("sub", cp.gl_sub), ("mul", cp.gl_mul)):
+        assert np.array_equal(to_np(fn(da, db)), O.binop(name, a, b)), name
+
+
+def test_binops_on_noncanonical_words_match_reference_formulas(cp):
+    """Words >= p: the device functions return the same word as the reference's
+    (the oracle restates those formulas), so even these agree bit for bit."""
+    r = random.Random(3)
+    vals = [P, P + 1, (1 << 64) - 1, (1 << 64) - 2, P - 1, 0, 1] + [r.randrange(1 << 64) for _ in range(500)]
+    a = np.array([r.choice(vals) for _ in range(4099)], dtype=np.uint64)
+    b = np.array([r.choice(vals) for _ in range(4099)], dtype=np.uint64)
+    da, db = to_dev(a), to_dev(b)
+    for name, fn in (("add", cp.gl_add), ("sub", cp.gl_sub), ("mul", cp.gl_mul)):
+        assert np.array_equal(to_np(fn(da, db)), O.binop(name, a, b)), name
+
+
+def test_unaligned_views_and_2d_shapes(cp):
+    a, b = rand_field(2001, 4), rand_field(2001, 5)
+    da, db = to_dev(a)[1:], to_dev(b)[1:]                 # 8-byte aligned only
+    assert np.array_equal(to_np(cp.gl_mul(da.contiguous(), db.contiguous())), O.binop("mul", a[1:], b[1:]))
+    a2, b2 = rand_field((7, 33), 6), rand_field((7, 33), 7)
+    out = cp.gl_add(to_dev(a2), to_dev(b2))
+    assert out.shape == (7, 33)
+    assert np.array_equal(to_np(out), O.binop("add", a2.reshape(-1), b2.reshape(-1)).reshape(7, 33))
+
+
+def test_neg_pow_inv_axpy(cp):
+    r = random.Random(1)
+    a_cpu = [0, 1, P - 1] + [r.randrange(P) for _ in range(254)]
+    a = to_dev(np.array(a_cpu, dtype=np.uint64))
+    assert to_np(cp.gl_neg(a)).tolist() == [(P - x) % P for x in a_cpu]
+    assert to_np(cp.gl_pow(a, 12345)).tolist() == [pow(x, 12345, P) for x in a_cpu]
+    assert to_np(cp.gl_pow(a, 0)).tolist() == [1] * len(a_cpu)
+    nz = [x for x in a_cpu if x]
+    d = to_dev(np.array(nz, dtype=np.uint64))
+    want = [pow(x, -1, P) for x in nz]
+    assert to_np(cp.gl_inv(d)).tolist() == want
+    assert to_np(cp.gl_inv_batched(d)).tolist() == want
+    assert torch.equal(cp.gl_mul(d, cp.gl_inv_batched(d)), torch.ones_like(d))
+    y_cpu, x_cpu = [r.randrange(P) for _ in range(4096)], [r.randrange(P) for _ in range(4096)]
+    alpha = r.randrange(P)
+    y, x = to_dev(np.array(y_cpu, dtype=np.uint64)), to_dev(np.array(x_cpu, dtype=np.uint64))
+    cp.gl_axpy(y, alpha, x)
+    assert to_np(y).tolist() == [(yy + alpha * xx) % P for yy, xx in zip(y_cpu, x_cpu)]
+
+
+def test_mul_bcast_is_the_expanded_product(cp):
+    a, row = rand_field((13, 64), 8), rand_field(64, 9)
+    got = cp.gl_mul_bcast(to_dev(a), to_dev(row))
+    want = O.binop("mul", a.reshape(-1), np.tile(row, 13)).reshape(13, 64)
+    assert np.array_equal(to_np(got), want)
+
+
+def test_argument_errors_raise_runtime_error(cp):
+    a = to_dev(rand_field(8, 1))
+    with pytest.raises(RuntimeError):
+        cp.gl_mul(a, to_dev(rand_field(9, 1)))
+    with pytest.raises(RuntimeError):
+        cp.gl_mul(a.cpu(), a.cpu())
+    with pytest.raises(RuntimeError):
+        cp.gl_add(a, a.view(torch.int64))
+    with pytest.raises(RuntimeError):
+        cp.gl_add(to_dev(rand_field((4, 4), 1)).view(torch.int64).t().view(torch.uint64), to_dev(rand_field((4, 4), 2)))
+    with pytest.raises(RuntimeError):
+        cp.gl_inv_batched(to_dev(rand_field((2, 2), 1)))
+    with pytest.raises(RuntimeError):
+        cp.ntt_forward(to_dev(rand_field(12, 1)))
+    with pytest.raises(RuntimeError):
+        cp.ntt_forward_batched(to_dev(rand_field(16, 1)))
+
+
+def test_gl_sum_and_fold_t():
+    from verinf_amd.layergkr import gpu
+    for n in (1, 2, 3, 255, 4096, 1 << 20, (1 << 20) + 7):
+        a = rand_field(n, 10 + n % 7)
+        want = int(np.sum(a.astype(object)) % P) if n <= 4096 else sum(int(x) for x in a) % P
+        assert int(gpu.gl_sum(to_dev(a)).cpu()[0].item()) == want
+    f = rand_field(1 << 12, 11)
+    r = 0x123456789ABCDEF1 % P
+    got = gpu.fold_t(to_dev(f), torch.tensor([r], dtype=torch.uint64).cuda())
+    assert np.array_equal(to_np(got), O.fold(f, r))
+    assert np.array_equal(to_np(gpu.fold_t(to_dev(f), r)), O.fold(f, r))

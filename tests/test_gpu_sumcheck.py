@@ -1,0 +1,190 @@
+"""GPU parity: sumcheck round kernels through the C ABI vs the oracle (bit-exact
+samples per round, challenges, claim) and the host verifier."""
+import json
+import os
+import random
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+from oracle import oracle as O  # noqa: E402
+from tests.gpu_util import P, rand_field, to_dev, to_np, unhex  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def mods():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from verinf_amd.layergkr import gpu, sumcheck
+    return gpu, sumcheck
+
+
+def _coins(n, seed):
+    r = random.Random(seed)
+    vals = [r.randrange(P) for _ in range(n)]
+    return vals, (lambda i: vals[i])
+
+
+def _check(gpu, tables_np, terms_idx, seed, as_tensor):
+    """Run the device prover on (tables, terms) and compare with the C oracle."""
+    v = tables_np[0].size.bit_length() - 1
+    coins, coin = _coins(max(v, 1), seed)
+    objs = [to_dev(t) if as_tensor else [int(x) for x in t] for t in tables_np]
+    terms = [(c, [objs[i] for i in fs]) for c, fs in terms_idx]
+    claim, polys, chals, mu = gpu.prove_terms_gpu(terms, coin, P)
+    want_claim, want_samples, _ = O.sumcheck_prove(tables_np, terms_idx, coins)
+    assert claim == want_claim
+    assert chals == coins[:v]
+    assert [[y for _, y in s] for s in polys] == want_samples
+    assert all([x for x, _ in s] == list(range(len(s))) for s in polys)
+    assert mu == 0
+    if as_tensor:
+        for t, o in zip(tables_np, objs):
+            assert np.array_equal(to_np(o), t), "caller's tensor was modified"
+
+
+def test_sumcheck_golden(mods, golden_dir):
+    gpu, _ = mods
+    for g in json.load(open(os.path.join(golden_dir, "sumcheck.json"))):
+        tables = [[int(x, 16) for x in t] for t in g["tables"]]
+        terms = [(int(c, 16), [tables[i] for i in fs]) for c, fs in g["terms"]]
+        coins = [int(c, 16) for c in g["coins"]]
+        claim, polys, chals, _ = gpu.prove_terms_gpu(terms, lambda i: coins[i], P)
+        assert claim == int(g["claim"], 16), g["name"]
+        assert [[y for _, y in s] for s in polys] == [[int(x, 16) for x in s] for s in g["samples"]], g["name"]
+        assert chals == coins[:len(polys)]
+
+
+@pytest.mark.parametrize("v", [1, 2, 3, 6, 9, 10, 13, 17])
+@pytest.mark.parametrize("nf", [1, 2, 3, 4])
+def test_single_product_matches_oracle(mods, v, nf):
+    gpu, _ = mods
+    tabs = [rand_field(1 << v, 10 * v + j) for j in range(nf)]
+    _check(gpu, tabs, [(1, list(range(nf)))], 99, as_tensor=(v % 2 == 1))
+
+
+def test_sum_of_products_shared_tables_and_coefficients(mods):
+    gpu, _ = mods
+    r = random.Random(6)
+    tabs = [rand_field(1 << 11, 40 + j) for j in range(5)]
+    terms = [(r.randrange(P), [0, 1, 2]), (P - 1, [3]), (5, [1, 1]), (7, [0, 3]), (r.randrange(P), [0, 4, 4])]
+    _check(gpu, tabs, terms, 7, as_tensor=True)
+    _check(gpu, tabs, terms, 8, as_tensor=False)
+    # the reference's relation shapes: hadamard a*b - c, booleanity b*b - b, each times eq
+    eq, a, b, c = (rand_field(1 << 9, 50 + j) for j in range(4))
+    _check(gpu, [eq, a, b, c], [(11, [0, 1, 2]), (P - 11, [0, 3]), (13, [0, 2, 2]), (P - 13, [0, 2])], 9, True)
+
+
+def test_more_tables_than_fit_in_registers(mods):
+    gpu, _ = mods
+    r = random.Random(12)
+    tabs = [rand_field(1 << 8, 60 + j) for j in range(11)]
+    terms = [(r.randrange(P), [j, (j + 1) % 11]) for j in range(11)] + [(3, [0, 5, 10])]
+    _check(gpu, tabs, terms, 13, as_tensor=True)
+
+
+def test_degree_above_three_and_limits(mods):
+    gpu, _ = mods
+    tabs = [rand_field(1 << 7, 70 + j) for j in range(6)]
+    _check(gpu, tabs, [(1, [0, 1, 2, 3, 4, 5]), (2, [0])], 14, as_tensor=True)
+    with pytest.raises(RuntimeError):
+        obj = [to_dev(t) for t in tabs]
+        gpu.prove_terms_gpu([(1, [obj[0]] * 8)], lambda i: 1, P)          # degree 8 is above the kernel limit
+
+
+def test_large_instance_matches_oracle(mods):
+    """2^22 x 3 factors, degree 3, 22 rounds: every round's samples against the C oracle."""
+    gpu, _ = mods
+    tabs = [rand_field(1 << 22, 80 + j) for j in range(3)]
+    _check(gpu, tabs, [(1, [0, 1, 2])], 15, as_tensor=True)
+
+
+def test_prove_verify_masked_and_tamper(mods):
+    """The reference's sumcheck gates (layergkr/tests/test_sumcheck.py) on the device prover."""
+    gpu, sc = mods
+    assert sc._sumcheck_gpu_ok()
+    N_VARS = 4
+
+    def factors(k, seed):
+        r = random.Random(seed)
+        return [[r.randrange(P) for _ in range(1 << N_VARS)] for _ in range(k)]
+
+    def coin():
+        r = random.Random(99)
+        vals = [r.randrange(P) for _ in range(N_VARS)]
+        return lambda i: vals[i]
+
+    def tape(n, seed=5):
+        r = random.Random(seed)
+        return sc.MaskTape([r.randrange(P) for _ in range(n)])
+
+    for k, seed in ((2, 17), (3, 23)):
+        f = factors(k, seed)
+        proof = sc.prove(f, coin())
+        ok, why = sc.verify(proof, f, coin())
+        assert ok, why
+    f = factors(2, 17)
+    bare = sc.prove(f, coin())
+    masked = sc.prove(f, coin(), tape=tape(2 * N_VARS), mu0=123456789)
+    ok, why = sc.verify(masked, f, coin())
+    assert ok, why
+    assert masked.claim == (bare.claim + 123456789) % P
+    assert masked.round_polys[0] != bare.round_polys[0]
+    # tamper cases
+    p1 = sc.prove(f, coin())
+    p1.claim = (p1.claim + 1) % P
+    ok, why = sc.verify(p1, f, coin())
+    assert not ok and "claim" in why
+    p2 = sc.prove(f, coin())
+    x, y = p2.round_polys[1][0]
+    p2.round_polys[1][0] = (x, (y + 1) % P)
+    assert not sc.verify(p2, f, coin())[0]
+    p3 = sc.prove(f, coin())
+    p3.challenges[2] = (p3.challenges[2] + 1) % P
+    ok, why = sc.verify(p3, f, coin())
+    assert not ok and "challenge" in why
+    for tp, mu0 in ((None, 0), (tape(2 * N_VARS), 4242)):
+        pf = sc.prove(f, coin(), tape=tp, mu0=mu0)
+        bad = [list(f[0]), list(f[1])]
+        bad[0][3] = (bad[0][3] + 1) % P
+        ok, why = sc.verify(pf, bad, coin())
+        assert not ok and "terminal" in why
+    with pytest.raises(RuntimeError):
+        sc.prove(f, coin(), tape=tape(2), mu0=1)
+    # masked device proof == oracle samples + host mask polynomial
+    tp = tape(2 * N_VARS)
+    vals = list(tp.values)
+    pf = sc.prove(f, coin(), tape=tp, mu0=77)
+    coins = [coin()(i) for i in range(N_VARS)]
+    _, samples, _ = O.sumcheck_prove([np.array(t, dtype=np.uint64) for t in f], [(1, [0, 1])], coins)
+    mu = 77
+    for rnd in range(N_VARS):
+        h = sc.mask_poly_coeffs(mu, vals[2 * rnd:2 * rnd + 2])
+        assert [y for _, y in pf.round_polys[rnd]] == [(samples[rnd][x] + sc.poly_eval_coeffs(h, x)) % P for x in range(3)]
+        mu = sc.poly_eval_coeffs(h, coins[rnd])
+    assert pf.final_mask == mu
+
+
+def test_fold_eval_in_place_c_abi(mods):
+    """vi_sumcheck_fold_eval with dst == src (fold in place) against the oracle."""
+    import ctypes
+    from verinf_amd import _lib
+    L = _lib.lib()
+    tabs = [rand_field(1 << 12, 90 + j) for j in range(3)]
+    dev = [to_dev(t) for t in tabs]
+    r = 0xDEADBEEFCAFEF00D % P
+    ptrs = (ctypes.c_void_p * 3)(*[t.data_ptr() for t in dev])
+    off = (ctypes.c_int * 2)(0, 3)
+    idx = (ctypes.c_int * 3)(0, 1, 2)
+    co = (ctypes.c_uint64 * 1)(1)
+    out = torch.zeros(4, dtype=torch.uint64, device="cuda")
+    ws = torch.empty(L.vi_sumcheck_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    _lib.check(L.vi_sumcheck_fold_eval(ptrs, ptrs, 3, 1 << 11, r, off, idx, co, 1, out.data_ptr(),
+                                       ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    folded = [O.fold(t, r) for t in tabs]
+    for t, f in zip(dev, folded):
+        assert np.array_equal(to_np(t)[: 1 << 11], f)
+    _, samples, _ = O.sumcheck_prove(folded, [(1, [0, 1, 2])], [0] * 11)
+    assert [int(x) for x in out.cpu().tolist()] == samples[0]

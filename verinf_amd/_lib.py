@@ -1,0 +1,102 @@
+"""ctypes binding of libverinf_hip.so (C ABI: include/verinf_hip.h).
+
+The library is built ahead of time by `python -m verinf_amd.build`; loading fails
+loudly if it is missing.  torch is imported first on purpose: its bundled HIP
+runtime must be the one the library binds to, so that tensor pointers and stream
+handles mean the same thing on both sides.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_double, c_int, c_int64, c_size_t, c_uint64, c_void_p
+
+import torch  # noqa: F401  (must precede the CDLL below)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libverinf_hip.so")
+
+EXPORTS = [
+    "vi_last_error", "vi_version",
+    "vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy",
+    "vi_gl_sum_workspace_bytes", "vi_gl_sum",
+    "vi_ntt_workspace_bytes", "vi_ntt_batched",
+    "vi_coset_lde_workspace_bytes", "vi_coset_lde_min_workspace_bytes", "vi_coset_lde",
+    "vi_kquant_to_field",
+    "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval",
+]
+
+_lib = None
+
+
+class VerinfHipError(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded library with argument types declared."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise VerinfHipError(
+            f"{LIB_PATH} is missing: build it with `python -m verinf_amd.build` "
+            "(there is no CPU fallback)")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i64, u64, sz = c_void_p, c_int64, c_uint64, c_size_t
+    ip = POINTER(c_int)
+    L.vi_last_error.restype = c_char_p
+    L.vi_version.restype = c_char_p
+    L.vi_gl_binop.argtypes = [c_int, vp, vp, vp, i64, vp]
+    L.vi_gl_binop_bcast.argtypes = [c_int, vp, vp, i64, vp, i64, vp]
+    L.vi_gl_unop.argtypes = [c_int, vp, u64, vp, i64, vp]
+    L.vi_gl_axpy.argtypes = [vp, u64, vp, i64, vp]
+    L.vi_gl_sum_workspace_bytes.restype = sz
+    L.vi_gl_sum_workspace_bytes.argtypes = [i64]
+    L.vi_gl_sum.argtypes = [vp, i64, vp, vp, sz, vp]
+    L.vi_ntt_workspace_bytes.restype = sz
+    L.vi_ntt_workspace_bytes.argtypes = [i64, i64]
+    L.vi_ntt_batched.argtypes = [vp, i64, i64, c_int, vp, sz, vp]
+    L.vi_coset_lde_workspace_bytes.restype = sz
+    L.vi_coset_lde_workspace_bytes.argtypes = [i64, i64, i64]
+    L.vi_coset_lde_min_workspace_bytes.restype = sz
+    L.vi_coset_lde_min_workspace_bytes.argtypes = [i64, i64]
+    L.vi_coset_lde.argtypes = [vp, i64, i64, i64, i64, i64, u64, vp, i64, vp, sz, vp]
+    L.vi_kquant_to_field.argtypes = [c_int, vp, i64, c_double, vp, vp]
+    L.vi_sumcheck_workspace_bytes.restype = sz
+    L.vi_sumcheck_workspace_bytes.argtypes = []
+    L.vi_sumcheck_eval.argtypes = [POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int, vp, vp, sz, vp]
+    L.vi_sumcheck_fold_eval.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, u64, ip, ip,
+                                        POINTER(u64), c_int, vp, vp, sz, vp]
+    for name in EXPORTS:
+        getattr(L, name)                     # AttributeError here = stale build
+    for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
+                 "vi_ntt_batched", "vi_coset_lde", "vi_kquant_to_field", "vi_sumcheck_eval",
+                 "vi_sumcheck_fold_eval"):
+        getattr(L, name).restype = c_int
+    _lib = L
+    return L
+
+
+def check(rc: int) -> None:
+    """Turn a negative C-ABI return code into an exception carrying vi_last_error()."""
+    if rc != 0:
+        msg = lib().vi_last_error().decode("utf-8", "replace")
+        raise VerinfHipError(f"libverinf_hip error {rc}: {msg}")
+
+
+def stream_ptr() -> int:
+    """hipStream_t of torch's current stream (kernels are queued behind torch's own work)."""
+    return torch.cuda.current_stream().cuda_stream
+
+
+_ws_cache = {}
+
+
+def workspace(nbytes: int, device=None, tag: str = "ws"):
+    """A cached uint8 device buffer of at least nbytes (grown, never shrunk)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    key = (tag, device.index)
+    buf = _ws_cache.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _ws_cache[key] = buf
+    return buf

@@ -1,0 +1,188 @@
+// Elementwise Goldilocks kernels and the field sum reduction.
+//
+// All of these are pure HBM streaming (24 B per element for a binary op) with a
+// handful of integer VALU ops per element; they use 64-bit indexing and a
+// grid-stride loop sized to keep every CU busy (the reference kernels index with
+// int, prover/cuda_primitives.py:208-233).
+#include "common.hpp"
+#include "gl_field.hpp"
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int MAX_BLOCKS = 256 * 16;      // 16 workgroups per CU
+
+inline unsigned grid_for(i64 n) {
+    i64 b = (n + BLOCK - 1) / BLOCK;
+    return (unsigned)(b < 1 ? 1 : (b > MAX_BLOCKS ? MAX_BLOCKS : b));
+}
+
+template <int OP>
+__device__ __forceinline__ u64 apply(u64 a, u64 b) {
+    return OP == 0 ? gl::add(a, b) : OP == 1 ? gl::sub(a, b) : gl::mul(a, b);
+}
+
+template <int OP>
+__global__ __launch_bounds__(BLOCK) void k_binop(const u64 *a, const u64 *b, u64 *out, i64 n) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) out[i] = apply<OP>(a[i], b[i]);
+}
+
+// two elements per lane through 16-byte accesses (operands 16-byte aligned, n even)
+template <int OP>
+__global__ __launch_bounds__(BLOCK) void k_binop_v2(const ulonglong2 *a, const ulonglong2 *b, ulonglong2 *out, i64 n2) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n2; i += stride) {
+        ulonglong2 x = a[i], y = b[i], r;
+        r.x = apply<OP>(x.x, y.x);
+        r.y = apply<OP>(x.y, y.y);
+        out[i] = r;
+    }
+}
+
+template <int OP>
+__global__ __launch_bounds__(BLOCK) void k_binop_bcast(const u64 *a, const u64 *b, i64 period, u64 *out, i64 n) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) out[i] = apply<OP>(a[i], b[i % period]);
+}
+
+__global__ __launch_bounds__(BLOCK) void k_unop(int op, const u64 *a, u64 arg, u64 *out, i64 n) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) {
+        u64 v = a[i];
+        out[i] = op == 0 ? gl::neg(v) : gl::pow(v, arg);
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void k_axpy(u64 *y, u64 alpha, const u64 *x, i64 n) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) y[i] = gl::add(y[i], gl::mul(alpha, x[i]));
+}
+
+__device__ __forceinline__ u64 wave_sum(u64 v) {
+    for (int off = 32; off > 0; off >>= 1) v = gl::add(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// block-wide field sum; the result is valid in thread 0
+__device__ __forceinline__ u64 block_sum(u64 v, u64 *lds4) {
+    v = wave_sum(v);
+    int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) lds4[w] = v;
+    __syncthreads();
+    u64 r = 0;
+    if (threadIdx.x == 0) {
+        r = lds4[0];
+        for (int i = 1; i < BLOCK / 64; ++i) r = gl::add(r, lds4[i]);
+    }
+    __syncthreads();
+    return r;
+}
+
+constexpr int SUM_BLOCKS = 1024;
+
+__global__ __launch_bounds__(BLOCK) void k_sum_partial(const u64 *a, i64 n, u64 *partial) {
+    __shared__ u64 lds4[BLOCK / 64];
+    i64 stride = (i64)gridDim.x * BLOCK;
+    u64 acc = 0;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) {
+        u64 v = a[i];
+        acc = gl::add(acc, v >= gl::P ? v - gl::P : v);
+    }
+    u64 r = block_sum(acc, lds4);
+    if (threadIdx.x == 0) partial[blockIdx.x] = r;
+}
+
+__global__ __launch_bounds__(BLOCK) void k_sum_final(const u64 *partial, int nb, u64 *out) {
+    __shared__ u64 lds4[BLOCK / 64];
+    u64 acc = 0;
+    for (int i = threadIdx.x; i < nb; i += BLOCK) acc = gl::add(acc, partial[i]);
+    u64 r = block_sum(acc, lds4);
+    if (threadIdx.x == 0) out[0] = r;
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+const char *vi_last_error(void) { return vi::err_buf(); }
+const char *vi_version(void) { return "0.1"; }
+
+int vi_gl_binop(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream) {
+    if (op < 0 || op > 2) return vi::fail(VI_EINVAL, "vi_gl_binop: op %d", op);
+    if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_binop: n = %lld", (long long)n);
+    if (n == 0) return VI_OK;
+    if (!a || !b || !out) return vi::fail(VI_EINVAL, "vi_gl_binop: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if ((n & 1) == 0 && aligned16(a) && aligned16(b) && aligned16(out)) {
+        i64 n2 = n / 2;
+        auto A = (const ulonglong2 *)a, B = (const ulonglong2 *)b;
+        auto O = (ulonglong2 *)out;
+        if (op == 0) hipLaunchKernelGGL(k_binop_v2<0>, dim3(grid_for(n2)), dim3(BLOCK), 0, s, A, B, O, n2);
+        if (op == 1) hipLaunchKernelGGL(k_binop_v2<1>, dim3(grid_for(n2)), dim3(BLOCK), 0, s, A, B, O, n2);
+        if (op == 2) hipLaunchKernelGGL(k_binop_v2<2>, dim3(grid_for(n2)), dim3(BLOCK), 0, s, A, B, O, n2);
+    } else {
+        if (op == 0) hipLaunchKernelGGL(k_binop<0>, dim3(grid_for(n)), dim3(BLOCK), 0, s, a, b, out, (i64)n);
+        if (op == 1) hipLaunchKernelGGL(k_binop<1>, dim3(grid_for(n)), dim3(BLOCK), 0, s, a, b, out, (i64)n);
+        if (op == 2) hipLaunchKernelGGL(k_binop<2>, dim3(grid_for(n)), dim3(BLOCK), 0, s, a, b, out, (i64)n);
+    }
+    VI_LAUNCH_CHECK("k_binop");
+    return VI_OK;
+}
+
+int vi_gl_binop_bcast(int op, const uint64_t *a, const uint64_t *b, int64_t period, uint64_t *out,
+                      int64_t n, void *stream) {
+    if (op < 0 || op > 2) return vi::fail(VI_EINVAL, "vi_gl_binop_bcast: op %d", op);
+    if (n < 0 || period <= 0) return vi::fail(VI_EINVAL, "vi_gl_binop_bcast: n = %lld period = %lld", (long long)n, (long long)period);
+    if (n == 0) return VI_OK;
+    if (!a || !b || !out) return vi::fail(VI_EINVAL, "vi_gl_binop_bcast: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (op == 0) hipLaunchKernelGGL(k_binop_bcast<0>, dim3(grid_for(n)), dim3(BLOCK), 0, s, a, b, (i64)period, out, (i64)n);
+    if (op == 1) hipLaunchKernelGGL(k_binop_bcast<1>, dim3(grid_for(n)), dim3(BLOCK), 0, s, a, b, (i64)period, out, (i64)n);
+    if (op == 2) hipLaunchKernelGGL(k_binop_bcast<2>, dim3(grid_for(n)), dim3(BLOCK), 0, s, a, b, (i64)period, out, (i64)n);
+    VI_LAUNCH_CHECK("k_binop_bcast");
+    return VI_OK;
+}
+
+int vi_gl_unop(int op, const uint64_t *a, uint64_t arg, uint64_t *out, int64_t n, void *stream) {
+    if (op < 0 || op > 2) return vi::fail(VI_EINVAL, "vi_gl_unop: op %d", op);
+    if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_unop: n = %lld", (long long)n);
+    if (n == 0) return VI_OK;
+    if (!a || !out) return vi::fail(VI_EINVAL, "vi_gl_unop: null pointer");
+    if (op == 2) { op = 1; arg = gl::P - 2; }
+    hipLaunchKernelGGL(k_unop, dim3(grid_for(n)), dim3(BLOCK), 0, (hipStream_t)stream, op, a, (u64)arg, out, (i64)n);
+    VI_LAUNCH_CHECK("k_unop");
+    return VI_OK;
+}
+
+int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *stream) {
+    if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_axpy: n = %lld", (long long)n);
+    if (n == 0) return VI_OK;
+    if (!y || !x) return vi::fail(VI_EINVAL, "vi_gl_axpy: null pointer");
+    hipLaunchKernelGGL(k_axpy, dim3(grid_for(n)), dim3(BLOCK), 0, (hipStream_t)stream, y, (u64)alpha, x, (i64)n);
+    VI_LAUNCH_CHECK("k_axpy");
+    return VI_OK;
+}
+
+size_t vi_gl_sum_workspace_bytes(int64_t n) {
+    (void)n;
+    return SUM_BLOCKS * sizeof(u64);
+}
+
+int vi_gl_sum(const uint64_t *a, int64_t n, uint64_t *out, void *ws, size_t ws_bytes, void *stream) {
+    if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_sum: n = %lld", (long long)n);
+    if (!out || (n > 0 && !a)) return vi::fail(VI_EINVAL, "vi_gl_sum: null pointer");
+    if (!ws || ws_bytes < SUM_BLOCKS * sizeof(u64)) return vi::fail(VI_ENOMEM, "vi_gl_sum: workspace below %zu bytes", SUM_BLOCKS * sizeof(u64));
+    i64 b = (n + BLOCK - 1) / BLOCK;
+    int nb = (int)(b < 1 ? 1 : (b > SUM_BLOCKS ? SUM_BLOCKS : b));
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_sum_partial, dim3(nb), dim3(BLOCK), 0, s, a, (i64)n, (u64 *)ws);
+    VI_LAUNCH_CHECK("k_sum_partial");
+    hipLaunchKernelGGL(k_sum_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, out);
+    VI_LAUNCH_CHECK("k_sum_final");
+    return VI_OK;
+}
+
+}  // extern "C"

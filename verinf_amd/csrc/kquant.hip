@@ -1,0 +1,142 @@
+// Fused K-quant super-block -> Goldilocks field decode.
+//
+// The value map is the one the reference declares to be the committed model
+// (prover/kquant_cuda.py:42-111): fp16 d/dmin widened to fp32, the fp32 expression
+// (d*sc)*q - dmin*mn (Q4_K, Q5_K) or (d*sc)*q (Q6_K) with every operation rounded
+// separately (no FMA contraction -- this file is built with -ffp-contract=off and
+// uses the explicit round-to-nearest intrinsics), then round-half-even of
+// double(v)*S, negatives stored as p - |x|.
+//
+// k_q4k: one wavefront per 256-weight super-block.  Lane l decodes weights
+// {2l, 2l+1} and {128+2l, 129+2l}: it needs two 16-bit quant loads, the 4-byte
+// d/dmin header and the 12 scale bytes (three dwords, identical for all lanes of the
+// wave), and issues two 16-byte stores, so each store instruction writes 1 KiB of
+// consecutive output.  The reference uses one thread per weight with byte loads.
+//
+// k_generic: one thread per weight, byte loads, any alignment (Q5_K, Q6_K, and
+// Q4_K buffers that are not 4-byte aligned).
+#include "common.hpp"
+#include "gl_field.hpp"
+
+namespace {
+
+constexpr int BLOCK = 256;
+
+__device__ __forceinline__ float half_bits_to_float(u32 bits) {
+    _Float16 h = __builtin_bit_cast(_Float16, (unsigned short)bits);
+    return (float)h;
+}
+
+__device__ __forceinline__ u64 to_field(float v, double S) {
+    long long x = __double2ll_rn(__dmul_rn((double)v, S));
+    return x >= 0 ? (u64)x : gl::P - (u64)(-x);
+}
+
+// 6-bit (scale, min) of sub-block s from the 12 packed bytes held as three dwords
+__device__ __forceinline__ void scale_min(u32 w0, u32 w1, u32 w2, int s, u32 &sc, u32 &mn) {
+    // bytes 0..3 = w0, 4..7 = w1, 8..11 = w2
+    int j = s & 3, sh = 8 * j;
+    u32 b_lo = (w0 >> sh) & 0xFF, b_mid = (w1 >> sh) & 0xFF, b_hi = (w2 >> sh) & 0xFF;
+    if (s < 4) {
+        sc = b_lo & 0x3F;
+        mn = b_mid & 0x3F;
+    } else {
+        sc = (b_hi & 0x0F) | ((b_lo >> 2) & 0x30);
+        mn = (b_hi >> 4) | ((b_mid >> 2) & 0x30);
+    }
+}
+
+__device__ __forceinline__ float dequant(float d, float dmin, u32 sc, u32 mn, u32 q) {
+    return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)sc), (float)q), __fmul_rn(dmin, (float)mn));
+}
+
+__global__ __launch_bounds__(BLOCK) void k_q4k(const unsigned char *__restrict__ raw, u64 *__restrict__ out, i64 n_blocks, double S) {
+    const int lane = threadIdx.x & 63;
+    const i64 wave = ((i64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const i64 n_waves = ((i64)gridDim.x * BLOCK) >> 6;
+    for (i64 b = wave; b < n_blocks; b += n_waves) {
+        const unsigned char *p = raw + b * 144;
+        const u32 *hdr = (const u32 *)p;
+        u32 h = hdr[0], w0 = hdr[1], w1 = hdr[2], w2 = hdr[3];
+        float d = half_bits_to_float(h & 0xFFFF), dmin = half_bits_to_float(h >> 16);
+        int s = lane >> 4;                                  // sub-block of weights 2l, 2l+1
+        int nib = 4 * (s & 1);
+        const unsigned short *qs = (const unsigned short *)(p + 16 + (lane >> 5) * 32 + ((2 * lane) & 31));
+        u32 qa = qs[0], qb = qs[32];                        // +64 bytes: same position, sub-block s+4
+        u32 sc, mn;
+        ulonglong2 r;
+        scale_min(w0, w1, w2, s, sc, mn);
+        r.x = to_field(dequant(d, dmin, sc, mn, (qa >> nib) & 0xF), S);
+        r.y = to_field(dequant(d, dmin, sc, mn, (qa >> (8 + nib)) & 0xF), S);
+        ulonglong2 *o = (ulonglong2 *)(out + b * 256);
+        o[lane] = r;
+        scale_min(w0, w1, w2, s + 4, sc, mn);
+        r.x = to_field(dequant(d, dmin, sc, mn, (qb >> nib) & 0xF), S);
+        r.y = to_field(dequant(d, dmin, sc, mn, (qb >> (8 + nib)) & 0xF), S);
+        o[64 + lane] = r;
+    }
+}
+
+template <int QT>
+__global__ __launch_bounds__(BLOCK) void k_generic(const unsigned char *__restrict__ raw, u64 *__restrict__ out, i64 n, double S) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 idx = (i64)blockIdx.x * BLOCK + threadIdx.x; idx < n; idx += stride) {
+        i64 b = idx >> 8;
+        int e = (int)(idx & 255);
+        float v;
+        if (QT == 6) {
+            const unsigned char *p = raw + b * 210;
+            float d = half_bits_to_float((u32)p[208] | ((u32)p[209] << 8));
+            int lo = (p[(e >> 7) * 64 + (e & 63)] >> (4 * ((e >> 6) & 1))) & 0xF;
+            int hi = (p[128 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e >> 5) & 3))) & 3;
+            int q = (int)(signed char)(lo | (hi << 4)) - 32;
+            int sc = (int)(signed char)p[192 + (e >> 4)];
+            v = __fmul_rn(__fmul_rn(d, (float)sc), (float)q);
+        } else {
+            const unsigned char *p = raw + b * (QT == 4 ? 144 : 176);
+            float d = half_bits_to_float((u32)p[0] | ((u32)p[1] << 8));
+            float dmin = half_bits_to_float((u32)p[2] | ((u32)p[3] << 8));
+            int s = e >> 5;
+            u32 sc, mn;
+            if (s < 4) {
+                sc = p[4 + s] & 0x3F;
+                mn = p[8 + s] & 0x3F;
+            } else {
+                int j = s - 4;
+                sc = (p[12 + j] & 0x0F) | ((p[4 + j] >> 2) & 0x30);
+                mn = (p[12 + j] >> 4) | ((p[8 + j] >> 2) & 0x30);
+            }
+            const unsigned char *qs = p + (QT == 4 ? 16 : 48);
+            u32 q = (qs[(e >> 6) * 32 + (e & 31)] >> (4 * ((e >> 5) & 1))) & 0xF;
+            if (QT == 5) q |= (u32)((p[16 + (e & 31)] >> (e >> 5)) & 1) << 4;
+            v = dequant(d, dmin, sc, mn, q);
+        }
+        out[idx] = to_field(v, S);
+    }
+}
+
+inline unsigned grid_cap(i64 blocks_needed, i64 cap) {
+    return (unsigned)(blocks_needed < 1 ? 1 : (blocks_needed > cap ? cap : blocks_needed));
+}
+
+}  // namespace
+
+extern "C" int vi_kquant_to_field(int qtype, const uint8_t *raw, int64_t n_blocks, double S, uint64_t *out, void *stream) {
+    if (qtype != 4 && qtype != 5 && qtype != 6) return vi::fail(VI_EINVAL, "vi_kquant_to_field: unsupported qtype %d", qtype);
+    if (n_blocks < 0) return vi::fail(VI_EINVAL, "vi_kquant_to_field: n_blocks = %lld", (long long)n_blocks);
+    if (n_blocks == 0) return VI_OK;
+    if (!raw || !out) return vi::fail(VI_EINVAL, "vi_kquant_to_field: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    const i64 n = n_blocks * 256;
+    if (qtype == 4 && ((uintptr_t)raw & 3) == 0 && ((uintptr_t)out & 15) == 0) {
+        unsigned g = grid_cap((n_blocks + 3) / 4, 256 * 32);
+        hipLaunchKernelGGL(k_q4k, dim3(g), dim3(BLOCK), 0, s, raw, out, (i64)n_blocks, S);
+    } else {
+        unsigned g = grid_cap((n + BLOCK - 1) / BLOCK, 256 * 32);
+        if (qtype == 4) hipLaunchKernelGGL(k_generic<4>, dim3(g), dim3(BLOCK), 0, s, raw, out, n, S);
+        if (qtype == 5) hipLaunchKernelGGL(k_generic<5>, dim3(g), dim3(BLOCK), 0, s, raw, out, n, S);
+        if (qtype == 6) hipLaunchKernelGGL(k_generic<6>, dim3(g), dim3(BLOCK), 0, s, raw, out, n, S);
+    }
+    VI_LAUNCH_CHECK("kquant");
+    return VI_OK;
+}

@@ -1,0 +1,229 @@
+// Batched Goldilocks NTT and coset low-degree extension for gfx950.
+//
+// One kernel, k_ntt_pass, runs every pass of the multi-pass transform described in
+// ntt_pass.hpp: gather a tile of T columns x L points into LDS, run the radix-2
+// levels of the length-L sub-transforms there, multiply by the inter-pass
+// twiddles precomputed in HBM and scatter.  The host side (ntt_plan.hpp) decides
+// the digit split, owns the cached tables and strings passes together into
+//   * vi_ntt_batched  -- in-place natural-order transform of (m, n) rows
+//     (prover/cuda_primitives.py:388-409);
+//   * vi_coset_lde    -- values at w_K^c -> codeword on shift*<w_N>
+//     (layergkr/gpu.py:141-203), with the zero-extension fused into the first
+//     gather and the rho = N/K cosets written interleaved by the last pass, so the
+//     padded (m, N) buffer of the reference recipe is never materialised.
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#include "common.hpp"
+#include "ntt_plan.hpp"
+
+using namespace ntt;
+
+__global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
+    __shared__ u64 lds[LDS_WORDS];
+    const int tid = threadIdx.x;
+    const i64 tile = blockIdx.x;
+    u64 reg[EPT];
+    ph_load(A, tile, tid, reg);
+    const int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
+    for (int t = 0; t < n_loop; ++t) {
+        ph_stage(A, tile, tid, t, reg, lds);
+        __syncthreads();
+        for (int s = 0; s < A.a; ++s) {
+            ph_level(A, tid, s, lds);
+            __syncthreads();
+        }
+        ph_store(A, tile, tid, t, lds);
+        __syncthreads();
+    }
+}
+
+namespace {
+
+struct DeviceTables {
+    Tables T;
+    std::vector<void *> owned;
+};
+
+std::mutex g_mu;
+std::map<std::tuple<int, int, int>, DeviceTables *> g_tables;        // (device, logn, inverse)
+std::map<std::pair<int, int>, u64 *> g_twl;                          // (device, inverse)
+std::map<std::tuple<int, int, int, u64>, u64 *> g_pre;               // (device, logK, logN, shift)
+
+int upload(const std::vector<u64> &h, u64 **out) {
+    void *d = nullptr;
+    VI_HIP(hipMalloc(&d, h.size() * sizeof(u64)));
+    VI_HIP(hipMemcpy(d, h.data(), h.size() * sizeof(u64), hipMemcpyHostToDevice));
+    *out = (u64 *)d;
+    return VI_OK;
+}
+
+int get_twl(int dev, int inv, const u64 **out) {
+    auto key = std::make_pair(dev, inv);
+    auto it = g_twl.find(key);
+    if (it == g_twl.end()) {
+        u64 *d = nullptr;
+        int rc = upload(make_twl(inv), &d);
+        if (rc) return rc;
+        it = g_twl.emplace(key, d).first;
+    }
+    *out = it->second;
+    return VI_OK;
+}
+
+// tables of one (logn, direction) on the current device; built on first use
+int get_tables(int logn, int inv, const Tables **out) {
+    int dev = 0;
+    VI_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto key = std::make_tuple(dev, logn, inv);
+    auto it = g_tables.find(key);
+    if (it == g_tables.end()) {
+        HostTables H = make_tables(logn, inv);
+        DeviceTables *D = new DeviceTables();
+        D->T.sp = H.sp;
+        D->T.logn = logn;
+        D->T.scale = H.scale;
+        for (int q = 0; q < 3; ++q) {
+            D->T.tw[q] = nullptr;
+            if (!H.tw[q].empty()) {
+                u64 *d = nullptr;
+                int rc = upload(H.tw[q], &d);
+                if (rc) return rc;
+                D->T.tw[q] = d;
+                D->owned.push_back(d);
+            }
+        }
+        int rc = get_twl(dev, inv, &D->T.twl);
+        if (rc) return rc;
+        it = g_tables.emplace(key, D).first;
+    }
+    *out = &it->second->T;
+    return VI_OK;
+}
+
+int get_pre(int logK, int logN, u64 shift, const u64 **out) {
+    int dev = 0;
+    VI_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto key = std::make_tuple(dev, logK, logN, shift);
+    auto it = g_pre.find(key);
+    if (it == g_pre.end()) {
+        u64 *d = nullptr;
+        int rc = upload(make_coset_pre(logK, logN, shift), &d);
+        if (rc) return rc;
+        it = g_pre.emplace(key, d).first;
+    }
+    *out = it->second;
+    return VI_OK;
+}
+
+int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
+    for (const PassArgs &A : passes) {
+        i64 tiles = pass_tiles(A);
+        if (tiles <= 0) continue;
+        if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
+        hipLaunchKernelGGL(k_ntt_pass, dim3((unsigned)tiles), dim3(NTHREADS), 0, s, A);
+        VI_LAUNCH_CHECK("k_ntt_pass");
+    }
+    return VI_OK;
+}
+
+// rows per launch so that grids stay below 2^31 tiles
+i64 max_rows_per_launch(int logn) { return ((i64)1 << 40) >> logn; }
+
+}  // namespace
+
+extern "C" {
+
+size_t vi_ntt_workspace_bytes(int64_t m, int64_t n) {
+    if (m <= 0 || !vi::is_pow2(n) || n < 2) return 0;
+    return split_digits(vi::ilog2(n)).p > 1 ? (size_t)m * (size_t)n * sizeof(u64) : 0;
+}
+
+int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, size_t ws_bytes,
+                   void *stream) {
+    if (m < 0) return vi::fail(VI_EINVAL, "vi_ntt_batched: m = %lld", (long long)m);
+    if (!vi::is_pow2(n) || n < 2 || n > ((int64_t)1 << 32))
+        return vi::fail(VI_EINVAL, "vi_ntt_batched: row length must be a power of 2 in [2, 2^32], got %lld", (long long)n);
+    if (m == 0) return VI_OK;
+    if (!rows) return vi::fail(VI_EINVAL, "vi_ntt_batched: null rows");
+    const int logn = vi::ilog2(n);
+    const Tables *T = nullptr;
+    int rc = get_tables(logn, inverse ? 1 : 0, &T);
+    if (rc) return rc;
+    i64 chunk = m;
+    if (T->sp.p > 1) {
+        i64 fit = (i64)(ws_bytes / ((size_t)n * sizeof(u64)));
+        if (!ws || fit < 1)
+            return vi::fail(VI_ENOMEM, "vi_ntt_batched: n = %lld needs a workspace of at least %zu bytes (one row)",
+                            (long long)n, (size_t)n * sizeof(u64));
+        if (fit < chunk) chunk = fit;
+    }
+    if (chunk > max_rows_per_launch(logn)) chunk = max_rows_per_launch(logn);
+    for (i64 lo = 0; lo < m; lo += chunk) {
+        i64 cnt = (m - lo < chunk) ? (m - lo) : chunk;
+        std::vector<PassArgs> passes;
+        build_ntt_passes(*T, rows + lo * n, (u64 *)ws, cnt, passes);
+        rc = launch_passes(passes, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return VI_OK;
+}
+
+size_t vi_coset_lde_min_workspace_bytes(int64_t K, int64_t N) {
+    if (!vi::is_pow2(K) || !vi::is_pow2(N) || K < 2 || N < K) return 0;
+    return (size_t)lde_ws_elems(vi::ilog2(K), vi::ilog2(N), 1) * sizeof(u64);
+}
+
+size_t vi_coset_lde_workspace_bytes(int64_t m, int64_t K, int64_t N) {
+    size_t one = vi_coset_lde_min_workspace_bytes(K, N);
+    if (!one || m <= 0) return 0;
+    // A chunk whose scratch stays within the 256 MiB last-level cache keeps the
+    // inter-pass traffic off HBM; more rows per chunk gain nothing.
+    const size_t target = (size_t)96 << 20;
+    size_t rows = target / one;
+    if (rows < 8) rows = 8;
+    if ((int64_t)rows > m) rows = (size_t)m;
+    return rows * one;
+}
+
+int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
+                 int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, void *ws,
+                 size_t ws_bytes, void *stream) {
+    if (!vi::is_pow2(K) || !vi::is_pow2(N) || K < 2 || N < K || N > ((int64_t)1 << 32))
+        return vi::fail(VI_EINVAL, "vi_coset_lde: need powers of two with 2 <= K <= N <= 2^32, got K=%lld N=%lld",
+                        (long long)K, (long long)N);
+    if (m < 0 || width < 0 || width > K || in_stride < width || out_stride < N)
+        return vi::fail(VI_EINVAL, "vi_coset_lde: bad shape m=%lld width=%lld in_stride=%lld out_stride=%lld",
+                        (long long)m, (long long)width, (long long)in_stride, (long long)out_stride);
+    if (shift == 0 || shift >= gl::P) return vi::fail(VI_EINVAL, "vi_coset_lde: shift must be in [1, p)");
+    if (m == 0) return VI_OK;
+    if (!in || !out) return vi::fail(VI_EINVAL, "vi_coset_lde: null pointer");
+    const int logK = vi::ilog2(K), logN = vi::ilog2(N);
+    size_t one = (size_t)lde_ws_elems(logK, logN, 1) * sizeof(u64);
+    i64 chunk = (i64)(ws_bytes / one);
+    if (!ws || chunk < 1)
+        return vi::fail(VI_ENOMEM, "vi_coset_lde: workspace of %zu bytes is below the one-row minimum %zu", ws_bytes, one);
+    if (chunk > m) chunk = m;
+    if (chunk > max_rows_per_launch(logN)) chunk = max_rows_per_launch(logN);
+    const Tables *Ti = nullptr, *Tf = nullptr;
+    const u64 *pre = nullptr;
+    int rc = get_tables(logK, 1, &Ti);
+    if (!rc) rc = get_tables(logK, 0, &Tf);
+    if (!rc) rc = get_pre(logK, logN, shift, &pre);
+    if (rc) return rc;
+    for (i64 lo = 0; lo < m; lo += chunk) {
+        i64 cnt = (m - lo < chunk) ? (m - lo) : chunk;
+        std::vector<PassArgs> passes;
+        build_lde_passes(*Ti, *Tf, pre, logN, in + lo * in_stride, width, in_stride, out + lo * out_stride,
+                         out_stride, (u64 *)ws, cnt, passes);
+        rc = launch_passes(passes, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return VI_OK;
+}
+
+}  // extern "C"

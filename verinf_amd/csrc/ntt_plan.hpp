@@ -1,0 +1,184 @@
+// Host-side planning for the multi-pass NTT: digit split, twiddle tables and the
+// list of passes (ntt::PassArgs) that realise a batched in-place transform or a
+// coset low-degree extension.  Pure host C++ (no HIP calls) so that both the HIP
+// launcher and the CPU build used by the tests share it.
+#pragma once
+#include <vector>
+
+#include "ntt_pass.hpp"
+
+namespace ntt {
+
+// 7^((p-1)/2^logn): the root the reference uses (prover/ref/goldilocks_ref.py:45-49,
+// prover/kernels/ntt.cuh:310-344)
+inline u64 root_of_unity(int logn) { return gl::pow(7, (gl::P - 1) >> logn); }
+inline u64 inverse(u64 a) { return gl::pow(a, gl::P - 2); }
+
+struct Split {
+    int p;
+    int a[4];
+};
+
+// n <= 2^12 is a single in-LDS pass; above that the digits are as even as possible
+// and at most 2^MAX_A, largest first.
+inline Split split_digits(int logn) {
+    Split s{};
+    if (logn <= TILE_LOG) { s.p = 1; s.a[0] = logn; return s; }
+    s.p = (logn + MAX_A - 1) / MAX_A;
+    int base = logn / s.p, extra = logn % s.p;
+    for (int q = 0; q < s.p; ++q) s.a[q] = base + (q < extra ? 1 : 0);
+    return s;
+}
+
+// host copies of the tables of one (logn, direction)
+struct HostTables {
+    int logn, inverse;
+    Split sp;
+    std::vector<u64> tw[3];     // one per non-final pass: [(k << logR) + r] = w_M^(k r) (pass 0 also carries 1/n on the inverse)
+    u64 scale;                  // 1/n when inverse and single pass, else 1
+};
+
+inline HostTables make_tables(int logn, int inv) {
+    HostTables H;
+    H.logn = logn;
+    H.inverse = inv;
+    H.sp = split_digits(logn);
+    u64 n_inv = inverse(((u64)1 << logn) % gl::P);
+    H.scale = (inv && H.sp.p == 1) ? n_inv : 1;
+    int used = 0;
+    for (int q = 0; q + 1 < H.sp.p; ++q) {
+        int a = H.sp.a[q], logR = logn - used - a, logM = a + logR;
+        u64 w = root_of_unity(logM);
+        if (inv) w = inverse(w);
+        std::vector<u64> &t = H.tw[q];
+        t.resize((size_t)1 << logM);
+        u64 first = (inv && q == 0) ? n_inv : 1;
+        u64 wk = 1;                                   // w^k
+        for (i64 k = 0; k < ((i64)1 << a); ++k) {
+            u64 cur = first;
+            u64 *row = t.data() + (k << logR);
+            for (i64 r = 0; r < ((i64)1 << logR); ++r) { row[r] = cur; cur = gl::mul(cur, wk); }
+            wk = gl::mul(wk, w);
+        }
+        used += a;
+    }
+    return H;
+}
+
+// w_4096^j (or inverse), j < 2048
+inline std::vector<u64> make_twl(int inv) {
+    std::vector<u64> t((size_t)1 << (TWL_LOG - 1));
+    u64 w = root_of_unity(TWL_LOG);
+    if (inv) w = inverse(w);
+    u64 c = 1;
+    for (auto &x : t) { x = c; c = gl::mul(c, w); }
+    return t;
+}
+
+// pre[t][i] = (shift * w_N^t)^i, t < rho, i < K: the coefficient twist that moves the
+// evaluation domain of coset t onto shift * w_N^t * <w_K>
+// (layergkr/gpu.py:128-138 for t = 0; prover/core.py:702-718 for the rho cosets)
+inline std::vector<u64> make_coset_pre(int logK, int logN, u64 shift) {
+    int log_rho = logN - logK;
+    std::vector<u64> t((size_t)1 << (logK + log_rho));
+    u64 wN = root_of_unity(logN);
+    u64 g = shift % gl::P;
+    for (i64 c = 0; c < ((i64)1 << log_rho); ++c) {
+        u64 cur = 1;
+        u64 *row = t.data() + (c << logK);
+        for (i64 i = 0; i < ((i64)1 << logK); ++i) { row[i] = cur; cur = gl::mul(cur, g); }
+        g = gl::mul(g, wN);
+    }
+    return t;
+}
+
+// device (or host) addresses of the tables of one (logn, direction)
+struct Tables {
+    Split sp;
+    int logn;
+    const u64 *tw[3];
+    const u64 *twl;
+    u64 scale;
+};
+
+inline PassArgs base_pass(const Tables &T, int q, i64 n_rows) {
+    PassArgs A{};
+    int used = 0;
+    for (int i = 0; i < q; ++i) used += T.sp.a[i];
+    A.logn = T.logn;
+    A.a = T.sp.a[q];
+    A.is_final = (q == T.sp.p - 1);
+    A.logR = T.logn - used - A.a;
+    A.B = used;
+    A.n_rows = n_rows;
+    A.src_width = (i64)1 << T.logn;
+    A.tw = A.is_final ? nullptr : T.tw[q];
+    A.twl = T.twl;
+    A.scale = A.is_final ? T.scale : 1;
+    A.ndig = 0;
+    if (A.is_final) {
+        A.ndig = T.sp.p - 1;
+        for (int i = 0; i < A.ndig; ++i) A.dig[i] = T.sp.a[i];
+    }
+    return A;
+}
+
+// In-place batched transform of m rows (row pitch = n) held at `buf`.
+// Multi-pass sizes go buf -> ws -> ... -> buf, so ws must hold m*n elements.
+inline void build_ntt_passes(const Tables &T, u64 *buf, u64 *ws, i64 m, std::vector<PassArgs> &out) {
+    const i64 n = (i64)1 << T.logn;
+    for (int q = 0; q < T.sp.p; ++q) {
+        PassArgs A = base_pass(T, q, m);
+        A.src = (q == 0) ? buf : ws;
+        A.dst = A.is_final ? buf : ws;
+        A.src_row_stride = A.dst_row_stride = n;
+        out.push_back(A);
+    }
+}
+
+// Coset LDE of m rows:  in (m rows of `w` values, pitch in_stride)  ->  out (m, N).
+//   inverse passes:  in -> [S] -> C           (values at w_K^c -> coefficients)
+//   forward passes:  C -> [S_t, t < rho] -> out, coefficients twisted per coset by pre[t][i],
+//                    cosets interleaved out[rho*k + t]
+// Workspace: C = m*K elements, followed by S = rho*m*K elements when K needs more
+// than one pass.
+inline i64 lde_ws_elems(int logK, int logN, i64 m) {
+    i64 K = (i64)1 << logK, rho = (i64)1 << (logN - logK);
+    return split_digits(logK).p == 1 ? m * K : m * K * (1 + rho);
+}
+
+inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre, int logN,
+                             const u64 *in, i64 w, i64 in_stride, u64 *out, i64 out_stride,
+                             u64 *ws, i64 m, std::vector<PassArgs> &passes) {
+    const int logK = Ti.logn, log_rho = logN - logK, p = Ti.sp.p;
+    const i64 K = (i64)1 << logK;
+    u64 *C = ws, *S = ws + m * K;
+    // inverse: in -> S (plane 0) -> C
+    for (int q = 0; q < p; ++q) {
+        PassArgs A = base_pass(Ti, q, m);
+        A.src = (q == 0) ? in : S;
+        A.src_row_stride = (q == 0) ? in_stride : K;
+        A.src_width = (q == 0) ? w : K;
+        A.dst = A.is_final ? C : S;
+        A.dst_row_stride = K;
+        passes.push_back(A);
+    }
+    // forward over rho cosets
+    for (int q = 0; q < p; ++q) {
+        bool first = (q == 0), last = (q == p - 1);
+        PassArgs A = base_pass(Tf, q, (first || last) ? m : (m << log_rho));
+        A.log_rho = (first || last) ? log_rho : 0;     // middle passes see rho*m plain rows
+        A.loop_cosets = first && !last;
+        A.pre = first ? pre : nullptr;
+        A.src = first ? C : S;
+        A.src_row_stride = K;
+        A.src_coset_stride = first ? 0 : m * K;
+        A.dst = last ? out : S;
+        A.dst_row_stride = last ? out_stride : K;
+        A.dst_coset_stride = m * K;
+        if (last && !first) A.log_rho = log_rho;
+        passes.push_back(A);
+    }
+}
+
+}  // namespace ntt

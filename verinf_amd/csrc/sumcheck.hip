@@ -1,0 +1,309 @@
+// Multilinear sumcheck round kernels (prover side).
+//
+// The reference composes a round out of elementwise torch launches
+// (layergkr/gpu.py:341-410): per evaluation point and factor a sub, a mul and an
+// add launch, a product chain, a log-depth gl_sum, and a host sync per sample.
+// Here one launch does the whole round: every thread takes an index i of the
+// (folded) half-table, forms f(x) = f[i] + x (f[h+i] - f[i]) for x = 0..deg by
+// repeated addition, multiplies the factors of every term and accumulates the
+// deg+1 partial sums; wavefront shuffles, then LDS, then a second single-block
+// launch over the per-block partials finish the reduction, so the only host
+// round trip per round is the read-back of the deg+1 samples that the verifier
+// coin needs.
+//
+// The fold by the previous challenge is fused into the same pass: thread i reads
+// the four entries {i, i+h', h+i, h+i+h'} (h = old half, h' = h/2) of each table,
+// writes the two folded values and immediately evaluates the next round on them.
+// Per fused round a table is read once and its folded half written once.
+//
+// Variable order is most-significant first, pairs are (i, half + i)
+// (layergkr/sumcheck.py:51-54).
+#include "common.hpp"
+#include "gl_field.hpp"
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int MAX_BLOCKS = 2048;
+constexpr int MAX_DEG = 7;                  // samples per round <= 8
+constexpr int NSAMP = MAX_DEG + 1;
+constexpr int REG_TABLES = 8;               // tables a thread can keep in registers
+
+struct Desc {
+    const u64 *src[VI_SC_MAX_TABLES];
+    u64 *dst[VI_SC_MAX_TABLES];
+    u64 coeff[VI_SC_MAX_TERMS];
+    unsigned char term_off[VI_SC_MAX_TERMS + 1];
+    unsigned char fidx[VI_SC_MAX_FACTORS];
+    int n_tables, n_terms, deg;
+    int coeff_at_end;                       // single term: apply its coefficient in the final reduction
+};
+
+__device__ __forceinline__ u64 fold1(u64 lo, u64 hi, u64 r) { return gl::add(lo, gl::mul(r, gl::sub(hi, lo))); }
+
+__device__ __forceinline__ u64 wave_sum(u64 v) {
+    for (int off = 32; off > 0; off >>= 1) v = gl::add(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// MODE 0: evaluate pairs (src[i], src[half+i]), i < half
+// MODE 1: fold by r into dst (i < half), no evaluation
+// MODE 2: fold by r and evaluate the next round: i < half/2
+template <int NT, int MODE>
+__global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial) {
+    __shared__ u64 red[BLOCK / 64][NSAMP];
+    const i64 count = (MODE == 2) ? (half >> 1) : half;
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    u64 acc[NSAMP];
+#pragma unroll
+    for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
+
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < count; i += stride) {
+        u64 lo[NT], hi[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (t < D.n_tables) {
+                const u64 *f = D.src[t];
+                if (MODE == 0) {
+                    lo[t] = f[i];
+                    hi[t] = f[half + i];
+                } else if (MODE == 1) {
+                    D.dst[t][i] = fold1(f[i], f[half + i], r);
+                } else {
+                    const i64 h2 = half >> 1;
+                    u64 a0 = f[i], a1 = f[i + h2], b0 = f[half + i], b1 = f[half + i + h2];
+                    lo[t] = fold1(a0, b0, r);
+                    hi[t] = fold1(a1, b1, r);
+                    D.dst[t][i] = lo[t];
+                    D.dst[t][i + h2] = hi[t];
+                }
+            }
+        }
+        if (MODE == 1) continue;
+        // f(x) for x = 0, 1, 2, ... by repeated addition of (hi - lo)
+        u64 cur[NT], dif[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            if (t < D.n_tables) { cur[t] = lo[t]; dif[t] = gl::sub(hi[t], lo[t]); }
+        for (int x = 0; x <= D.deg; ++x) {
+            u64 sx = 0;
+            for (int k = 0; k < D.n_terms; ++k) {
+                u64 prod = D.coeff_at_end ? 1 : D.coeff[k];
+                bool first = D.coeff_at_end;
+                for (int j = D.term_off[k]; j < D.term_off[k + 1]; ++j) {
+                    int t = D.fidx[j];
+                    u64 v = 0;
+#pragma unroll
+                    for (int u = 0; u < NT; ++u)
+                        if (u == t) v = cur[u];
+                    prod = first ? v : gl::mul(prod, v);
+                    first = false;
+                }
+                sx = gl::add(sx, prod);
+            }
+#pragma unroll
+            for (int y = 0; y < NSAMP; ++y)
+                if (y == x) acc[y] = gl::add(acc[y], sx);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                if (t < D.n_tables) cur[t] = gl::add(cur[t], dif[t]);
+        }
+    }
+    if (MODE == 1) return;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int x = 0; x < NSAMP; ++x) {
+        u64 v = wave_sum(acc[x]);
+        if (lane == 0) red[w][x] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < NSAMP) {
+        u64 v = red[0][threadIdx.x];
+        for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
+        partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
+    }
+}
+
+// tables kept in memory: for problems with more than REG_TABLES distinct tables.
+// The fold (if any) has already been done by k_round<*, 1>.
+__global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 *partial) {
+    __shared__ u64 red[BLOCK / 64][NSAMP];
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    u64 acc[NSAMP];
+#pragma unroll
+    for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride) {
+        for (int k = 0; k < D.n_terms; ++k) {
+            u64 prod[NSAMP];
+#pragma unroll
+            for (int x = 0; x < NSAMP; ++x) prod[x] = D.coeff[k];
+            for (int j = D.term_off[k]; j < D.term_off[k + 1]; ++j) {
+                const u64 *f = D.src[D.fidx[j]];
+                u64 cur = f[i], dif = gl::sub(f[half + i], cur);
+#pragma unroll
+                for (int x = 0; x < NSAMP; ++x) {
+                    if (x <= D.deg) prod[x] = gl::mul(prod[x], cur);
+                    cur = gl::add(cur, dif);
+                }
+            }
+#pragma unroll
+            for (int x = 0; x < NSAMP; ++x)
+                if (x <= D.deg) acc[x] = gl::add(acc[x], prod[x]);
+        }
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int x = 0; x < NSAMP; ++x) {
+        u64 v = wave_sum(acc[x]);
+        if (lane == 0) red[w][x] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < NSAMP) {
+        u64 v = red[0][threadIdx.x];
+        for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
+        partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
+    }
+}
+
+// cross-block tree: one workgroup adds the per-block partials of every sample
+__global__ __launch_bounds__(BLOCK) void k_final(const u64 *partial, int nb, int deg, u64 scale, u64 *out) {
+    __shared__ u64 red[BLOCK / 64];
+    for (int x = 0; x <= deg; ++x) {
+        u64 acc = 0;
+        for (int b = threadIdx.x; b < nb; b += BLOCK) acc = gl::add(acc, partial[(i64)b * NSAMP + x]);
+        acc = wave_sum(acc);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            u64 v = red[0];
+            for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i]);
+            out[x] = scale == 1 ? v : gl::mul(v, scale);
+        }
+        __syncthreads();
+    }
+}
+
+int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_tables, const int *term_off,
+              const int *factor_idx, const uint64_t *coeffs, int n_terms, bool need_terms, const char *who) {
+    if (n_tables < 1 || n_tables > VI_SC_MAX_TABLES) return vi::fail(VI_EINVAL, "%s: n_tables = %d (1..%d)", who, n_tables, VI_SC_MAX_TABLES);
+    D.n_tables = n_tables;
+    for (int t = 0; t < n_tables; ++t) {
+        if (!src[t] || (dst && !dst[t])) return vi::fail(VI_EINVAL, "%s: null table %d", who, t);
+        D.src[t] = src[t];
+        D.dst[t] = dst ? dst[t] : nullptr;
+    }
+    D.n_terms = 0;
+    D.deg = 0;
+    D.coeff_at_end = 0;
+    if (!need_terms) return VI_OK;
+    if (n_terms < 1 || n_terms > VI_SC_MAX_TERMS) return vi::fail(VI_EINVAL, "%s: n_terms = %d (1..%d)", who, n_terms, VI_SC_MAX_TERMS);
+    if (!term_off || !factor_idx || !coeffs) return vi::fail(VI_EINVAL, "%s: null term descriptor", who);
+    if (term_off[0] != 0 || term_off[n_terms] > VI_SC_MAX_FACTORS) return vi::fail(VI_EINVAL, "%s: %d factors exceed %d", who, term_off[n_terms], VI_SC_MAX_FACTORS);
+    D.n_terms = n_terms;
+    for (int k = 0; k < n_terms; ++k) {
+        int nf = term_off[k + 1] - term_off[k];
+        if (nf < 1 || nf > MAX_DEG) return vi::fail(VI_EINVAL, "%s: term %d has %d factors (1..%d)", who, k, nf, MAX_DEG);
+        if (nf > D.deg) D.deg = nf;
+        D.coeff[k] = coeffs[k] % gl::P;
+        D.term_off[k] = (unsigned char)term_off[k];
+    }
+    D.term_off[n_terms] = (unsigned char)term_off[n_terms];
+    for (int j = 0; j < term_off[n_terms]; ++j) {
+        if (factor_idx[j] < 0 || factor_idx[j] >= n_tables) return vi::fail(VI_EINVAL, "%s: factor index %d out of range", who, factor_idx[j]);
+        D.fidx[j] = (unsigned char)factor_idx[j];
+    }
+    D.coeff_at_end = (n_terms == 1);
+    return VI_OK;
+}
+
+inline int blocks_for(i64 count) {
+    i64 b = (count + BLOCK - 1) / BLOCK;
+    return (int)(b < 1 ? 1 : (b > MAX_BLOCKS ? MAX_BLOCKS : b));
+}
+
+template <int MODE>
+void launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, hipStream_t s) {
+    int nt = D.n_tables;
+    if (nt <= 1) hipLaunchKernelGGL((k_round<1, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
+    else if (nt <= 2) hipLaunchKernelGGL((k_round<2, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
+    else if (nt <= 3) hipLaunchKernelGGL((k_round<3, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
+    else if (nt <= 4) hipLaunchKernelGGL((k_round<4, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
+    else hipLaunchKernelGGL((k_round<REG_TABLES, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t vi_sumcheck_workspace_bytes(void) { return (size_t)MAX_BLOCKS * NSAMP * sizeof(u64); }
+
+int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
+                     const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                     uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream) {
+    Desc D;
+    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, "vi_sumcheck_eval");
+    if (rc) return rc;
+    if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_eval: half = %lld", (long long)half);
+    if (!out_samples) return vi::fail(VI_EINVAL, "vi_sumcheck_eval: null out_samples");
+    if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
+    hipStream_t s = (hipStream_t)stream;
+    int nb = blocks_for(half);
+    if (n_tables <= REG_TABLES) launch_round<0>(D, half, 0, (u64 *)ws, nb, s);
+    else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, (u64 *)ws);
+    VI_LAUNCH_CHECK("sumcheck eval");
+    u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, out_samples);
+    VI_LAUNCH_CHECK("sumcheck final");
+    return VI_OK;
+}
+
+int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
+                          int64_t half, uint64_t r, const int *term_off, const int *factor_idx,
+                          const uint64_t *coeffs, int n_terms, uint64_t *out_samples, void *ws,
+                          size_t ws_bytes, void *stream) {
+    const bool eval = out_samples != nullptr;
+    Desc D;
+    if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
+    int rc = fill_desc(D, src, dst, n_tables, term_off, factor_idx, coeffs, n_terms, eval, "vi_sumcheck_fold_eval");
+    if (rc) return rc;
+    if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: half = %lld", (long long)half);
+    if (eval && half < 2) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: no next round after half = 1; pass out_samples = NULL");
+    if (eval && (!ws || ws_bytes < vi_sumcheck_workspace_bytes())) return vi::fail(VI_ENOMEM, "vi_sumcheck_fold_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
+    r %= gl::P;
+    hipStream_t s = (hipStream_t)stream;
+    if (!eval) {
+        for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {       // any number of tables, REG_TABLES per launch
+            Desc E = D;
+            E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
+            for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
+            launch_round<1>(E, half, r, nullptr, blocks_for(half), s);
+            VI_LAUNCH_CHECK("sumcheck fold");
+        }
+        return VI_OK;
+    }
+    int nb;
+    if (n_tables <= REG_TABLES) {
+        nb = blocks_for(half >> 1);
+        launch_round<2>(D, half, r, (u64 *)ws, nb, s);
+        VI_LAUNCH_CHECK("sumcheck fold+eval");
+    } else {
+        for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {
+            Desc E = D;
+            E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
+            for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
+            launch_round<1>(E, half, r, nullptr, blocks_for(half), s);
+            VI_LAUNCH_CHECK("sumcheck fold");
+        }
+        Desc E = D;
+        for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+        nb = blocks_for(half >> 1);
+        hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws);
+        VI_LAUNCH_CHECK("sumcheck eval");
+    }
+    u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, out_samples);
+    VI_LAUNCH_CHECK("sumcheck final");
+    return VI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,279 @@
+"""Drop-in for the field / NTT / Reed-Solomon part of the reference's
+`prover/cuda_primitives.py` on MI355X.
+
+Same public names, argument conventions and error behaviour
+(prover/cuda_primitives.py:1-41, 198-456, 1086-1183): every function works on
+contiguous `torch.uint64` tensors that live on the GPU ("cuda" is ROCm's device
+name in PyTorch), binary ops want equal shapes and return a new tensor, the NTTs
+are in place and return None, violations raise RuntimeError.  Underneath, each
+call is one ctypes hop into libverinf_hip.so on torch's current stream; nothing
+is JIT-compiled and there is no CPU fallback.
+
+Additions over the reference surface:
+  coset_lde(messages, k_deg, n_lig, shift)   the fused iNTT -> twist -> zero-extend -> NTT
+  gl_mul_bcast(a, b_row)                     a * (b_row broadcast over rows) without materialising it
+"""
+import torch
+
+from .. import _lib
+
+P = (1 << 64) - (1 << 32) + 1
+GLOBAL_G = 7
+
+_OPS = {"add": 0, "sub": 1, "mul": 2}
+
+
+def _check_u64(t, name):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be CUDA")
+    if t.dtype != torch.uint64:
+        raise RuntimeError(f"{name} dtype must be uint64")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _binop(op, a, b, who):
+    _check_u64(a, "a")
+    _check_u64(b, "b")
+    if a.shape != b.shape:
+        raise RuntimeError(f"{who}: shape mismatch")
+    out = torch.empty_like(a)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().vi_gl_binop(_OPS[op], a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                          a.numel(), _lib.stream_ptr()))
+    return out
+
+
+# ---- elementwise field (cuda_primitives.py:1086-1106) ---------------------------
+def gl_mul(a, b):
+    return _binop("mul", a, b, "gl_mul")
+
+
+def gl_add(a, b):
+    return _binop("add", a, b, "gl_add")
+
+
+def gl_sub(a, b):
+    return _binop("sub", a, b, "gl_sub")
+
+
+def gl_mul_bcast(a, b_row):
+    """a[..., i] * b_row[i]: the coset twist without `expand().contiguous()`."""
+    _check_u64(a, "a")
+    _check_u64(b_row, "b_row")
+    if b_row.dim() != 1 or a.shape[-1] != b_row.numel():
+        raise RuntimeError("gl_mul_bcast: last dimension mismatch")
+    out = torch.empty_like(a)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().vi_gl_binop_bcast(2, a.data_ptr(), b_row.data_ptr(), b_row.numel(),
+                                                out.data_ptr(), a.numel(), _lib.stream_ptr()))
+    return out
+
+
+def _unop(op, a, arg):
+    _check_u64(a, "a")
+    out = torch.empty_like(a)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().vi_gl_unop(op, a.data_ptr(), int(arg) & ((1 << 64) - 1), out.data_ptr(),
+                                         a.numel(), _lib.stream_ptr()))
+    return out
+
+
+def gl_neg(a):
+    return _unop(0, a, 0)
+
+
+def gl_pow(base, exp):
+    exp = int(exp)
+    if exp < 0 or exp >= (1 << 64):
+        raise RuntimeError("gl_pow: exponent must fit an unsigned 64-bit integer")
+    return _unop(1, base, exp)
+
+
+def gl_inv(a):
+    """Elementwise Fermat inverse a^(P-2)."""
+    return _unop(2, a, 0)
+
+
+def gl_inv_batched(a):
+    """Inverse of every element of a 1-D tensor (one Fermat power per lane, as the
+    reference does since cuda_primitives.py:289-303)."""
+    _check_u64(a, "a")
+    if a.dim() != 1:
+        raise RuntimeError("gl_inv_batched: 1-D input only")
+    return _unop(2, a, 0)
+
+
+def gl_axpy(y, alpha, x):
+    """In-place y += alpha * x mod P."""
+    _check_u64(y, "y")
+    _check_u64(x, "x")
+    if y.shape != x.shape:
+        raise RuntimeError("gl_axpy: shape mismatch")
+    with torch.cuda.device(y.device):
+        _lib.check(_lib.lib().vi_gl_axpy(y.data_ptr(), int(alpha) % P, x.data_ptr(), y.numel(),
+                                         _lib.stream_ptr()))
+
+
+# ---- NTT (cuda_primitives.py:347-409, 1111-1114) --------------------------------
+def _is_pow2(n):
+    return n > 0 and (n & (n - 1)) == 0
+
+
+def _ntt(rows, m, n, inverse):
+    L = _lib.lib()
+    with torch.cuda.device(rows.device):
+        need = L.vi_ntt_workspace_bytes(m, n)
+        ws = _lib.workspace(need, rows.device, "ntt") if need else None
+        _lib.check(L.vi_ntt_batched(rows.data_ptr(), m, n, int(inverse),
+                                    ws.data_ptr() if ws is not None else None,
+                                    ws.numel() if ws is not None else 0, _lib.stream_ptr()))
+
+
+def _ntt_1d(a, inverse):
+    _check_u64(a, "a")
+    if a.dim() != 1:
+        raise RuntimeError("NTT input must be 1-D")
+    n = a.numel()
+    if not (_is_pow2(n) and n >= 2):
+        raise RuntimeError("NTT length must be power of 2 >= 2")
+    _ntt(a, 1, n, inverse)
+
+
+def _ntt_2d(rows, inverse):
+    _check_u64(rows, "rows")
+    if rows.dim() != 2:
+        raise RuntimeError("batched NTT expects (m, n)")
+    m, n = int(rows.shape[0]), int(rows.shape[1])
+    if not (_is_pow2(n) and n >= 2):
+        raise RuntimeError("row length must be power of 2 >= 2")
+    if m:
+        _ntt(rows, m, n, inverse)
+
+
+def ntt_forward(a):
+    _ntt_1d(a, False)
+
+
+def ntt_inverse(a):
+    _ntt_1d(a, True)
+
+
+def ntt_forward_batched(rows):
+    _ntt_2d(rows, False)
+
+
+def ntt_inverse_batched(rows):
+    _ntt_2d(rows, True)
+
+
+# ---- Reed-Solomon ------------------------------------------------------------------
+def coset_lde(messages, k_deg, n_lig, shift=GLOBAL_G, out=None):
+    """(m, w <= K) values at the K-th roots of unity -> (m, N) codewords on the coset
+    shift * <w_N>, in one fused pipeline: inverse NTT_K, coefficient twist, zero
+    extension and forward transform (the recipe of layergkr/gpu.py:141-203 and
+    prover/core.py:721-743, 798).  Rows may be a strided view with unit column
+    stride, so `buf[:, :ELL]` needs no copy."""
+    if not isinstance(messages, torch.Tensor) or not messages.is_cuda:
+        raise RuntimeError("messages must be CUDA")
+    if messages.dtype != torch.uint64:
+        raise RuntimeError("messages dtype must be uint64")
+    if messages.dim() != 2:
+        raise RuntimeError("coset_lde expects (m, width)")
+    k_deg, n_lig = int(k_deg), int(n_lig)
+    m, w = int(messages.shape[0]), int(messages.shape[1])
+    if not (_is_pow2(k_deg) and k_deg >= 2):
+        raise RuntimeError("k_deg must be power of 2 >= 2")
+    if not (_is_pow2(n_lig) and n_lig >= k_deg):
+        raise RuntimeError("n_lig must be a power of 2 >= k_deg")
+    if w > k_deg:
+        raise RuntimeError("messages' second dim must be <= k_deg")
+    if m and w and messages.stride(1) != 1:
+        raise RuntimeError("messages must have unit column stride")
+    in_stride = int(messages.stride(0)) if (m > 1 and w) else max(w, 1)
+    if in_stride < w:
+        raise RuntimeError("messages rows overlap")
+    if out is None:
+        out = torch.empty((m, n_lig), dtype=torch.uint64, device=messages.device)
+    else:
+        _check_u64(out, "out")
+        if tuple(out.shape) != (m, n_lig):
+            raise RuntimeError("out must be (m, n_lig)")
+    if m == 0:
+        return out
+    if w == 0:                      # an empty message is the zero polynomial
+        return out.view(torch.int64).zero_().view(torch.uint64)
+    L = _lib.lib()
+    with torch.cuda.device(messages.device):
+        ws = _lib.workspace(L.vi_coset_lde_workspace_bytes(m, k_deg, n_lig), messages.device, "lde")
+        _lib.check(L.vi_coset_lde(messages.data_ptr(), m, w, in_stride, k_deg, n_lig, int(shift) % P,
+                                  out.data_ptr(), n_lig, ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    return out
+
+
+def rs_encode_rows(messages, n_lig, k_deg):
+    """(m, K_DEG) uint64 -> (m, N_LIG): iNTT_K, zero-extend, NTT_N with NO coset shift
+    (cuda_primitives.py:417-456) -- the legacy encoder, i.e. the LDE with shift 1."""
+    _check_u64(messages, "messages")
+    if messages.dim() != 2:
+        raise RuntimeError("rs_encode_rows expects (m, K_DEG)")
+    if int(messages.shape[1]) != int(k_deg):
+        raise RuntimeError("messages's second dim must equal k_deg")
+    return coset_lde(messages, k_deg, n_lig, shift=1)
+
+
+# ---- polynomials in coefficient form (cuda_primitives.py:1138-1183) -----------------
+def _next_pow2(n):
+    p = 2
+    while p < n:
+        p *= 2
+    return p
+
+
+def _padded(src, shape):
+    out = torch.zeros(shape, dtype=torch.uint64, device=src.device)
+    if src.dim() == 1:
+        out.view(torch.int64)[: src.numel()] = src.view(torch.int64)
+    else:
+        out.view(torch.int64)[:, : src.shape[1]] = src.view(torch.int64)
+    return out
+
+
+def poly_mul(a, b):
+    """Product of two coefficient vectors via NTT."""
+    assert a.dim() == 1 and b.dim() == 1
+    if a.numel() == 0 or b.numel() == 0:
+        return torch.empty(0, dtype=torch.uint64, device=a.device)
+    out_len = a.numel() + b.numel() - 1
+    n = _next_pow2(out_len)
+    fa, fb = _padded(a, (n,)), _padded(b, (n,))
+    ntt_forward(fa)
+    ntt_forward(fb)
+    prod = gl_mul(fa, fb)
+    ntt_inverse(prod)
+    return prod[:out_len].contiguous()
+
+
+def poly_add(a, b):
+    """Sum of two coefficient vectors of possibly different lengths."""
+    assert a.dim() == 1 and b.dim() == 1
+    n = max(a.numel(), b.numel())
+    if n == 0:
+        return torch.empty(0, dtype=torch.uint64, device=a.device)
+    return gl_add(_padded(a, (n,)), _padded(b, (n,)))
+
+
+def poly_mul_batched(A, B):
+    """Row-wise poly_mul of two (m, d) tensors -> (m, 2d - 1)."""
+    assert A.dim() == 2 and B.dim() == 2 and A.shape == B.shape
+    m, d = int(A.shape[0]), int(A.shape[1])
+    out_len = 2 * d - 1
+    n = _next_pow2(out_len)
+    fa, fb = _padded(A, (m, n)), _padded(B, (m, n))
+    ntt_forward_batched(fa)
+    ntt_forward_batched(fb)
+    prod = gl_mul(fa, fb)
+    ntt_inverse_batched(prod)
+    return prod.view(torch.int64)[:, :out_len].contiguous().view(torch.uint64)
