@@ -1,0 +1,210 @@
+"""Headline benchmark: batched Goldilocks coset LDE, 1024 rows x 2^16 -> 2^18, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" = one pass of the hot path over one batch of synthetic input: the coset
+low-degree extension of 1024 seeded rows of 2^16 field elements to 2^18 (BASELINE
+configs[1]), input and output resident in HBM.  Prints ONE JSON line with the
+metric (output elements per second), the roofline of the dominant kernel and a CPU
+baseline (the C oracle on the host cores, bounded sample, same inputs, outputs
+compared bit for bit with the GPU's).  The sumcheck (config 4) and K-quant
+(config 3) rates of the same run are reported under "extra".
+
+    python bench.py --copy-probe      plain device copy of known size (calibrates the
+                                      FETCH_SIZE / WRITE_SIZE counters, see profiles/)
+"""
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+P = (1 << 64) - (1 << 32) + 1
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
+
+
+def _events(torch):
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def rand_field(torch, shape, seed):
+    """Seeded canonical field elements on the device (uniform below 2^63 < p)."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return torch.randint(0, (1 << 63) - 1, shape, generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
+
+
+def bench_lde(torch, steps, warmup):
+    from verinf_amd import _lib
+    from verinf_amd.prover import cuda_primitives as cp
+    m, K, N = 1024, 1 << 16, 1 << 18
+    msgs = rand_field(torch, (m, K), 0)
+    out = torch.empty((m, N), dtype=torch.uint64, device="cuda")
+    for _ in range(warmup):
+        cp.coset_lde(msgs, K, N, 7, out=out)
+    torch.cuda.synchronize()
+    s, e = _events(torch)
+    s.record()
+    for _ in range(steps):
+        cp.coset_lde(msgs, K, N, 7, out=out)
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / steps
+    L = _lib.lib()
+    ws_bytes = L.vi_coset_lde_workspace_bytes(m, K, N)
+    launches = int(L.vi_coset_lde_launches(m, K, N, ws_bytes))
+    alg_bytes = 8 * (K + N) * m                       # compulsory traffic of one step
+    res = {
+        "ms_per_step": ms,
+        "elems_per_s": m * N / (ms * 1e-3),
+        "launches_per_step": launches,
+        "kernel_avg_us": ms * 1e3 / launches,
+        "alg_bytes_per_launch": alg_bytes / launches,
+        "achieved_gbs": alg_bytes / (ms * 1e-3) / 1e9,
+    }
+    return res, msgs, out
+
+
+def cpu_baseline_lde(torch, msgs, out, rows):
+    """C oracle (radix-2 iNTT -> twist -> zero-extend -> NTT per row, OpenMP over rows)
+    on the first `rows` rows of the same input; also the bit-exact check of the GPU output."""
+    import numpy as np
+    from oracle import oracle as O
+    K, N = msgs.shape[1], out.shape[1]
+    sample = msgs[:rows].cpu().numpy()
+    O.coset_lde_rows(sample[:2], K, N, 7)             # warm the library / page in
+    t0 = time.perf_counter()
+    want = O.coset_lde_rows(sample, K, N, 7)
+    dt = time.perf_counter() - t0
+    got = out[:rows].cpu().numpy()
+    return {"value": rows * N / dt, "unit": "elem/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"first {rows} of the 1024 rows, 2^16 -> 2^18, {dt:.2f} s wall",
+            "bit_exact_vs_gpu": bool(np.array_equal(got, want))}
+
+
+def bench_sumcheck(torch, v=26):
+    """Config 4: three 2^26 tables, degree 3, 26 rounds; per-round device time from
+    HIP events around each round's launches, plus the whole proof's wall time."""
+    from verinf_amd.layergkr import gpu
+    tabs = [rand_field(torch, (1 << v,), 10 + j) for j in range(3)]
+    r = random.Random(1)
+    coins = [r.randrange(P) for _ in range(v)]
+    gpu.prove_terms_gpu([(1, tabs)], lambda i: coins[i], P)            # warm-up
+    torch.cuda.synchronize()
+    stamps = []
+
+    def coin(i):
+        stamps.append(time.perf_counter())
+        return coins[i]
+
+    t0 = time.perf_counter()
+    gpu.prove_terms_gpu([(1, tabs)], coin, P)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    total = t1 - t0
+    # round 0 = first evaluation (reads 24*N bytes); round r >= 1 = fused fold+eval (36 * n_r bytes)
+    n = 1 << v
+    per_round = []
+    prev = t0
+    for i, st in enumerate(stamps):
+        byts = 24 * n if i == 0 else 36 * (n >> (i - 1))
+        per_round.append(byts / (st - prev) / 1e9)
+        prev = st
+    return {"total_ms": total * 1e3, "proof_gbs_algorithmic": 96 * n / total / 1e9,
+            "round_gbs": [round(x, 1) for x in per_round[:8]],
+            "note": "wall-clock per round incl. the sample read-back the verifier coin needs"}
+
+
+def bench_kquant(torch, steps=20):
+    from verinf_amd.prover import kquant_cuda as kq
+    nb = 4096 * 11008 // 256
+    g = torch.Generator(device="cuda").manual_seed(3)
+    raw = torch.randint(0, 256, (nb, 144), generator=g, dtype=torch.uint8, device="cuda")
+    hd = (torch.randn((nb, 2), generator=g, device="cuda") * 0.01).abs().to(torch.float16).view(torch.uint8)
+    raw[:, 0:4] = hd.reshape(nb, 4)
+    for _ in range(3):
+        kq.kquant_to_field(raw, "Q4_K", 4096)
+    torch.cuda.synchronize()
+    s, e = _events(torch)
+    s.record()
+    for _ in range(steps):
+        kq.kquant_to_field(raw, "Q4_K", 4096)
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / steps
+    return {"ms": ms, "weights_per_s": nb * 256 / (ms * 1e-3), "gbs_algorithmic": nb * 2192 / (ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": nb * 2192 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+
+def copy_probe(torch):
+    """1 GiB device-to-device copy, five times: FETCH_SIZE / WRITE_SIZE read for this
+    kernel against the known 2^30 bytes give the counters' scale factor."""
+    a = torch.zeros(1 << 27, dtype=torch.int64, device="cuda")
+    b = torch.empty_like(a)
+    for _ in range(5):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    print(json.dumps({"copy_probe_bytes_read": 1 << 30, "copy_probe_bytes_written": 1 << 30, "launches": 5}))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--cpu-rows", type=int, default=256, help="rows of the CPU baseline sample")
+    ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
+    ap.add_argument("--copy-probe", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows of the LDE are independent, "
+                 "so N GPUs would each take 1/N of the rows with no exchange)")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    if args.copy_probe:
+        copy_probe(torch)
+        return
+
+    lde, msgs, out = bench_lde(torch, args.steps, args.warmup)
+    cpu = cpu_baseline_lde(torch, msgs, out, args.cpu_rows)
+    del msgs, out
+    torch.cuda.empty_cache()
+    extra = {}
+    if not args.no_extra:
+        extra["sumcheck_3x2^26_deg3"] = bench_sumcheck(torch)
+        torch.cuda.empty_cache()
+        extra["kquant_q4k_4096x11008"] = bench_kquant(torch)
+
+    line = {
+        "metric": "goldilocks_coset_lde_2^16_to_2^18_output_elems_per_s",
+        "value": lde["elems_per_s"],
+        "unit": "elem/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": lde["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u64",
+        "data": "synthetic (seeded uniform field elements, resident in HBM)",
+        "config": {"workload": "coset LDE 1024 rows x 2^16 -> 2^18, shift 7 (BASELINE configs[1])",
+                   "rows": 1024, "K": 1 << 16, "N": 1 << 18},
+        "roofline": {"bound": "hbm", "achieved": lde["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "k_ntt_pass", "launches_per_step": lde["launches_per_step"],
+                     "avg_launch_us": lde["kernel_avg_us"],
+                     "algorithmic_bytes_per_launch": lde["alg_bytes_per_launch"]},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

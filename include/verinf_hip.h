@@ -82,6 +82,9 @@ int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, 
  * least that is accepted (one row). */
 size_t vi_coset_lde_workspace_bytes(int64_t m, int64_t K, int64_t N);
 size_t vi_coset_lde_min_workspace_bytes(int64_t K, int64_t N);
+/* Number of kernel launches one vi_coset_lde call with these arguments issues
+ * (for profilers and benchmarks); 0 on bad arguments. */
+int64_t vi_coset_lde_launches(int64_t m, int64_t K, int64_t N, size_t ws_bytes);
 int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
                  int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, void *ws,
                  size_t ws_bytes, void *stream);

@@ -25,12 +25,46 @@ Owned *make_owned(int logn, int inv) {
     o->T.sp = o->H.sp;
     o->T.logn = logn;
     for (int q = 0; q < 3; ++q) o->T.tw[q] = o->H.tw[q].empty() ? nullptr : o->H.tw[q].data();
+    for (int q = 0; q < 4; ++q) o->T.twi[q] = o->H.twi[q].empty() ? nullptr : o->H.twi[q].data();
+    o->T.inverse = inv;
     o->T.twl = o->twl.data();
     o->T.scale = o->H.scale;
     return o;
 }
 
+int g_use_fast = 1;
+
+template <int A2, bool INV>
+void run_fast(const PassArgs &A) {
+    i64 tiles = pass_tiles(A);
+    std::vector<u64> lds(fast_lds_words(A.a));
+    std::vector<u64> regs((size_t)NTHREADS * 16);
+    int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
+    for (i64 tile = 0; tile < tiles; ++tile) {
+        for (int tid = 0; tid < NTHREADS; ++tid)
+            fast_load<A2>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]));
+        for (int t = 0; t < n_loop; ++t) {
+            for (int tid = 0; tid < NTHREADS; ++tid)
+                fast_stage1<A2, INV>(A, tile, tid, t, *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
+                                     A.twi, lds.data());
+            for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV>(A, tile, tid, t, lds.data());
+        }
+    }
+}
+
 void run_pass(const PassArgs &A) {
+    if (g_use_fast && fast_ok(A.a)) {
+        switch ((A.a - FAST_A1) * 2 + (A.inverse ? 1 : 0)) {
+            case 2: run_fast<1, false>(A); return;
+            case 3: run_fast<1, true>(A); return;
+            case 4: run_fast<2, false>(A); return;
+            case 5: run_fast<2, true>(A); return;
+            case 6: run_fast<3, false>(A); return;
+            case 7: run_fast<3, true>(A); return;
+            case 8: run_fast<4, false>(A); return;
+            case 9: run_fast<4, true>(A); return;
+        }
+    }
     i64 tiles = pass_tiles(A);
     std::vector<u64> lds(LDS_WORDS);
     std::vector<u64> regs((size_t)NTHREADS * EPT);
@@ -52,6 +86,7 @@ void run_pass(const PassArgs &A) {
 
 extern "C" {
 
+void emu_set_fast(int on) { g_use_fast = on; }
 u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
 u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
 u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }

@@ -28,6 +28,7 @@ def emu():
         f.argtypes = [c_uint64, c_uint64]
     L.emu_mul_pow2.restype = c_uint64
     L.emu_mul_pow2.argtypes = [c_uint64, c_uint]
+    L.emu_set_fast.argtypes = [c_int]
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
     return L
@@ -59,16 +60,19 @@ def test_device_field_functions(emu):
             assert emu.emu_mul_pow2(a, s) == a * (1 << s) % P, (a, s)
 
 
-@pytest.mark.parametrize("logn,m", [(1, 3), (2, 5), (4, 300), (6, 7), (8, 33), (10, 5), (12, 3),
-                                    (13, 2), (14, 3), (16, 2), (18, 1)])
+@pytest.mark.parametrize("logn,m", [(1, 3), (2, 5), (4, 300), (5, 9), (6, 7), (7, 70), (8, 33), (10, 5), (12, 3),
+                                    (13, 2), (14, 3), (15, 2), (16, 2), (17, 1), (18, 1), (19, 1)])
 def test_ntt_passes_match_oracle(emu, logn, m):
     a = _rand((m, 1 << logn), 100 + logn)
     want = O.ntt_rows(a)
-    got = a.copy()
-    emu.emu_ntt_batched(_p(got), m, logn, 0)
-    assert np.array_equal(got, want)
-    emu.emu_ntt_batched(_p(got), m, logn, 1)
-    assert np.array_equal(got, a)
+    for fast in (1, 0):                      # register-blocked passes, then the generic radix-2 passes
+        emu.emu_set_fast(fast)
+        got = a.copy()
+        emu.emu_ntt_batched(_p(got), m, logn, 0)
+        assert np.array_equal(got, want), fast
+        emu.emu_ntt_batched(_p(got), m, logn, 1)
+        assert np.array_equal(got, a), fast
+    emu.emu_set_fast(1)
 
 
 def test_ntt_25_bit_split_is_well_formed(emu):
@@ -86,9 +90,12 @@ def test_ntt_25_bit_split_is_well_formed(emu):
 def test_lde_passes_match_oracle(emu, logK, logN, m, w):
     msgs = _rand((m, w), 200 + logK)
     want = O.coset_lde_rows(msgs, 1 << logK, 1 << logN, 7)
-    got = np.zeros((m, 1 << logN), dtype=np.uint64)
-    emu.emu_coset_lde(_p(msgs), m, w, w, logK, logN, 7, _p(got))
-    assert np.array_equal(got, want)
+    for fast in (1, 0):
+        emu.emu_set_fast(fast)
+        got = np.zeros((m, 1 << logN), dtype=np.uint64)
+        emu.emu_coset_lde(_p(msgs), m, w, w, logK, logN, 7, _p(got))
+        assert np.array_equal(got, want), fast
+    emu.emu_set_fast(1)
 
 
 def test_lde_strided_input_and_other_shift(emu):

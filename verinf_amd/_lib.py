@@ -19,7 +19,8 @@ EXPORTS = [
     "vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy",
     "vi_gl_sum_workspace_bytes", "vi_gl_sum",
     "vi_ntt_workspace_bytes", "vi_ntt_batched",
-    "vi_coset_lde_workspace_bytes", "vi_coset_lde_min_workspace_bytes", "vi_coset_lde",
+    "vi_coset_lde_workspace_bytes", "vi_coset_lde_min_workspace_bytes", "vi_coset_lde_launches",
+    "vi_coset_lde",
     "vi_kquant_to_field",
     "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval",
 ]
@@ -59,6 +60,8 @@ def lib():
     L.vi_coset_lde_workspace_bytes.argtypes = [i64, i64, i64]
     L.vi_coset_lde_min_workspace_bytes.restype = sz
     L.vi_coset_lde_min_workspace_bytes.argtypes = [i64, i64]
+    L.vi_coset_lde_launches.restype = i64
+    L.vi_coset_lde_launches.argtypes = [i64, i64, i64, sz]
     L.vi_coset_lde.argtypes = [vp, i64, i64, i64, i64, i64, u64, vp, i64, vp, sz, vp]
     L.vi_kquant_to_field.argtypes = [c_int, vp, i64, c_double, vp, vp]
     L.vi_sumcheck_workspace_bytes.restype = sz

@@ -20,6 +20,15 @@
 #define VI_HD inline
 #endif
 
+// Fence for the instruction scheduler (device code only): keeps it from hoisting a
+// whole phase's loads above the arithmetic of the previous one, which costs more
+// live registers than the latency it hides.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define VI_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define VI_SCHED_FENCE() ((void)0)
+#endif
+
 typedef uint64_t u64;
 typedef uint32_t u32;
 typedef int64_t i64;

@@ -40,6 +40,28 @@ __global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
     }
 }
 
+// Register-blocked pass for digits of 2^5 .. 2^8 points (ntt_fast.hpp): one LDS
+// crossing, shift-only butterflies, 16 elements per thread held in registers.
+template <int A2, bool INV>
+__global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
+    __shared__ u64 lds[TILE + (16 << A2)];
+    __shared__ u64 twi[16 << A2];
+    const int tid = threadIdx.x;
+    const i64 tile = blockIdx.x;
+    // blockIdx.y = coset of a pass that expands one source tile into rho cosets.  The
+    // rho workgroups of a tile re-read it (tiles % 8 == 0 keeps them on one XCD, so
+    // the re-reads hit that XCD's L2); a loop over cosets inside the workgroup would
+    // make every address loop-invariant and cost ~50 more live registers.
+    const int t = blockIdx.y;
+    for (int i = tid; i < (16 << A2); i += NTHREADS) twi[i] = A.twi[i];
+    __syncthreads();
+    u64 reg[16];
+    fast_load<A2>(A, tile, tid, reg);
+    fast_stage1<A2, INV>(A, tile, tid, t, reg, twi, lds);
+    __syncthreads();
+    fast_stage2<A2, INV>(A, tile, tid, t, lds);
+}
+
 namespace {
 
 struct DeviceTables {
@@ -86,6 +108,17 @@ int get_tables(int logn, int inv, const Tables **out) {
         D->T.sp = H.sp;
         D->T.logn = logn;
         D->T.scale = H.scale;
+        D->T.inverse = inv;
+        for (int q = 0; q < 4; ++q) {
+            D->T.twi[q] = nullptr;
+            if (!H.twi[q].empty()) {
+                u64 *d = nullptr;
+                int rc = upload(H.twi[q], &d);
+                if (rc) return rc;
+                D->T.twi[q] = d;
+                D->owned.push_back(d);
+            }
+        }
         for (int q = 0; q < 3; ++q) {
             D->T.tw[q] = nullptr;
             if (!H.tw[q].empty()) {
@@ -125,7 +158,22 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
         i64 tiles = pass_tiles(A);
         if (tiles <= 0) continue;
         if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
-        hipLaunchKernelGGL(k_ntt_pass, dim3((unsigned)tiles), dim3(NTHREADS), 0, s, A);
+        dim3 grid((unsigned)tiles), block(NTHREADS);
+        if (fast_ok(A.a) && A.twi) {
+            if (!A.is_final && A.loop_cosets) grid.y = 1u << A.log_rho;
+            switch ((A.a - FAST_A1) * 2 + (A.inverse ? 1 : 0)) {
+                case 2: hipLaunchKernelGGL((k_ntt_fast<1, false>), grid, block, 0, s, A); break;
+                case 3: hipLaunchKernelGGL((k_ntt_fast<1, true>), grid, block, 0, s, A); break;
+                case 4: hipLaunchKernelGGL((k_ntt_fast<2, false>), grid, block, 0, s, A); break;
+                case 5: hipLaunchKernelGGL((k_ntt_fast<2, true>), grid, block, 0, s, A); break;
+                case 6: hipLaunchKernelGGL((k_ntt_fast<3, false>), grid, block, 0, s, A); break;
+                case 7: hipLaunchKernelGGL((k_ntt_fast<3, true>), grid, block, 0, s, A); break;
+                case 8: hipLaunchKernelGGL((k_ntt_fast<4, false>), grid, block, 0, s, A); break;
+                default: hipLaunchKernelGGL((k_ntt_fast<4, true>), grid, block, 0, s, A); break;
+            }
+        } else {
+            hipLaunchKernelGGL(k_ntt_pass, grid, block, 0, s, A);
+        }
         VI_LAUNCH_CHECK("k_ntt_pass");
     }
     return VI_OK;
@@ -188,6 +236,15 @@ size_t vi_coset_lde_workspace_bytes(int64_t m, int64_t K, int64_t N) {
     if (rows < 8) rows = 8;
     if ((int64_t)rows > m) rows = (size_t)m;
     return rows * one;
+}
+
+int64_t vi_coset_lde_launches(int64_t m, int64_t K, int64_t N, size_t ws_bytes) {
+    size_t one = vi_coset_lde_min_workspace_bytes(K, N);
+    if (!one || m <= 0 || ws_bytes < one) return 0;
+    i64 chunk = (i64)(ws_bytes / one);
+    if (chunk > m) chunk = m;
+    if (chunk > max_rows_per_launch(vi::ilog2(N))) chunk = max_rows_per_launch(vi::ilog2(N));
+    return ((m + chunk - 1) / chunk) * 2 * split_digits(vi::ilog2(K)).p;
 }
 
 int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,

@@ -1,0 +1,211 @@
+// Register-blocked form of one NTT pass for digits of 2^5 .. 2^8 points.
+//
+// The length-L sub-transform (L = 16 * E2, E2 = 2, 4, 8 or 16) is itself split as
+// n = n1*E2 + n2, k = k1 + 16*k2:
+//   stage 1   A[k1][n2] = sum_{n1<16} x[n1*E2 + n2] w_16^(n1 k1), times w_L^(n2 k1)
+//   stage 2   X[k1 + 16 k2] = sum_{n2<E2} A[k1][n2] w_E2^(n2 k2)
+// Every thread runs one 16-point stage-1 transform and 16/E2 stage-2 transforms
+// entirely in registers; the tile crosses LDS exactly once in between.  Because
+// the 64th roots of unity of this field are powers of two (w_64 = 2^39), every
+// butterfly twiddle inside a register transform is +-2^s and costs a shift and a
+// fold instead of a 64x64 multiplication; full multiplications remain only for
+// the w_L^(n2 k1) layer, the inter-pass twiddles and the coset pre-multipliers.
+//
+// Global accesses: a strided pass reads/writes runs of T consecutive elements (T =
+// TILE / L columns), the final pass reads whole contiguous sub-rows and writes runs of
+// T consecutive outputs.  LDS holds [k1][n2][column] with one element of padding per
+// (k1, n2) row so both access directions are bank-conflict free.
+//
+// Written as per-thread phases (see ntt_pass.hpp) so the CPU build can run it.
+#pragma once
+#include "ntt_pass.hpp"
+
+namespace ntt {
+
+// exponent e such that w = 2^e for the twiddle w_(2^A)^(j * 2^(A-1-s)) of level s
+template <int A, bool INV>
+VI_HD constexpr int level_exp(int s, int j) {
+    int e = (39 * (64 >> A) * (j << (A - 1 - s))) % 192;
+    return INV ? (192 - e) % 192 : e;
+}
+
+template <int A>
+VI_HD constexpr int brev(int i) {
+    int r = 0;
+    for (int b = 0; b < A; ++b) r |= ((i >> b) & 1) << (A - 1 - b);
+    return r;
+}
+
+// in-register transform of 2^A points, natural order in and out, canonical values
+template <int A, bool INV>
+VI_HD void dft_reg(u64 (&x)[1 << A]) {
+    constexpr int N = 1 << A;
+    u64 y[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) y[i] = x[brev<A>(i)];
+#pragma unroll
+    for (int s = 0; s < A; ++s) {
+#pragma unroll
+        for (int b = 0; b < N / 2; ++b) {
+            const int half = 1 << s;
+            const int j = b & (half - 1), i0 = ((b >> s) << (s + 1)) + j, i1 = i0 + half;
+            const int e = level_exp<A, INV>(s, j);
+            u64 u = y[i0], v = y[i1];
+            if (e == 0) {
+                y[i0] = gl::add(u, v);
+                y[i1] = gl::sub(u, v);
+            } else if (e < 96) {
+                v = gl::mul_pow2(v, (u32)e);
+                y[i0] = gl::add(u, v);
+                y[i1] = gl::sub(u, v);
+            } else {                                   // 2^e = -2^(e-96)
+                v = gl::mul_pow2(v, (u32)(e - 96));
+                y[i0] = gl::sub(u, v);
+                y[i1] = gl::add(u, v);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] = y[i];
+}
+
+constexpr int FAST_A1 = 4;
+constexpr int FAST_E1 = 16;
+VI_HD bool fast_ok(int a) { return a >= 5 && a <= 8; }
+VI_HD int fast_lds_words(int a) { return TILE + (1 << a); }      // (L rows) x (T + 1)
+
+// per-thread description of the one column it serves in a stage
+struct ColRef {
+    bool valid;
+    i64 src_base;      // element offset of (column, point 0) in src
+    i64 idx_base;      // index inside the source row of (column, point 0)
+    i64 dst_base;      // element offset of (column, output 0) in dst
+    i64 tw_base;       // r (strided pass): twiddle index of output k is (k << logR) + r
+    int t;             // coset of the column (final pass)
+};
+
+VI_HD ColRef col_ref(const PassArgs &A, i64 tile, int c) {
+    ColRef R;
+    const i64 T = (i64)1 << logT(A);
+    const i64 g = tile * T + c;
+    R.t = 0;
+    if (!A.is_final) {
+        const int lc = A.B + A.logR;
+        const i64 row = g >> lc, col = g & (((i64)1 << lc) - 1);
+        R.valid = row < A.n_rows;
+        const i64 prefix = col >> A.logR, r = col & (((i64)1 << A.logR) - 1);
+        R.idx_base = (prefix << (A.a + A.logR)) + r;
+        R.src_base = row * A.src_row_stride + R.idx_base;
+        R.dst_base = row * A.dst_row_stride + R.idx_base;
+        R.tw_base = r;
+    } else {
+        const int lc = A.B + A.log_rho;
+        const i64 row = g >> lc, v = g & (((i64)1 << lc) - 1);
+        R.valid = row < A.n_rows;
+        R.t = (int)(v & (((i64)1 << A.log_rho) - 1));
+        R.idx_base = storage_prefix(A, v >> A.log_rho) << A.a;
+        R.src_base = (i64)R.t * A.src_coset_stride + row * A.src_row_stride + R.idx_base;
+        R.dst_base = row * A.dst_row_stride + v;
+        R.tw_base = 0;
+    }
+    return R;
+}
+
+// stage-1 thread -> (column, n2)
+template <int A2>
+VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
+    const int lt = logT(A);
+    if (!A.is_final) { c = tid & ((1 << lt) - 1); n2 = tid >> lt; }
+    else { n2 = tid & ((1 << A2) - 1); c = tid >> A2; }
+}
+
+// phase 1: this thread's 16 stage-1 inputs x[n1*E2 + n2], zero beyond src_width
+template <int A2>
+VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16]) {
+    int c, n2;
+    s1_coords<A2>(A, tid, c, n2);
+    const ColRef R = col_ref(A, tile, c);
+    const int sh = A.is_final ? 0 : A.logR;
+#pragma unroll
+    for (int n1 = 0; n1 < 16; ++n1) {
+        const i64 l = (i64)((n1 << A2) + n2) << sh;
+        reg[n1] = (R.valid && R.idx_base + l < A.src_width) ? A.src[R.src_base + l] : 0;
+    }
+}
+
+// phase 2: optional coset pre-multiplier, 16-point transform, w_L^(n2 k1), into LDS
+// twi: w_L^(n2 k1) at [n2 * 16 + k1]
+template <int A2, bool INV>
+VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, const u64 (&reg)[16],
+                       const u64 *twi, u64 *lds) {
+    int c, n2;
+    s1_coords<A2>(A, tid, c, n2);
+    u64 x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[i] = reg[i];
+    if (A.pre) {
+        const ColRef R = col_ref(A, tile, c);
+        if (R.valid) {
+            const int sh = A.is_final ? 0 : A.logR;
+            const int t = A.is_final ? R.t : t_loop;
+            const u64 *pre = A.pre + ((i64)t << A.logn) + R.idx_base;
+#pragma unroll
+            for (int g = 0; g < 16; g += 4) {
+#pragma unroll
+                for (int n1 = g; n1 < g + 4; ++n1) x[n1] = gl::mul(x[n1], pre[(i64)((n1 << A2) + n2) << sh]);
+                VI_SCHED_FENCE();
+            }
+        }
+    }
+    VI_SCHED_FENCE();
+    dft_reg<4, INV>(x);
+    VI_SCHED_FENCE();
+    const int st = (1 << logT(A)) + 1;
+#pragma unroll
+    for (int g = 0; g < 16; g += 4) {
+#pragma unroll
+        for (int k1 = g; k1 < g + 4; ++k1) {
+            u64 v = x[k1];
+            if (k1 > 0) v = gl::mul(v, twi[n2 * 16 + k1]);
+            lds[((k1 << A2) + n2) * st + c] = v;
+        }
+        VI_SCHED_FENCE();
+    }
+}
+
+// phase 3: 16/E2 stage-2 transforms, inter-pass twiddle (or final scale), scatter
+template <int A2, bool INV>
+VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u64 *lds) {
+    constexpr int E2 = 1 << A2;
+    const int lt = logT(A);
+    const int st = (1 << lt) + 1;
+    const int c = tid & ((1 << lt) - 1);
+    const ColRef R = col_ref(A, tile, c);
+    const int lc = A.B + A.log_rho;
+#pragma unroll
+    for (int i = 0; i < 16 / E2; ++i) {
+        const int k1 = (tid + i * NTHREADS) >> lt;
+        u64 x[E2];
+#pragma unroll
+        for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
+        VI_SCHED_FENCE();
+        dft_reg<A2, INV>(x);
+        VI_SCHED_FENCE();
+        if (!R.valid) continue;
+#pragma unroll
+        for (int k2 = 0; k2 < E2; ++k2) {
+            const i64 k = k1 + 16 * k2;
+            u64 v = x[k2];
+            if (!A.is_final) {
+                v = gl::mul(v, A.tw[(k << A.logR) + R.tw_base]);
+                A.dst[(i64)t_loop * A.dst_coset_stride + R.dst_base + (k << A.logR)] = v;
+            } else {
+                if (A.scale != 1) v = gl::mul(v, A.scale);
+                A.dst[R.dst_base + (k << lc)] = v;
+            }
+            if ((k2 & 3) == 3) VI_SCHED_FENCE();
+        }
+    }
+}
+
+}  // namespace ntt

@@ -53,7 +53,9 @@ struct PassArgs {
     const u64 *tw;                            // non-final: w_M^(k r) at [(k << logR) + r]
     const u64 *pre;                           // optional pre-multipliers at [(t << logn) + i]
     const u64 *twl;                           // w_4096^j (or its inverse), j < 2048
+    const u64 *twi;                           // register-blocked kernel: w_L^(n2 k1) at [n2 * 16 + k1]
     u64 scale;                                // final pass: scalar multiplier (1 = none)
+    int inverse;                              // direction of the transform
 };
 
 VI_HD int logT(const PassArgs &A) { return TILE_LOG - A.a; }
@@ -76,10 +78,11 @@ inline i64 pass_tiles(const PassArgs &A) {
 // final pass: column u in output order (k_1 lowest) -> prefix index in storage order (k_1 highest)
 VI_HD i64 storage_prefix(const PassArgs &A, i64 u) {
     i64 pre = 0;
-    for (int d = 0; d < A.ndig; ++d) {
-        pre = (pre << A.dig[d]) | (u & (((i64)1 << A.dig[d]) - 1));
-        u >>= A.dig[d];
-    }
+    // at most three earlier digits; spelled out so that the by-value argument
+    // struct is never indexed dynamically (that would force it into scratch memory)
+    if (A.ndig > 0) { pre = u & (((i64)1 << A.dig[0]) - 1); u >>= A.dig[0]; }
+    if (A.ndig > 1) { pre = (pre << A.dig[1]) | (u & (((i64)1 << A.dig[1]) - 1)); u >>= A.dig[1]; }
+    if (A.ndig > 2) { pre = (pre << A.dig[2]) | (u & (((i64)1 << A.dig[2]) - 1)); }
     return pre;
 }
 

@@ -5,7 +5,7 @@
 #pragma once
 #include <vector>
 
-#include "ntt_pass.hpp"
+#include "ntt_fast.hpp"
 
 namespace ntt {
 
@@ -35,6 +35,7 @@ struct HostTables {
     int logn, inverse;
     Split sp;
     std::vector<u64> tw[3];     // one per non-final pass: [(k << logR) + r] = w_M^(k r) (pass 0 also carries 1/n on the inverse)
+    std::vector<u64> twi[4];    // per pass with a digit of 2^5..2^8: w_L^(n2 k1) at [n2 * 16 + k1]
     u64 scale;                  // 1/n when inverse and single pass, else 1
 };
 
@@ -61,6 +62,20 @@ inline HostTables make_tables(int logn, int inv) {
             wk = gl::mul(wk, w);
         }
         used += a;
+    }
+    for (int q = 0; q < H.sp.p; ++q) {
+        int a = H.sp.a[q];
+        if (!fast_ok(a)) continue;
+        u64 w = root_of_unity(a);
+        if (inv) w = inverse(w);
+        std::vector<u64> &t = H.twi[q];
+        t.resize((size_t)1 << a);
+        u64 wn = 1;                                   // w^n2
+        for (int n2 = 0; n2 < (1 << (a - FAST_A1)); ++n2) {
+            u64 cur = 1;
+            for (int k1 = 0; k1 < FAST_E1; ++k1) { t[n2 * FAST_E1 + k1] = cur; cur = gl::mul(cur, wn); }
+            wn = gl::mul(wn, w);
+        }
     }
     return H;
 }
@@ -97,8 +112,10 @@ struct Tables {
     Split sp;
     int logn;
     const u64 *tw[3];
+    const u64 *twi[4];
     const u64 *twl;
     u64 scale;
+    int inverse;
 };
 
 inline PassArgs base_pass(const Tables &T, int q, i64 n_rows) {
@@ -114,6 +131,8 @@ inline PassArgs base_pass(const Tables &T, int q, i64 n_rows) {
     A.src_width = (i64)1 << T.logn;
     A.tw = A.is_final ? nullptr : T.tw[q];
     A.twl = T.twl;
+    A.twi = T.twi[q];
+    A.inverse = T.inverse;
     A.scale = A.is_final ? T.scale : 1;
     A.ndig = 0;
     if (A.is_final) {
