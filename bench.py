@@ -38,24 +38,31 @@ def rand_field(torch, shape, seed):
     return torch.randint(0, (1 << 63) - 1, shape, generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
 
 
-def bench_lde(torch, steps, warmup):
+def bench_lde(torch, steps, warmup, ws_mb=0):
     from verinf_amd import _lib
-    from verinf_amd.prover import cuda_primitives as cp
     m, K, N = 1024, 1 << 16, 1 << 18
     msgs = rand_field(torch, (m, K), 0)
     out = torch.empty((m, N), dtype=torch.uint64, device="cuda")
+    L = _lib.lib()
+    # the library's own default workspace (what cuda_primitives.coset_lde passes), or an override
+    ws_bytes = (ws_mb << 20) if ws_mb else L.vi_coset_lde_workspace_bytes(m, K, N)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    stream = _lib.stream_ptr()
+
+    def step():
+        _lib.check(L.vi_coset_lde(msgs.data_ptr(), m, K, K, K, N, 7, out.data_ptr(), N, ws.data_ptr(),
+                                  ws_bytes, stream))
+
     for _ in range(warmup):
-        cp.coset_lde(msgs, K, N, 7, out=out)
+        step()
     torch.cuda.synchronize()
     s, e = _events(torch)
     s.record()
     for _ in range(steps):
-        cp.coset_lde(msgs, K, N, 7, out=out)
+        step()
     e.record()
     torch.cuda.synchronize()
     ms = s.elapsed_time(e) / steps
-    L = _lib.lib()
-    ws_bytes = L.vi_coset_lde_workspace_bytes(m, K, N)
     launches = int(L.vi_coset_lde_launches(m, K, N, ws_bytes))
     alg_bytes = 8 * (K + N) * m                       # compulsory traffic of one step
     res = {
@@ -159,6 +166,9 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=256, help="rows of the CPU baseline sample")
     ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
     ap.add_argument("--copy-probe", action="store_true")
+    ap.add_argument("--ws-mb", type=int, default=0, help="override the LDE workspace size (MiB); 0 = library default")
+    ap.add_argument("--only", choices=["sumcheck", "kquant"], default=None,
+                    help="run just one of the extra legs and print its JSON (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (rows of the LDE are independent, "
@@ -169,8 +179,14 @@ def main():
     if args.copy_probe:
         copy_probe(torch)
         return
+    if args.only == "sumcheck":
+        print(json.dumps(bench_sumcheck(torch)))
+        return
+    if args.only == "kquant":
+        print(json.dumps(bench_kquant(torch)))
+        return
 
-    lde, msgs, out = bench_lde(torch, args.steps, args.warmup)
+    lde, msgs, out = bench_lde(torch, args.steps, args.warmup, args.ws_mb)
     cpu = cpu_baseline_lde(torch, msgs, out, args.cpu_rows)
     del msgs, out
     torch.cuda.empty_cache()

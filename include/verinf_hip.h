@@ -108,8 +108,9 @@ int vi_kquant_to_field(int qtype, const uint8_t *raw, int64_t n_blocks, double S
  *
  * The descriptor arrays (tables, term_off, factor_idx, coeffs) are HOST memory;
  * they are passed to the kernel by value (limits: VI_SC_MAX_TABLES, VI_SC_MAX_TERMS,
- * VI_SC_MAX_FACTORS).  out_samples: deg+1 device words.  ws: device scratch of
- * vi_sumcheck_workspace_bytes() bytes. */
+ * VI_SC_MAX_FACTORS).  out_samples: deg+1 words the GPU can write -- device memory or
+ * pinned host memory (hipHostMalloc), the latter saves the copy back.  ws: device
+ * scratch of vi_sumcheck_workspace_bytes() bytes. */
 #define VI_SC_MAX_TABLES 32
 #define VI_SC_MAX_TERMS 32
 #define VI_SC_MAX_FACTORS 64

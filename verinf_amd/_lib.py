@@ -12,7 +12,9 @@ from ctypes import POINTER, c_char_p, c_double, c_int, c_int64, c_size_t, c_uint
 import torch  # noqa: F401  (must precede the CDLL below)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libverinf_hip.so")
+# VERINF_HIP_LIB points at an alternative build of the same library (e.g. one compiled
+# with different tuning flags); the default is the in-tree build.
+LIB_PATH = os.environ.get("VERINF_HIP_LIB") or os.path.join(_HERE, "libverinf_hip.so")
 
 EXPORTS = [
     "vi_last_error", "vi_version",

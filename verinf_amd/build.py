@@ -21,9 +21,9 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Wall", "-Wno-unused-function"]
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, out: str = LIB, extra_flags=()) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-shared", "-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES]
+    cmd = [hipcc] + FLAGS + list(extra_flags) + ["-shared", "-o", out] + [os.path.join(CSRC, s) for s in SOURCES]
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -32,7 +32,7 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":

@@ -53,6 +53,21 @@ VI_HD u64 sub(u64 a, u64 b) {
 
 VI_HD u64 neg(u64 a) { return a == 0 ? 0 : P - a; }
 
+// Sum of two CANONICAL values (cheaper than add(): the wrap past 2^64 and the
+// overshoot past p take the same correction, + (2^32 - 1) mod 2^64, so one select
+// serves both).  Not for arbitrary words: with both operands >= p it can be wrong.
+VI_HD u64 addc(u64 a, u64 b) {
+    u64 s = a + b;
+    u64 r = s + EPS;
+    return ((s < a) | (r < s)) ? r : s;
+}
+
+// x mod p for an arbitrary 64-bit word
+VI_HD u64 canon(u64 x) {
+    u64 r = x + EPS;
+    return (r < x) ? r : x;
+}
+
 // (hi:lo) -> [0, p).  hi = hh*2^32 + hl  =>  value = lo - hh + hl*(2^32 - 1).
 VI_HD u64 reduce128(u64 lo, u64 hi) {
     u32 hh = (u32)(hi >> 32), hl = (u32)hi;

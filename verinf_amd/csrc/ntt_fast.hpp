@@ -36,7 +36,8 @@ VI_HD constexpr int brev(int i) {
     return r;
 }
 
-// in-register transform of 2^A points, natural order in and out, canonical values
+// in-register transform of 2^A points, natural order in and out; inputs must be
+// canonical, outputs are canonical
 template <int A, bool INV>
 VI_HD void dft_reg(u64 (&x)[1 << A]) {
     constexpr int N = 1 << A;
@@ -52,16 +53,16 @@ VI_HD void dft_reg(u64 (&x)[1 << A]) {
             const int e = level_exp<A, INV>(s, j);
             u64 u = y[i0], v = y[i1];
             if (e == 0) {
-                y[i0] = gl::add(u, v);
+                y[i0] = gl::addc(u, v);
                 y[i1] = gl::sub(u, v);
             } else if (e < 96) {
                 v = gl::mul_pow2(v, (u32)e);
-                y[i0] = gl::add(u, v);
+                y[i0] = gl::addc(u, v);
                 y[i1] = gl::sub(u, v);
             } else {                                   // 2^e = -2^(e-96)
                 v = gl::mul_pow2(v, (u32)(e - 96));
                 y[i0] = gl::sub(u, v);
-                y[i1] = gl::add(u, v);
+                y[i1] = gl::addc(u, v);
             }
         }
     }
@@ -129,7 +130,8 @@ VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16]) {
 #pragma unroll
     for (int n1 = 0; n1 < 16; ++n1) {
         const i64 l = (i64)((n1 << A2) + n2) << sh;
-        reg[n1] = (R.valid && R.idx_base + l < A.src_width) ? A.src[R.src_base + l] : 0;
+        u64 v = (R.valid && R.idx_base + l < A.src_width) ? A.src[R.src_base + l] : 0;
+        reg[n1] = A.canon_src ? gl::canon(v) : v;
     }
 }
 

@@ -28,10 +28,10 @@ namespace ntt {
 
 constexpr int TILE_LOG = 12;
 constexpr int TILE = 1 << TILE_LOG;       // elements per workgroup tile (32 KiB of LDS + padding)
-constexpr int NTHREADS = 256;
-constexpr int EPT = TILE / NTHREADS;      // elements per thread
+constexpr int EPT = 16;                   // elements per thread
+constexpr int NTHREADS = TILE / EPT;
 constexpr int MAX_A = 8;                  // largest digit of a multi-pass split
-constexpr int TWL_LOG = 12;               // master table of w_4096^j, j < 2048
+constexpr int TWL_LOG = 12;               // master table of w_4096^j, j < 2048 (TILE_LOG <= 12)
 constexpr int LDS_WORDS = TILE + (TILE >> 1);   // worst-case padded size (T = 1 needs none, T >= 2 needs L <= TILE/2 pads)
 
 struct PassArgs {
@@ -56,6 +56,7 @@ struct PassArgs {
     const u64 *twi;                           // register-blocked kernel: w_L^(n2 k1) at [n2 * 16 + k1]
     u64 scale;                                // final pass: scalar multiplier (1 = none)
     int inverse;                              // direction of the transform
+    int canon_src;                            // src is caller data: reduce every word mod p on load
 };
 
 VI_HD int logT(const PassArgs &A) { return TILE_LOG - A.a; }
@@ -170,7 +171,8 @@ VI_HD Elem scatter_elem(const PassArgs &A, i64 tile, int e, int t_loop) {
 VI_HD void ph_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[EPT]) {
     for (int i = 0; i < EPT; ++i) {
         Elem E = gather_elem(A, tile, tid + i * NTHREADS);
-        reg[i] = (E.valid && E.idx < A.src_width) ? A.src[E.addr] : 0;
+        u64 v = (E.valid && E.idx < A.src_width) ? A.src[E.addr] : 0;
+        reg[i] = A.canon_src ? gl::canon(v) : v;
     }
 }
 
@@ -199,7 +201,7 @@ VI_HD void ph_level(const PassArgs &A, int tid, int s, u64 *lds) {
         int i0 = (grp << (s + 1)) + j, i1 = i0 + half;
         u64 x = lds[(i64)i0 * st + c], y = lds[(i64)i1 * st + c];
         if (s > 0) y = gl::mul(y, A.twl[(i64)j << (TWL_LOG - 1 - s)]);
-        lds[(i64)i0 * st + c] = gl::add(x, y);
+        lds[(i64)i0 * st + c] = gl::addc(x, y);
         lds[(i64)i1 * st + c] = gl::sub(x, y);
     }
 }

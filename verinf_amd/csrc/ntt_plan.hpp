@@ -149,6 +149,7 @@ inline void build_ntt_passes(const Tables &T, u64 *buf, u64 *ws, i64 m, std::vec
     for (int q = 0; q < T.sp.p; ++q) {
         PassArgs A = base_pass(T, q, m);
         A.src = (q == 0) ? buf : ws;
+        A.canon_src = (q == 0);
         A.dst = A.is_final ? buf : ws;
         A.src_row_stride = A.dst_row_stride = n;
         out.push_back(A);
@@ -176,6 +177,7 @@ inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre,
     for (int q = 0; q < p; ++q) {
         PassArgs A = base_pass(Ti, q, m);
         A.src = (q == 0) ? in : S;
+        A.canon_src = (q == 0);
         A.src_row_stride = (q == 0) ? in_stride : K;
         A.src_width = (q == 0) ? w : K;
         A.dst = A.is_final ? C : S;

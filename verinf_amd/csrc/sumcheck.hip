@@ -49,8 +49,13 @@ __device__ __forceinline__ u64 wave_sum(u64 v) {
 // MODE 0: evaluate pairs (src[i], src[half+i]), i < half
 // MODE 1: fold by r into dst (i < half), no evaluation
 // MODE 2: fold by r and evaluate the next round: i < half/2
-template <int NT, int MODE>
-__global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial) {
+// U = indices per thread per loop trip: the evaluation-only round issues just two
+// loads per table and index, so two indices are kept in flight to cover HBM latency.
+// `direct`: a single-workgroup launch writes the finished samples itself (small rounds
+// need no second launch).
+template <int NT, int MODE, int U>
+__global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial, u64 *out,
+                                                 u64 scale, int direct) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const i64 count = (MODE == 2) ? (half >> 1) : half;
     const i64 stride = (i64)gridDim.x * BLOCK;
@@ -58,28 +63,38 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
 #pragma unroll
     for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
 
-    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < count; i += stride) {
-        u64 lo[NT], hi[NT];
+    for (i64 i0 = (i64)blockIdx.x * BLOCK + threadIdx.x; i0 < count; i0 += stride * U) {
+      u64 lo_u[U][NT], hi_u[U][NT];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const i64 i = i0 + u * stride;
+        if (i >= count) continue;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             if (t < D.n_tables) {
                 const u64 *f = D.src[t];
                 if (MODE == 0) {
-                    lo[t] = f[i];
-                    hi[t] = f[half + i];
+                    lo_u[u][t] = f[i];
+                    hi_u[u][t] = f[half + i];
                 } else if (MODE == 1) {
                     D.dst[t][i] = fold1(f[i], f[half + i], r);
                 } else {
                     const i64 h2 = half >> 1;
                     u64 a0 = f[i], a1 = f[i + h2], b0 = f[half + i], b1 = f[half + i + h2];
-                    lo[t] = fold1(a0, b0, r);
-                    hi[t] = fold1(a1, b1, r);
-                    D.dst[t][i] = lo[t];
-                    D.dst[t][i + h2] = hi[t];
+                    lo_u[u][t] = fold1(a0, b0, r);
+                    hi_u[u][t] = fold1(a1, b1, r);
+                    D.dst[t][i] = lo_u[u][t];
+                    D.dst[t][i + h2] = hi_u[u][t];
                 }
             }
         }
-        if (MODE == 1) continue;
+      }
+      if (MODE == 1) continue;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (i0 + u * stride >= count) continue;
+        u64 (&lo)[NT] = lo_u[u];
+        u64 (&hi)[NT] = hi_u[u];
         // f(x) for x = 0, 1, 2, ... by repeated addition of (hi - lo)
         u64 cur[NT], dif[NT];
 #pragma unroll
@@ -108,6 +123,7 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
             for (int t = 0; t < NT; ++t)
                 if (t < D.n_tables) cur[t] = gl::add(cur[t], dif[t]);
         }
+      }
     }
     if (MODE == 1) return;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -120,7 +136,11 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
     if (threadIdx.x < NSAMP) {
         u64 v = red[0][threadIdx.x];
         for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
-        partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
+        if (direct) {
+            if ((int)threadIdx.x <= D.deg) out[threadIdx.x] = scale == 1 ? v : gl::mul(v, scale);
+        } else {
+            partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
+        }
     }
 }
 
@@ -221,14 +241,26 @@ inline int blocks_for(i64 count) {
     return (int)(b < 1 ? 1 : (b > MAX_BLOCKS ? MAX_BLOCKS : b));
 }
 
-template <int MODE>
-void launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, hipStream_t s) {
+// rounds this small run as ONE workgroup that also finishes the reduction
+constexpr i64 DIRECT_MAX = 256;     // one loop trip per thread
+
+template <int MODE, int U>
+void launch_round_u(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
+                    hipStream_t s) {
     int nt = D.n_tables;
-    if (nt <= 1) hipLaunchKernelGGL((k_round<1, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
-    else if (nt <= 2) hipLaunchKernelGGL((k_round<2, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
-    else if (nt <= 3) hipLaunchKernelGGL((k_round<3, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
-    else if (nt <= 4) hipLaunchKernelGGL((k_round<4, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
-    else hipLaunchKernelGGL((k_round<REG_TABLES, MODE>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial);
+    if (nt <= 1) hipLaunchKernelGGL((k_round<1, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    else if (nt <= 2) hipLaunchKernelGGL((k_round<2, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    else if (nt <= 3) hipLaunchKernelGGL((k_round<3, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    else if (nt <= 4) hipLaunchKernelGGL((k_round<4, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    else hipLaunchKernelGGL((k_round<REG_TABLES, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+}
+
+template <int MODE>
+void launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
+                  hipStream_t s) {
+    // two indices in flight for the load-light evaluation round on few tables
+    if (MODE == 0 && D.n_tables <= 4 && nb > 1) launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, s);
+    else launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, s);
 }
 
 }  // namespace
@@ -248,10 +280,15 @@ int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, 
     if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
     hipStream_t s = (hipStream_t)stream;
     int nb = blocks_for(half);
-    if (n_tables <= REG_TABLES) launch_round<0>(D, half, 0, (u64 *)ws, nb, s);
+    u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
+    if (n_tables <= REG_TABLES && half <= DIRECT_MAX) {
+        launch_round<0>(D, half, 0, (u64 *)ws, 1, out_samples, scale, 1, s);
+        VI_LAUNCH_CHECK("sumcheck eval");
+        return VI_OK;
+    }
+    if (n_tables <= REG_TABLES) launch_round<0>(D, half, 0, (u64 *)ws, nb, nullptr, 1, 0, s);
     else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, (u64 *)ws);
     VI_LAUNCH_CHECK("sumcheck eval");
-    u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, out_samples);
     VI_LAUNCH_CHECK("sumcheck final");
     return VI_OK;
@@ -276,22 +313,28 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
             Desc E = D;
             E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
             for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
-            launch_round<1>(E, half, r, nullptr, blocks_for(half), s);
+            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, s);
             VI_LAUNCH_CHECK("sumcheck fold");
         }
         return VI_OK;
     }
     int nb;
+    const u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
     if (n_tables <= REG_TABLES) {
+        if ((half >> 1) <= DIRECT_MAX) {
+            launch_round<2>(D, half, r, (u64 *)ws, 1, out_samples, scale, 1, s);
+            VI_LAUNCH_CHECK("sumcheck fold+eval");
+            return VI_OK;
+        }
         nb = blocks_for(half >> 1);
-        launch_round<2>(D, half, r, (u64 *)ws, nb, s);
+        launch_round<2>(D, half, r, (u64 *)ws, nb, nullptr, 1, 0, s);
         VI_LAUNCH_CHECK("sumcheck fold+eval");
     } else {
         for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {
             Desc E = D;
             E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
             for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
-            launch_round<1>(E, half, r, nullptr, blocks_for(half), s);
+            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, s);
             VI_LAUNCH_CHECK("sumcheck fold");
         }
         Desc E = D;
@@ -300,7 +343,6 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
         hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws);
         VI_LAUNCH_CHECK("sumcheck eval");
     }
-    u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, out_samples);
     VI_LAUNCH_CHECK("sumcheck final");
     return VI_OK;

@@ -247,7 +247,6 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
 
     with torch.cuda.device(dev):
         ws = _lib.workspace(L.vi_sumcheck_workspace_bytes(), dev, "sumcheck")
-        samples_dev = torch.empty(deg + 1, dtype=torch.uint64, device=dev)
         if n_rounds == 0:
             # a single point: the claim is the term sum at that point
             total = 0
@@ -259,18 +258,35 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
                 total += prod
             return (total + mu) % field_p, [], [], mu
 
-        def read_samples():
-            return [int(v) for v in samples_dev.cpu().tolist()]
+        # The kernels write the deg+1 samples of a round straight into pinned host memory;
+        # one stream synchronisation per round is the only host round trip (the verifier
+        # coin needs the samples before the next fold can start).
+        stream = torch.cuda.current_stream()
+        sptr, ws_ptr, ws_len = stream.cuda_stream, ws.data_ptr(), ws.numel()
+        import os
+        if os.environ.get("VERINF_SC_READBACK", "pinned") == "pinned":
+            samples_host = _pinned_samples()
+            out_ptr = samples_host.data_ptr()
+
+            def read_samples():
+                stream.synchronize()
+                return samples_host[: deg + 1].tolist()
+        else:
+            samples_dev = torch.empty(deg + 1, dtype=torch.uint64, device=dev)
+            out_ptr = samples_dev.data_ptr()
+
+            def read_samples():
+                return samples_dev.cpu().tolist()
 
         half = size // 2
-        _lib.check(L.vi_sumcheck_eval(_Problem.ptrs(tables), prob.n_tables, half, prob.term_off,
-                                      prob.factor_idx, prob.coeffs, prob.n_terms, samples_dev.data_ptr(),
-                                      ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+        src_ptrs = _Problem.ptrs(tables)
+        _lib.check(L.vi_sumcheck_eval(src_ptrs, prob.n_tables, half, prob.term_off, prob.factor_idx,
+                                      prob.coeffs, prob.n_terms, out_ptr, ws_ptr, ws_len, sptr))
         ys = read_samples()
         claim = (ys[0] + ys[1] + mu) % field_p      # S(0) + S(1) is the sum over the cube
 
         round_polys, challenges = [], []
-        cur, work = tables, None
+        work = work_ptrs = None
         for rnd in range(n_rounds):
             samples = list(enumerate(ys))
             h = None
@@ -288,14 +304,24 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
             # leaves the caller's tables untouched, later ones work in place
             if work is None:
                 work = [torch.empty(half, dtype=torch.uint64, device=dev) for _ in tables]
-            _lib.check(L.vi_sumcheck_fold_eval(_Problem.ptrs(cur), _Problem.ptrs(work), prob.n_tables, half, r,
-                                               prob.term_off, prob.factor_idx, prob.coeffs, prob.n_terms,
-                                               samples_dev.data_ptr(), ws.data_ptr(), ws.numel(),
-                                               _lib.stream_ptr()))
-            cur = work
+                work_ptrs = _Problem.ptrs(work)
+            _lib.check(L.vi_sumcheck_fold_eval(src_ptrs, work_ptrs, prob.n_tables, half, r, prob.term_off,
+                                               prob.factor_idx, prob.coeffs, prob.n_terms, out_ptr, ws_ptr,
+                                               ws_len, sptr))
+            src_ptrs = work_ptrs
             half //= 2
             ys = read_samples()
     return claim, round_polys, challenges, mu
+
+
+_PINNED = {}
+
+
+def _pinned_samples():
+    """8 pinned host words the round kernels write their samples into (one per process)."""
+    if "buf" not in _PINNED:
+        _PINNED["buf"] = torch.zeros(8, dtype=torch.uint64).pin_memory()
+    return _PINNED["buf"]
 
 
 def _poly_eval(coeffs: Sequence[int], x: int, p: int) -> int:
