@@ -213,7 +213,7 @@ def main():
                    "rows": 1024, "K": 1 << 16, "N": 1 << 18},
         "roofline": {"bound": "hbm", "achieved": lde["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "k_ntt_pass", "launches_per_step": lde["launches_per_step"],
+                     "kernel": "k_ntt_fast", "launches_per_step": lde["launches_per_step"],
                      "avg_launch_us": lde["kernel_avg_us"],
                      "algorithmic_bytes_per_launch": lde["alg_bytes_per_launch"]},
         "cpu_baseline": cpu,
