@@ -147,6 +147,79 @@ def bench_kquant(torch, steps=20):
             "frac_of_hbm_peak": nb * 2192 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
+def bench_layer(torch):
+    """Config 5: one Llama-2-7B-shape layer proof core.  Commit = coset LDE of every weight
+    and activation row at the production geometry ELL = 8192, K = 2^14, N = 2^16 (a row of
+    n_in > 8192 values spans two rows); then the GKR sumchecks: one degree-2 contraction
+    per matmul (width next_pow2(n_in), layergkr/full_layer.py:216-224) and one degree-3
+    eq*a*b gate batch over S*d_ff -> 2^24 (layergkr/relations.py:104-124).  Column hashing
+    and the projection seam between the two are outside this package; random field tables
+    stand in for the projected vectors."""
+    from verinf_amd.layergkr import gpu
+    from verinf_amd.prover import cuda_primitives as cp
+    d, dff, S = 4096, 11008, 1000
+    ELL, K, N = 8192, 1 << 14, 1 << 16
+    g = torch.Generator(device="cuda").manual_seed(5)
+
+    def signed_field(shape, lo, hi):
+        v = torch.randint(lo, hi, shape, generator=g, dtype=torch.int64, device="cuda")
+        return torch.where(v >= 0, v, v - ((1 << 32) - 1)).view(torch.uint64)   # negatives as p - |x|: p + v = 2^64 + v - (2^32 - 1)
+
+    def rows_of(n_rows, n_in, lo, hi):
+        """(n_rows, n_in) values as message rows of at most ELL slots."""
+        if n_in <= ELL:
+            return [signed_field((n_rows, n_in), lo, hi)]
+        return [signed_field((n_rows, ELL), lo, hi), signed_field((n_rows, n_in - ELL), lo, hi)]
+
+    weights = {"Wq": (d, d), "Wk": (d, d), "Wv": (d, d), "Wo": (d, d), "Wgate": (dff, d), "Wup": (dff, d), "Wdown": (d, dff)}
+    acts = {"X": (S, d), "Q": (S, d), "K": (S, d), "V": (S, d), "attn": (S, d), "gate": (S, dff), "up": (S, dff),
+            "act": (S, dff), "out": (S, d)}
+    msgs = []
+    for name, (n_out, n_in) in weights.items():
+        msgs += rows_of(n_out, n_in, -128, 128)
+    for name, (n_rows, n_in) in acts.items():
+        msgs += rows_of(n_rows, n_in, -(1 << 15), 1 << 15)
+    total_rows = sum(int(m.shape[0]) for m in msgs)
+    out = torch.empty((max(int(m.shape[0]) for m in msgs), N), dtype=torch.uint64, device="cuda")
+    widths = [1 << 12] * 6 + [1 << 14]
+    mm_tabs = [[rand_field(torch, (w,), 100 + 2 * i), rand_field(torch, (w,), 101 + 2 * i)] for i, w in enumerate(widths)]
+    gate_tabs = [rand_field(torch, (1 << 24,), 200 + j) for j in range(3)]
+    r = random.Random(7)
+    coins = [r.randrange(P) for _ in range(24)]
+
+    def commit():
+        for m in msgs:
+            cp.coset_lde(m, K, N, 7, out=out[: m.shape[0]])
+
+    def sumchecks():
+        for tabs in mm_tabs:
+            gpu.prove_terms_gpu([(1, tabs)], lambda i: coins[i], P)
+        gpu.prove_terms_gpu([(1, gate_tabs)], lambda i: coins[i], P)
+
+    commit(); sumchecks()                        # warm-up (twiddle tables, workspaces)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    commit()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    sumchecks()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    t3 = time.perf_counter()
+    gpu.prove_terms_gpu([(1, gate_tabs)], lambda i: coins[i], P)
+    torch.cuda.synchronize()
+    t4 = time.perf_counter()
+    lde_bytes = 8 * (K + N) * total_rows
+    return {"rows_committed": total_rows, "geometry": "ELL=8192 K=2^14 N=2^16",
+            "end_to_end_ms": (t2 - t0) * 1e3,
+            "commit_lde_ms": (t1 - t0) * 1e3, "commit_lde_gbs_algorithmic": lde_bytes / (t1 - t0) / 1e9,
+            "commit_lde_gelems_per_s": total_rows * N / (t1 - t0) / 1e9,
+            "sumchecks_ms": (t2 - t1) * 1e3,
+            "gate_sumcheck_2^24_deg3_ms": (t4 - t3) * 1e3,
+            "gate_sumcheck_gbs_algorithmic": 96 * (1 << 24) / (t4 - t3) / 1e9,
+            "matmul_sumchecks": "6 x width 2^12 + 1 x width 2^14, degree 2 (launch-latency bound)"}
+
+
 def copy_probe(torch):
     """1 GiB device-to-device copy, five times: FETCH_SIZE / WRITE_SIZE read for this
     kernel against the known 2^30 bytes give the counters' scale factor."""
@@ -167,7 +240,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
     ap.add_argument("--copy-probe", action="store_true")
     ap.add_argument("--ws-mb", type=int, default=0, help="override the LDE workspace size (MiB); 0 = library default")
-    ap.add_argument("--only", choices=["sumcheck", "kquant"], default=None,
+    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer"], default=None,
                     help="run just one of the extra legs and print its JSON (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -185,6 +258,9 @@ def main():
     if args.only == "kquant":
         print(json.dumps(bench_kquant(torch)))
         return
+    if args.only == "layer":
+        print(json.dumps(bench_layer(torch)))
+        return
 
     lde, msgs, out = bench_lde(torch, args.steps, args.warmup, args.ws_mb)
     cpu = cpu_baseline_lde(torch, msgs, out, args.cpu_rows)
@@ -195,6 +271,8 @@ def main():
         extra["sumcheck_3x2^26_deg3"] = bench_sumcheck(torch)
         torch.cuda.empty_cache()
         extra["kquant_q4k_4096x11008"] = bench_kquant(torch)
+        torch.cuda.empty_cache()
+        extra["llama2_7b_layer"] = bench_layer(torch)
 
     line = {
         "metric": "goldilocks_coset_lde_2^16_to_2^18_output_elems_per_s",

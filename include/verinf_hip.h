@@ -124,11 +124,32 @@ int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, 
 /* fold every table by r (sumcheck.py:51-54 / gpu.py:341-347): dst[t][i] = src[t][i] +
  * r (src[t][half+i] - src[t][i]), i < half; and, when half >= 2, also return the
  * NEXT round's samples computed from the folded tables in the same pass.
- * dst[t] may equal src[t] (fold in place).  out_samples may be NULL (fold only). */
+ * dst[t] may equal src[t] (fold in place).  out_samples may be NULL (fold only).
+ * claim (host pointer, may be NULL): the value the next round's polynomial must sum to,
+ * S(0) + S(1) = S_previous(r), which the caller knows by interpolating the previous
+ * samples at r.  When given, S(1) is returned as claim - S(0) instead of being summed
+ * (same value, a quarter less work at degree 3). */
 int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
                           int64_t half, uint64_t r, const int *term_off, const int *factor_idx,
-                          const uint64_t *coeffs, int n_terms, uint64_t *out_samples, void *ws,
-                          size_t ws_bytes, void *stream);
+                          const uint64_t *coeffs, int n_terms, const uint64_t *claim,
+                          uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream);
+
+/* The whole prover loop of layergkr/gpu.py:381-409 / layergkr/sumcheck.py:191-223 on the
+ * host side of the library: evaluate, wait, hand the round's deg+1 samples to `coin`, fold
+ * by the challenge it returns while evaluating the next round, ... for log2(size) rounds.
+ * `coin(round, samples, n_samples, &r, user)` runs on the calling thread between launches
+ * and returns 0, or non-zero to abort (the call then returns VI_EINVAL).
+ *   tables        n_tables device tables of `size` = 2^v words (left untouched)
+ *   work          n_tables device buffers of size/2 words (the folded tables live here)
+ *   host_samples  >= 8 words of PINNED host memory the kernels write each round's samples to
+ *   out_samples   host, v * (deg+1) words: S_round(x) for x = 0..deg (no mask applied)
+ *   out_challenges host, v words: the challenges, reduced mod p
+ * The final fold (after the last round) is not performed, as nothing reads it. */
+typedef int (*vi_coin_fn)(int round, const uint64_t *samples, int n_samples, uint64_t *challenge, void *user);
+int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                      const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                      vi_coin_fn coin, void *user, uint64_t *host_samples, uint64_t *out_samples,
+                      uint64_t *out_challenges, void *ws, size_t ws_bytes, void *stream);
 
 #ifdef __cplusplus
 }

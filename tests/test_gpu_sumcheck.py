@@ -181,7 +181,7 @@ def test_fold_eval_in_place_c_abi(mods):
     co = (ctypes.c_uint64 * 1)(1)
     out = torch.zeros(4, dtype=torch.uint64, device="cuda")
     ws = torch.empty(L.vi_sumcheck_workspace_bytes(), dtype=torch.uint8, device="cuda")
-    _lib.check(L.vi_sumcheck_fold_eval(ptrs, ptrs, 3, 1 << 11, r, off, idx, co, 1, out.data_ptr(),
+    _lib.check(L.vi_sumcheck_fold_eval(ptrs, ptrs, 3, 1 << 11, r, off, idx, co, 1, None, out.data_ptr(),
                                        ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
     folded = [O.fold(t, r) for t in tabs]
     for t, f in zip(dev, folded):

@@ -24,8 +24,10 @@ EXPORTS = [
     "vi_coset_lde_workspace_bytes", "vi_coset_lde_min_workspace_bytes", "vi_coset_lde_launches",
     "vi_coset_lde",
     "vi_kquant_to_field",
-    "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval",
+    "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval", "vi_sumcheck_prove",
 ]
+
+COIN_FN = ctypes.CFUNCTYPE(c_int, c_int, POINTER(c_uint64), c_int, POINTER(c_uint64), c_void_p)
 
 _lib = None
 
@@ -70,7 +72,10 @@ def lib():
     L.vi_sumcheck_workspace_bytes.argtypes = []
     L.vi_sumcheck_eval.argtypes = [POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int, vp, vp, sz, vp]
     L.vi_sumcheck_fold_eval.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, u64, ip, ip,
-                                        POINTER(u64), c_int, vp, vp, sz, vp]
+                                        POINTER(u64), c_int, POINTER(u64), vp, vp, sz, vp]
+    L.vi_sumcheck_prove.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int,
+                                    COIN_FN, vp, vp, POINTER(u64), POINTER(u64), vp, sz, vp]
+    L.vi_sumcheck_prove.restype = c_int
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",

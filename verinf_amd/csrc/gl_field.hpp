@@ -80,6 +80,18 @@ VI_HD u64 reduce128(u64 lo, u64 hi) {
     return r;
 }
 
+// (hi:lo) -> some 64-bit word congruent to it (not necessarily below p): reduce128 without
+// its last conditional subtraction.  Good enough as an operand of mul / mul_wide.
+VI_HD u64 reduce128_lazy(u64 lo, u64 hi) {
+    u32 hh = (u32)(hi >> 32), hl = (u32)hi;
+    u64 t0 = lo - hh;
+    if (lo < hh) t0 -= EPS;
+    u64 t1 = ((u64)hl << 32) - hl;
+    u64 r = t0 + t1;
+    if (r < t0) r += EPS;
+    return r;
+}
+
 // 64x64 -> 128 from 32-bit halves; every line is one v_mad_u64_u32 (the addends
 // cannot overflow: (2^32-1)^2 + 2*(2^32-1) < 2^64).
 VI_HD void mul_wide(u64 a, u64 b, u64 &lo, u64 &hi) {
@@ -96,6 +108,13 @@ VI_HD u64 mul(u64 a, u64 b) {
     u64 lo, hi;
     mul_wide(a, b, lo, hi);
     return reduce128(lo, hi);
+}
+
+// product as a non-canonical word (see reduce128_lazy): for chains of multiplications
+VI_HD u64 mul_lazy(u64 a, u64 b) {
+    u64 lo, hi;
+    mul_wide(a, b, lo, hi);
+    return reduce128_lazy(lo, hi);
 }
 
 VI_HD u64 pow(u64 base, u64 e) {

@@ -37,12 +37,14 @@ struct Desc {
     unsigned char fidx[VI_SC_MAX_FACTORS];
     int n_tables, n_terms, deg;
     int coeff_at_end;                       // single term: apply its coefficient in the final reduction
+    int skip1;                              // S(1) is not summed: it is claim - S(0) (the round's known total)
+    u64 claim;                              // S(0) + S(1) when skip1
 };
 
 __device__ __forceinline__ u64 fold1(u64 lo, u64 hi, u64 r) { return gl::add(lo, gl::mul(r, gl::sub(hi, lo))); }
 
 __device__ __forceinline__ u64 wave_sum(u64 v) {
-    for (int off = 32; off > 0; off >>= 1) v = gl::add(v, __shfl_xor(v, off, 64));
+    for (int off = 32; off > 0; off >>= 1) v = gl::addc(v, __shfl_xor(v, off, 64));
     return v;
 }
 
@@ -101,27 +103,32 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         for (int t = 0; t < NT; ++t)
             if (t < D.n_tables) { cur[t] = lo[t]; dif[t] = gl::sub(hi[t], lo[t]); }
         for (int x = 0; x <= D.deg; ++x) {
-            u64 sx = 0;
-            for (int k = 0; k < D.n_terms; ++k) {
-                u64 prod = D.coeff_at_end ? 1 : D.coeff[k];
-                bool first = D.coeff_at_end;
-                for (int j = D.term_off[k]; j < D.term_off[k + 1]; ++j) {
-                    int t = D.fidx[j];
-                    u64 v = 0;
+            if (!(D.skip1 && x == 1)) {
+                u64 sx = 0;
+                for (int k = 0; k < D.n_terms; ++k) {
+                    // factors are canonical; partial products may stay non-canonical words,
+                    // only the last multiplication of a term reduces fully
+                    u64 prod = D.coeff_at_end ? 1 : D.coeff[k];
+                    bool first = D.coeff_at_end;
+                    const int j1 = D.term_off[k + 1];
+                    for (int j = D.term_off[k]; j < j1; ++j) {
+                        int t = D.fidx[j];
+                        u64 v = 0;
 #pragma unroll
-                    for (int u = 0; u < NT; ++u)
-                        if (u == t) v = cur[u];
-                    prod = first ? v : gl::mul(prod, v);
-                    first = false;
+                        for (int u = 0; u < NT; ++u)
+                            if (u == t) v = cur[u];
+                        prod = first ? v : (j + 1 < j1 ? gl::mul_lazy(prod, v) : gl::mul(prod, v));
+                        first = false;
+                    }
+                    sx = gl::addc(sx, prod);
                 }
-                sx = gl::add(sx, prod);
+#pragma unroll
+                for (int y = 0; y < NSAMP; ++y)
+                    if (y == x) acc[y] = gl::addc(acc[y], sx);
             }
 #pragma unroll
-            for (int y = 0; y < NSAMP; ++y)
-                if (y == x) acc[y] = gl::add(acc[y], sx);
-#pragma unroll
             for (int t = 0; t < NT; ++t)
-                if (t < D.n_tables) cur[t] = gl::add(cur[t], dif[t]);
+                if (t < D.n_tables) cur[t] = gl::addc(cur[t], dif[t]);
         }
       }
     }
@@ -137,7 +144,13 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         u64 v = red[0][threadIdx.x];
         for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
         if (direct) {
-            if ((int)threadIdx.x <= D.deg) out[threadIdx.x] = scale == 1 ? v : gl::mul(v, scale);
+            if (D.skip1 && threadIdx.x == 1) {           // S(1) = claim - S(0)
+                u64 s0 = red[0][0];
+                for (int i = 1; i < BLOCK / 64; ++i) s0 = gl::add(s0, red[i][0]);
+                out[1] = gl::sub(D.claim, scale == 1 ? s0 : gl::mul(s0, scale));
+            } else if ((int)threadIdx.x <= D.deg) {
+                out[threadIdx.x] = scale == 1 ? v : gl::mul(v, scale);
+            }
         } else {
             partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
         }
@@ -186,18 +199,27 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
 }
 
 // cross-block tree: one workgroup adds the per-block partials of every sample
-__global__ __launch_bounds__(BLOCK) void k_final(const u64 *partial, int nb, int deg, u64 scale, u64 *out) {
+// skip1: sample 1 was not summed; it is claim - sample 0
+__global__ __launch_bounds__(BLOCK) void k_final(const u64 *partial, int nb, int deg, u64 scale, int skip1, u64 claim,
+                                                 u64 *out) {
     __shared__ u64 red[BLOCK / 64];
+    u64 s0 = 0;
     for (int x = 0; x <= deg; ++x) {
+        if (skip1 && x == 1) {
+            if (threadIdx.x == 0) out[1] = gl::sub(claim, s0);
+            continue;
+        }
         u64 acc = 0;
-        for (int b = threadIdx.x; b < nb; b += BLOCK) acc = gl::add(acc, partial[(i64)b * NSAMP + x]);
+        for (int b = threadIdx.x; b < nb; b += BLOCK) acc = gl::addc(acc, partial[(i64)b * NSAMP + x]);
         acc = wave_sum(acc);
         if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
         __syncthreads();
         if (threadIdx.x == 0) {
             u64 v = red[0];
             for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i]);
-            out[x] = scale == 1 ? v : gl::mul(v, scale);
+            v = scale == 1 ? v : gl::mul(v, scale);
+            out[x] = v;
+            if (x == 0) s0 = v;
         }
         __syncthreads();
     }
@@ -215,6 +237,8 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
     D.n_terms = 0;
     D.deg = 0;
     D.coeff_at_end = 0;
+    D.skip1 = 0;
+    D.claim = 0;
     if (!need_terms) return VI_OK;
     if (n_terms < 1 || n_terms > VI_SC_MAX_TERMS) return vi::fail(VI_EINVAL, "%s: n_terms = %d (1..%d)", who, n_terms, VI_SC_MAX_TERMS);
     if (!term_off || !factor_idx || !coeffs) return vi::fail(VI_EINVAL, "%s: null term descriptor", who);
@@ -244,23 +268,47 @@ inline int blocks_for(i64 count) {
 // rounds this small run as ONE workgroup that also finishes the reduction
 constexpr i64 DIRECT_MAX = 256;     // one loop trip per thread
 
-template <int MODE, int U>
-void launch_round_u(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
-                    hipStream_t s) {
-    int nt = D.n_tables;
-    if (nt <= 1) hipLaunchKernelGGL((k_round<1, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
-    else if (nt <= 2) hipLaunchKernelGGL((k_round<2, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
-    else if (nt <= 3) hipLaunchKernelGGL((k_round<3, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
-    else if (nt <= 4) hipLaunchKernelGGL((k_round<4, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
-    else hipLaunchKernelGGL((k_round<REG_TABLES, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+// The round kernels are grid-stride loops: a grid larger than what is resident at once
+// would run its surplus workgroups as a second, mostly empty wave (measured: 8 waves
+// per SIMD requested, 7 resident -> almost 2x the time).  So the grid is capped at the
+// kernel's own occupancy times the CU count.
+template <typename K>
+int resident_blocks(K kernel) {
+    int per_cu = 0, dev = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, BLOCK, 0) != hipSuccess || per_cu < 1) per_cu = 4;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+        cus = 256;
+    int nb = per_cu * cus;
+    return nb > MAX_BLOCKS ? MAX_BLOCKS : nb;
 }
 
+template <int NT, int MODE, int U>
+int launch_k(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
+    static const int cap = resident_blocks(k_round<NT, MODE, U>);     // per instantiation, first use
+    if (nb > cap) nb = cap;
+    hipLaunchKernelGGL((k_round<NT, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    return nb;
+}
+
+template <int MODE, int U>
+int launch_round_u(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
+                   hipStream_t s) {
+    int nt = D.n_tables;
+    if (nt <= 1) return launch_k<1, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
+    if (nt <= 2) return launch_k<2, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
+    if (nt <= 3) return launch_k<3, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
+    if (nt <= 4) return launch_k<4, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
+    return launch_k<REG_TABLES, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
+}
+
+// returns the number of workgroups actually launched (= partials written)
 template <int MODE>
-void launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
-                  hipStream_t s) {
+int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
+                 hipStream_t s) {
     // two indices in flight for the load-light evaluation round on few tables
-    if (MODE == 0 && D.n_tables <= 4 && nb > 1) launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, s);
-    else launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, s);
+    if (MODE == 0 && D.n_tables <= 4 && nb > 1) return launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, s);
+    return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, s);
 }
 
 }  // namespace
@@ -286,18 +334,18 @@ int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, 
         VI_LAUNCH_CHECK("sumcheck eval");
         return VI_OK;
     }
-    if (n_tables <= REG_TABLES) launch_round<0>(D, half, 0, (u64 *)ws, nb, nullptr, 1, 0, s);
+    if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, (u64 *)ws, nb, nullptr, 1, 0, s);
     else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, (u64 *)ws);
     VI_LAUNCH_CHECK("sumcheck eval");
-    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, out_samples);
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, 0, (u64)0, out_samples);
     VI_LAUNCH_CHECK("sumcheck final");
     return VI_OK;
 }
 
 int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
                           int64_t half, uint64_t r, const int *term_off, const int *factor_idx,
-                          const uint64_t *coeffs, int n_terms, uint64_t *out_samples, void *ws,
-                          size_t ws_bytes, void *stream) {
+                          const uint64_t *coeffs, int n_terms, const uint64_t *claim,
+                          uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream) {
     const bool eval = out_samples != nullptr;
     Desc D;
     if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
@@ -307,6 +355,11 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
     if (eval && half < 2) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: no next round after half = 1; pass out_samples = NULL");
     if (eval && (!ws || ws_bytes < vi_sumcheck_workspace_bytes())) return vi::fail(VI_ENOMEM, "vi_sumcheck_fold_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
     r %= gl::P;
+    // the tables-in-memory path sums every sample itself
+    if (eval && claim && n_tables <= REG_TABLES) {
+        D.skip1 = 1;
+        D.claim = *claim % gl::P;
+    }
     hipStream_t s = (hipStream_t)stream;
     if (!eval) {
         for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {       // any number of tables, REG_TABLES per launch
@@ -326,8 +379,7 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
             VI_LAUNCH_CHECK("sumcheck fold+eval");
             return VI_OK;
         }
-        nb = blocks_for(half >> 1);
-        launch_round<2>(D, half, r, (u64 *)ws, nb, nullptr, 1, 0, s);
+        nb = launch_round<2>(D, half, r, (u64 *)ws, blocks_for(half >> 1), nullptr, 1, 0, s);
         VI_LAUNCH_CHECK("sumcheck fold+eval");
     } else {
         for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {
@@ -343,8 +395,60 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
         hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws);
         VI_LAUNCH_CHECK("sumcheck eval");
     }
-    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, out_samples);
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, D.skip1, D.claim, out_samples);
     VI_LAUNCH_CHECK("sumcheck final");
+    return VI_OK;
+}
+
+// value at x of the polynomial through (0, y[0]), ..., (n-1, y[n-1])
+static u64 interpolate_at(const u64 *y, int n, u64 x) {
+    u64 total = 0;
+    for (int i = 0; i < n; ++i) {
+        u64 num = y[i], den = 1;
+        for (int k = 0; k < n; ++k) {
+            if (k == i) continue;
+            num = gl::mul(num, gl::sub(x, (u64)k));
+            den = gl::mul(den, gl::sub((u64)i, (u64)k));
+        }
+        total = gl::add(total, gl::mul(num, gl::pow(den, gl::P - 2)));
+    }
+    return total;
+}
+
+int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                      const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                      vi_coin_fn coin, void *user, uint64_t *host_samples, uint64_t *out_samples,
+                      uint64_t *out_challenges, void *ws, size_t ws_bytes, void *stream) {
+    if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: size must be a power of two >= 2, got %lld", (long long)size);
+    if (!coin || !host_samples || !out_samples || !out_challenges || !work) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: null pointer");
+    Desc D;
+    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, "vi_sumcheck_prove");
+    if (rc) return rc;
+    const int ns = D.deg + 1;
+    hipStream_t s = (hipStream_t)stream;
+    int64_t half = size / 2;
+    rc = vi_sumcheck_eval(tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, host_samples, ws, ws_bytes, stream);
+    if (rc) return rc;
+    const uint64_t *const *src = tables;
+    int round = 0;
+    for (;;) {
+        VI_HIP(hipStreamSynchronize(s));
+        u64 y[NSAMP];
+        for (int x = 0; x < ns; ++x) y[x] = out_samples[(size_t)round * ns + x] = host_samples[x];
+        uint64_t r = 0;
+        int stop = coin(round, y, ns, &r, user);
+        if (stop) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: coin callback asked to stop in round %d", round);
+        r %= gl::P;
+        out_challenges[round] = r;
+        ++round;
+        if (half < 2) break;
+        const uint64_t claim = interpolate_at(y, ns, r);
+        rc = vi_sumcheck_fold_eval(src, work, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, &claim,
+                                   host_samples, ws, ws_bytes, stream);
+        if (rc) return rc;
+        src = work;
+        half /= 2;
+    }
     return VI_OK;
 }
 

@@ -180,7 +180,7 @@ def _fold_tables(src, dst, half: int, r: int):
     L = _lib.lib()
     with torch.cuda.device(src[0].device):
         _lib.check(L.vi_sumcheck_fold_eval(_Problem.ptrs(src), _Problem.ptrs(dst), len(src), half, r % P,
-                                           None, None, None, 0, None, None, 0, _lib.stream_ptr()))
+                                           None, None, None, 0, None, None, None, 0, _lib.stream_ptr()))
 
 
 def fold_t(f, r_t):
@@ -258,59 +258,45 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
                 total += prod
             return (total + mu) % field_p, [], [], mu
 
-        # The kernels write the deg+1 samples of a round straight into pinned host memory;
-        # one stream synchronisation per round is the only host round trip (the verifier
-        # coin needs the samples before the next fold can start).
-        stream = torch.cuda.current_stream()
-        sptr, ws_ptr, ws_len = stream.cuda_stream, ws.data_ptr(), ws.numel()
-        import os
-        if os.environ.get("VERINF_SC_READBACK", "pinned") == "pinned":
-            samples_host = _pinned_samples()
-            out_ptr = samples_host.data_ptr()
-
-            def read_samples():
-                stream.synchronize()
-                return samples_host[: deg + 1].tolist()
-        else:
-            samples_dev = torch.empty(deg + 1, dtype=torch.uint64, device=dev)
-            out_ptr = samples_dev.data_ptr()
-
-            def read_samples():
-                return samples_dev.cpu().tolist()
-
-        half = size // 2
-        src_ptrs = _Problem.ptrs(tables)
-        _lib.check(L.vi_sumcheck_eval(src_ptrs, prob.n_tables, half, prob.term_off, prob.factor_idx,
-                                      prob.coeffs, prob.n_terms, out_ptr, ws_ptr, ws_len, sptr))
-        ys = read_samples()
-        claim = (ys[0] + ys[1] + mu) % field_p      # S(0) + S(1) is the sum over the cube
-
+        # The round loop runs inside the library (vi_sumcheck_prove): per round one fused
+        # launch, one stream synchronisation, the samples read from pinned host memory, and
+        # this callback -- the only Python left in the loop -- which applies the optional
+        # scalar mask and asks the verifier coin for the challenge.
+        samples_host = _pinned_samples()
+        work = [torch.empty(size // 2, dtype=torch.uint64, device=dev) for _ in tables] if n_rounds > 1 else tables
         round_polys, challenges = [], []
-        work = work_ptrs = None
-        for rnd in range(n_rounds):
-            samples = list(enumerate(ys))
-            h = None
-            if mask is not None:
-                h = mask(deg, mu)
-                samples = [(x, (y + _poly_eval(h, x, field_p)) % field_p) for x, y in samples]
-            round_polys.append(samples)
-            r = coin(rnd) % field_p
-            challenges.append(r)
-            if mask is not None:
-                mu = _poly_eval(h, r, field_p)
-            if rnd == n_rounds - 1:
-                break
-            # fold by r and evaluate the next round in the same pass; the first fold
-            # leaves the caller's tables untouched, later ones work in place
-            if work is None:
-                work = [torch.empty(half, dtype=torch.uint64, device=dev) for _ in tables]
-                work_ptrs = _Problem.ptrs(work)
-            _lib.check(L.vi_sumcheck_fold_eval(src_ptrs, work_ptrs, prob.n_tables, half, r, prob.term_off,
-                                               prob.factor_idx, prob.coeffs, prob.n_terms, out_ptr, ws_ptr,
-                                               ws_len, sptr))
-            src_ptrs = work_ptrs
-            half //= 2
-            ys = read_samples()
+        state = {"mu": mu, "error": None}
+
+        def on_round(rnd, samples_p, n, r_out, _user):
+            try:
+                samples = [(x, samples_p[x]) for x in range(n)]
+                if mask is not None:
+                    h = mask(deg, state["mu"])
+                    samples = [(x, (y + _poly_eval(h, x, field_p)) % field_p) for x, y in samples]
+                round_polys.append(samples)
+                r = coin(rnd) % field_p
+                challenges.append(r)
+                if mask is not None:
+                    state["mu"] = _poly_eval(h, r, field_p)
+                r_out[0] = r
+                return 0
+            except BaseException as exc:            # never unwind through the C frames
+                state["error"] = exc
+                return 1
+
+        cb = _lib.COIN_FN(on_round)
+        out_samples = (ctypes.c_uint64 * (n_rounds * (deg + 1)))()
+        out_chals = (ctypes.c_uint64 * n_rounds)()
+        rc = L.vi_sumcheck_prove(_Problem.ptrs(tables), _Problem.ptrs(work), prob.n_tables, size, prob.term_off,
+                                 prob.factor_idx, prob.coeffs, prob.n_terms, cb, None, samples_host.data_ptr(),
+                                 out_samples, out_chals, ws.data_ptr(), ws.numel(),
+                                 torch.cuda.current_stream().cuda_stream)
+        if state["error"] is not None:
+            raise state["error"]
+        _lib.check(rc)
+        # S(0) + S(1) of the first round is the sum over the cube
+        claim = (int(out_samples[0]) + int(out_samples[1]) + mu0) % field_p
+        mu = state["mu"]
     return claim, round_polys, challenges, mu
 
 
