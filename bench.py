@@ -196,12 +196,27 @@ def bench_layer(torch):
             gpu.prove_terms_gpu([(1, tabs)], lambda i: coins[i], P)
         gpu.prove_terms_gpu([(1, gate_tabs)], lambda i: coins[i], P)
 
-    commit(); sumchecks()                        # warm-up (twiddle tables, workspaces)
+    n_w = sum(2 if n_in > ELL else 1 for (_, n_in) in weights.values())      # weight message blocks
+    chis = [rand_field(torch, (1, int(m.shape[0])), 300 + i) for i, m in enumerate(msgs[:n_w])]
+
+    def projections():
+        """chi^T W per weight block: the (1 x n_out) @ (n_out x width) seam product of
+        layergkr/projection.py:150-167; streams every committed weight message once."""
+        for chi, m in zip(chis, msgs[:n_w]):
+            cp.gl_matmul(chi, m)
+
+    commit(); projections(); sumchecks()         # warm-up (twiddle tables, workspaces)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     commit()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    projections()
+    torch.cuda.synchronize()
+    tp = time.perf_counter()
+    proj_ms = (tp - t1) * 1e3
+    proj_bytes = sum(int(m.numel()) * 8 for m in msgs[:n_w])
+    t1b = time.perf_counter()
     sumchecks()
     torch.cuda.synchronize()
     t2 = time.perf_counter()
@@ -212,9 +227,10 @@ def bench_layer(torch):
     lde_bytes = 8 * (K + N) * total_rows
     return {"rows_committed": total_rows, "geometry": "ELL=8192 K=2^14 N=2^16",
             "end_to_end_ms": (t2 - t0) * 1e3,
+            "projection_matvec_ms": proj_ms, "projection_matvec_gbs": proj_bytes / proj_ms / 1e6,
             "commit_lde_ms": (t1 - t0) * 1e3, "commit_lde_gbs_algorithmic": lde_bytes / (t1 - t0) / 1e9,
             "commit_lde_gelems_per_s": total_rows * N / (t1 - t0) / 1e9,
-            "sumchecks_ms": (t2 - t1) * 1e3,
+            "sumchecks_ms": (t2 - t1b) * 1e3,
             "gate_sumcheck_2^24_deg3_ms": (t4 - t3) * 1e3,
             "gate_sumcheck_gbs_algorithmic": 96 * (1 << 24) / (t4 - t3) / 1e9,
             "matmul_sumchecks": "6 x width 2^12 + 1 x width 2^14, degree 2 (launch-latency bound)"}

@@ -59,6 +59,21 @@ int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *
 size_t vi_gl_sum_workspace_bytes(int64_t n);
 int vi_gl_sum(const uint64_t *a, int64_t n, uint64_t *out, void *ws, size_t ws_bytes, void *stream);
 
+/* ---- dense products and Horner evaluation ------------------------------------------
+ * Replace gl_matmul / gl_matvec (prover/cuda_primitives.py:485-510,
+ * prover/kernels/gl_matmul.cuh:29-59) and poly_eval (cuda_primitives.py:462-479,
+ * prover/kernels/gl_extras.cuh:93-108).  All matrices row-major and dense.
+ *   vi_gl_matmul   C (m x n) = A (m x k) B (k x n); at most 65535 rows of A; the shape it is
+ *                  tuned for is a few rows of A against a tall B (projection seam, combine).
+ *   vi_gl_matvec   w (m) = M (m x n) v (n)
+ *   vi_poly_eval   out[r][p] = sum_i coeffs[r][i] points[p]^i, coeffs (m x d), out (m x k) */
+size_t vi_gl_matmul_workspace_bytes(int64_t m, int64_t k, int64_t n);
+int vi_gl_matmul(const uint64_t *A, const uint64_t *B, uint64_t *C, int64_t m, int64_t k, int64_t n,
+                 void *ws, size_t ws_bytes, void *stream);
+int vi_gl_matvec(const uint64_t *M, const uint64_t *v, uint64_t *w, int64_t m, int64_t n, void *stream);
+int vi_poly_eval(const uint64_t *coeffs, int64_t m, int64_t d, const uint64_t *points, int64_t k,
+                 uint64_t *out, void *stream);
+
 /* ---- NTT ---------------------------------------------------------------------
  * Replaces ntt_forward / ntt_inverse / ntt_forward_batched / ntt_inverse_batched
  * (prover/cuda_primitives.py:347-409, 1111-1114; prover/kernels/ntt.cuh:667-770):

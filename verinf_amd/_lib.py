@@ -20,6 +20,7 @@ EXPORTS = [
     "vi_last_error", "vi_version",
     "vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy",
     "vi_gl_sum_workspace_bytes", "vi_gl_sum",
+    "vi_gl_matmul_workspace_bytes", "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
     "vi_ntt_workspace_bytes", "vi_ntt_batched",
     "vi_coset_lde_workspace_bytes", "vi_coset_lde_min_workspace_bytes", "vi_coset_lde_launches",
     "vi_coset_lde",
@@ -57,6 +58,11 @@ def lib():
     L.vi_gl_sum_workspace_bytes.restype = sz
     L.vi_gl_sum_workspace_bytes.argtypes = [i64]
     L.vi_gl_sum.argtypes = [vp, i64, vp, vp, sz, vp]
+    L.vi_gl_matmul_workspace_bytes.restype = sz
+    L.vi_gl_matmul_workspace_bytes.argtypes = [i64, i64, i64]
+    L.vi_gl_matmul.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, vp]
+    L.vi_gl_matvec.argtypes = [vp, vp, vp, i64, i64, vp]
+    L.vi_poly_eval.argtypes = [vp, i64, i64, vp, i64, vp, vp]
     L.vi_ntt_workspace_bytes.restype = sz
     L.vi_ntt_workspace_bytes.argtypes = [i64, i64]
     L.vi_ntt_batched.argtypes = [vp, i64, i64, c_int, vp, sz, vp]
@@ -79,6 +85,7 @@ def lib():
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
+                 "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
                  "vi_ntt_batched", "vi_coset_lde", "vi_kquant_to_field", "vi_sumcheck_eval",
                  "vi_sumcheck_fold_eval"):
         getattr(L, name).restype = c_int

@@ -14,8 +14,9 @@ one fused kernel plus a single-block reduction instead of ~(deg+1)*(4*factors +
 log n) elementwise launches; the only host synchronisation per round is the
 read-back of the deg+1 samples that the verifier coin needs.
 
-The dense `gl_matmul` encoders, `combine_t` and the BLAKE3 `hash_and_tree` of the
-reference module are outside this package.
+`linear_combination` and `combine_t` (gpu.py:113-122, 301-308) run on `gl_matmul`.
+The dense Lagrange-matrix encoders (`encode_batch[_t]`) and the BLAKE3 `hash_and_tree` of
+the reference module are outside this package (the NTT encoder is the one encoder here).
 """
 import ctypes
 from typing import Optional, Sequence
@@ -132,6 +133,29 @@ def selftest_ntt_spot(cfg: Config, n_cols: int = 24, seed: int = 5) -> Optional[
         if ref != int(got[j]):
             return f"column {j}: dense {ref} != ntt {int(got[j])}"
     return None
+
+
+def _u64_row(values):
+    import numpy as np
+    return torch.from_numpy(np.array([[int(v) % P for v in values]], dtype=np.uint64)).cuda()
+
+
+def linear_combination(cfg: Config, codewords, coeffs: Sequence[int]):
+    """sum_i coeffs[i] * codewords[i] as a (1 x rows) @ (rows x N) product; Python rows in,
+    Python list out (gpu.py:113-122)."""
+    _require_gpu()
+    import numpy as np
+    if len(codewords) != len(coeffs):
+        raise ValueError("coeffs/codewords length mismatch")
+    B = torch.from_numpy(np.array([[int(v) % P for v in c] for c in codewords], dtype=np.uint64)).cuda()
+    return [int(v) for v in cp.gl_matmul(_u64_row(coeffs), B)[0].cpu().tolist()]
+
+
+def combine_t(cfg: Config, mat, coeffs: Sequence[int]):
+    """sum_i coeffs[i] * mat[i] for a device matrix, staying on the device: (1, N) tensor
+    (gpu.py:301-308)."""
+    _require_gpu()
+    return cp.gl_matmul(_u64_row(coeffs), mat)
 
 
 def column(mat, col: int):

@@ -76,6 +76,11 @@ class Commit:
         from . import gpu
         return gpu.column(self.mat, col)
 
+    def combine(self, coeffs: Sequence[int]):
+        """sum_i coeffs[i] * row_i as a (1, N) device tensor (rs.py:254-259)."""
+        from . import gpu
+        return gpu.combine_t(self.cfg, self.mat, coeffs)
+
     @property
     def root(self) -> bytes:
         raise NotImplementedError("column hashing / Merkle tree are outside verinf_amd")

@@ -224,7 +224,68 @@ def rs_encode_rows(messages, n_lig, k_deg):
     return coset_lde(messages, k_deg, n_lig, shift=1)
 
 
+# ---- linear algebra mod P (cuda_primitives.py:485-510, 1188-1189) --------------------
+def gl_matmul(A, B):
+    """(m, k) @ (k, n) over the field."""
+    _check_u64(A, "A")
+    _check_u64(B, "B")
+    if A.dim() != 2 or B.dim() != 2:
+        raise RuntimeError("gl_matmul: 2-D inputs")
+    m, k, kb, n = int(A.shape[0]), int(A.shape[1]), int(B.shape[0]), int(B.shape[1])
+    if k != kb:
+        raise RuntimeError("gl_matmul: inner dim mismatch")
+    C = torch.empty((m, n), dtype=torch.uint64, device=A.device)
+    L = _lib.lib()
+    with torch.cuda.device(A.device):
+        for lo in range(0, m, 65535):
+            hi = min(lo + 65535, m)
+            need = L.vi_gl_matmul_workspace_bytes(hi - lo, k, n)
+            ws = _lib.workspace(need, A.device, "matmul") if need else None
+            _lib.check(L.vi_gl_matmul(A[lo:hi].data_ptr() if m else None, B.data_ptr(), C[lo:hi].data_ptr() if m else None,
+                                      hi - lo, k, n, ws.data_ptr() if ws is not None else None,
+                                      ws.numel() if ws is not None else 0, _lib.stream_ptr()))
+    return C
+
+
+def gl_matvec(M, v):
+    """(m, n) @ (n,) over the field."""
+    _check_u64(M, "M")
+    _check_u64(v, "v")
+    if M.dim() != 2 or v.dim() != 1:
+        raise RuntimeError("gl_matvec: (m,n) @ (n,)")
+    m, n = int(M.shape[0]), int(M.shape[1])
+    if int(v.shape[0]) != n:
+        raise RuntimeError("gl_matvec: dim mismatch")
+    out = torch.empty((m,), dtype=torch.uint64, device=M.device)
+    with torch.cuda.device(M.device):
+        _lib.check(_lib.lib().vi_gl_matvec(M.data_ptr(), v.data_ptr(), out.data_ptr(), m, n, _lib.stream_ptr()))
+    return out
+
+
 # ---- polynomials in coefficient form (cuda_primitives.py:1138-1183) -----------------
+def poly_eval(coeffs, points):
+    """Horner evaluation; coeffs (d,) -> (k,) or (m, d) -> (m, k)."""
+    _check_u64(coeffs, "coeffs")
+    _check_u64(points, "points")
+    if points.dim() != 1:
+        raise RuntimeError("points must be 1-D")
+    if coeffs.dim() not in (1, 2):
+        raise RuntimeError("coeffs must be 1-D or 2-D")
+    one_d = coeffs.dim() == 1
+    m = 1 if one_d else int(coeffs.shape[0])
+    d = int(coeffs.shape[-1])
+    k = int(points.shape[0])
+    out = torch.empty((m, k), dtype=torch.uint64, device=coeffs.device)
+    L = _lib.lib()
+    with torch.cuda.device(coeffs.device):
+        for lo in range(0, m, 65535):
+            hi = min(lo + 65535, m)
+            src = coeffs if one_d else coeffs[lo:hi]
+            _lib.check(L.vi_poly_eval(src.data_ptr(), hi - lo, d, points.data_ptr(), k, out[lo:hi].data_ptr(),
+                                      _lib.stream_ptr()))
+    return out.reshape(k) if one_d else out
+
+
 def _next_pow2(n):
     p = 2
     while p < n:
