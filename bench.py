@@ -93,7 +93,7 @@ def cpu_baseline_lde(torch, msgs, out, rows):
             "bit_exact_vs_gpu": bool(np.array_equal(got, want))}
 
 
-def bench_sumcheck(torch, v=26):
+def bench_sumcheck(torch, v=26, cpu=True):
     """Config 4: three 2^26 tables, degree 3, 26 rounds; per-round device time from
     HIP events around each round's launches, plus the whole proof's wall time."""
     from verinf_amd.layergkr import gpu
@@ -121,12 +121,25 @@ def bench_sumcheck(torch, v=26):
         byts = 24 * n if i == 0 else 36 * (n >> (i - 1))
         per_round.append(byts / (st - prev) / 1e9)
         prev = st
-    return {"total_ms": total * 1e3, "proof_gbs_algorithmic": 96 * n / total / 1e9,
-            "round_gbs": [round(x, 1) for x in per_round[:8]],
-            "note": "wall-clock per round incl. the sample read-back the verifier coin needs"}
+    res = {"total_ms": total * 1e3, "proof_gbs_algorithmic": 96 * n / total / 1e9,
+           "round_gbs": [round(x, 1) for x in per_round[:8]],
+           "note": "wall-clock per round incl. the sample read-back the verifier coin needs"}
+    if cpu:
+        # C oracle (sumcheck.prove_terms loop, OpenMP) on a bounded instance: 3 x 2^22, 22 rounds
+        from oracle import oracle as O
+        vb = 22
+        small = [t[: 1 << vb].cpu().numpy() for t in tabs]
+        claim, polys, _, _ = gpu.prove_terms_gpu([(1, [t[: 1 << vb].contiguous() for t in tabs])], lambda i: coins[i], P)
+        c0 = time.perf_counter()
+        want_claim, want_samples, _ = O.sumcheck_prove(small, [(1, [0, 1, 2])], coins)
+        dt = time.perf_counter() - c0
+        res["cpu_baseline"] = {"value": 96 * (1 << vb) / dt / 1e9, "unit": "GB/s algorithmic", "cores": O.num_threads(),
+                               "kind": "port", "sample": f"3 x 2^{vb} tables, {vb} rounds, {dt:.2f} s wall",
+                               "bit_exact_vs_gpu": bool(claim == want_claim and [[y for _, y in s] for s in polys] == want_samples)}
+    return res
 
 
-def bench_kquant(torch, steps=20):
+def bench_kquant(torch, steps=20, cpu=True):
     from verinf_amd.prover import kquant_cuda as kq
     nb = 4096 * 11008 // 256
     g = torch.Generator(device="cuda").manual_seed(3)
@@ -143,8 +156,22 @@ def bench_kquant(torch, steps=20):
     e.record()
     torch.cuda.synchronize()
     ms = s.elapsed_time(e) / steps
-    return {"ms": ms, "weights_per_s": nb * 256 / (ms * 1e-3), "gbs_algorithmic": nb * 2192 / (ms * 1e-3) / 1e9,
-            "frac_of_hbm_peak": nb * 2192 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    res = {"ms": ms, "weights_per_s": nb * 256 / (ms * 1e-3), "gbs_algorithmic": nb * 2192 / (ms * 1e-3) / 1e9,
+           "frac_of_hbm_peak": nb * 2192 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    if cpu:
+        # C oracle (scalar byte map, OpenMP over blocks) on the whole matrix, compared bit for bit
+        import numpy as np
+        from oracle import oracle as O
+        host = raw.cpu().numpy()
+        O.kquant_to_field(host[:64], "Q4_K", 4096)
+        c0 = time.perf_counter()
+        want = O.kquant_to_field(host, "Q4_K", 4096)
+        dt = time.perf_counter() - c0
+        got = kq.kquant_to_field(raw, "Q4_K", 4096).cpu().numpy()
+        res["cpu_baseline"] = {"value": nb * 256 / dt, "unit": "weights/s", "cores": O.num_threads(), "kind": "port",
+                               "sample": f"all {nb} super-blocks, {dt:.2f} s wall",
+                               "bit_exact_vs_gpu": bool(np.array_equal(got, want))}
+    return res
 
 
 def bench_layer(torch):
