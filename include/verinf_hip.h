@@ -166,6 +166,35 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
                       vi_coin_fn coin, void *user, uint64_t *host_samples, uint64_t *out_samples,
                       uint64_t *out_challenges, void *ws, size_t ws_bytes, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * BLAKE3 column digests and Merkle levels of a committed codeword matrix.
+ *
+ * vi_hash_columns replaces hash_columns_streamed (prover/cuda_primitives.py:1252-1254,
+ * kernel prover/kernels/blake3_columns.cuh:47-170): digests[j] = BLAKE3 of column j of the
+ * row-major (m, n) matrix (row pitch row_stride words) taken as m little-endian 8-byte words,
+ * the leaf prover/protocol.py:100-104 defines.  m = 0 hashes the empty message.
+ * Workspace: vi_hash_columns_workspace_bytes(m, n) = 48 * n * ceil(m / 128) bytes.
+ *
+ * vi_hash_columns_update / _finalize replace the streaming accumulator
+ * (prover/cuda_primitives.py:1297-1386: hash_columns_stream_init/_update/_finalize): the matrix
+ * arrives in row slabs; every slab but the last holds a multiple of 128 rows (one BLAKE3 chunk)
+ * and states its first chunk's index chunk0; n_chunks_total = ceil(m / 128) is fixed up front.
+ * Slabs may arrive in any order and on any stream as long as finalize is ordered after them.
+ * The workspace is the accumulator state and must persist from the first update to finalize.
+ *
+ * vi_merkle_level replaces merkle_one_level + the odd-node duplication around it
+ * (prover/cuda_primitives.py:1388-1402, layergkr/rs.py:135-144): out[i] = BLAKE3(nodes[2i] ||
+ * nodes[2i+1]) over 32-byte nodes, the odd last node paired with itself; out holds
+ * ceil(count / 2) nodes.  nodes and out must not overlap. */
+size_t vi_hash_columns_workspace_bytes(int64_t m, int64_t n);
+int vi_hash_columns(const uint64_t *mat, int64_t m, int64_t n, int64_t row_stride, uint8_t *digests, void *ws,
+                    size_t ws_bytes, void *stream);
+int vi_hash_columns_update(const uint64_t *rows, int64_t slab_rows, int64_t n, int64_t row_stride, int64_t chunk0,
+                           int64_t n_chunks_total, void *ws, size_t ws_bytes, void *stream);
+int vi_hash_columns_finalize(int64_t n, int64_t n_chunks_total, void *ws, size_t ws_bytes, uint8_t *digests,
+                             void *stream);
+int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -66,6 +66,10 @@ def lib():
         L.vo_kquant_to_field.restype = c_int
         L.vo_kquant_to_field.argtypes = [c_int, u8p, c_size_t, c_double, u64p]
         L.vo_num_threads.restype = c_int
+        L.vo_blake3.argtypes = [u8p, c_size_t, u8p]
+        L.vo_hash_columns.argtypes = [u64p, c_size_t, c_size_t, u8p]
+        L.vo_merkle_level.restype = c_size_t
+        L.vo_merkle_level.argtypes = [u8p, c_size_t, u8p]
         _lib = L
     return _lib
 
@@ -170,6 +174,46 @@ def kquant_to_field(raw: np.ndarray, qtype: str, S: float) -> np.ndarray:
                                   float(S), _p64(out))
     assert rc == 0
     return out
+
+
+def _p8(a: np.ndarray):
+    return a.ctypes.data_as(POINTER(c_uint8))
+
+
+def blake3(data: bytes) -> bytes:
+    """32-byte BLAKE3 digest (default hash mode)."""
+    buf = np.frombuffer(bytes(data) + b"\x00", dtype=np.uint8).copy()
+    out = np.empty(32, dtype=np.uint8)
+    lib().vo_blake3(_p8(buf), len(data), _p8(out))
+    return out.tobytes()
+
+
+def hash_columns(mat: np.ndarray) -> np.ndarray:
+    """(m, n) uint64 -> (n, 32) uint8: BLAKE3 of each column's little-endian words."""
+    mat = np.ascontiguousarray(mat, dtype=np.uint64)
+    m, n = mat.shape
+    out = np.empty((n, 32), dtype=np.uint8)
+    if n:
+        lib().vo_hash_columns(_p64(mat if m else np.zeros(1, dtype=np.uint64)), m, n, _p8(out))
+    return out
+
+
+def merkle_level(nodes: np.ndarray) -> np.ndarray:
+    """(k, 32) uint8 -> (ceil(k/2), 32): parent = BLAKE3(left || right), odd last node doubled."""
+    nodes = np.ascontiguousarray(nodes, dtype=np.uint8).reshape(-1, 32)
+    k = nodes.shape[0]
+    out = np.empty(((k + 1) // 2, 32), dtype=np.uint8)
+    got = lib().vo_merkle_level(_p8(nodes), k, _p8(out))
+    assert got == out.shape[0]
+    return out
+
+
+def merkle_levels(leaves: np.ndarray):
+    """All levels from the leaves up to the (1, 32) root."""
+    levels = [np.ascontiguousarray(leaves, dtype=np.uint8).reshape(-1, 32)]
+    while levels[-1].shape[0] > 1:
+        levels.append(merkle_level(levels[-1]))
+    return levels
 
 
 # ------------------------------------------------- pure-Python definitions ----

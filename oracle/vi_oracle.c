@@ -412,3 +412,124 @@ int vo_num_threads(void) {
     return 1;
 #endif
 }
+
+/* ---- BLAKE3 (column hashing / Merkle), restated from the published specification ----
+ * The reference hashes committed columns with BLAKE3 (prover/kernels/blake3_compress.cuh,
+ * blake3_hash.cuh, blake3_columns.cuh, merkle.cuh; leaf = BLAKE3 of the column's values as
+ * little-endian 8-byte words, prover/protocol.py:100-105; parent = BLAKE3(left || right),
+ * layergkr/rs.py:135-146).  The third-party `blake3` package (1.0.9 in uv.lock) is not
+ * available offline; this is the algorithm of the BLAKE3 paper, pinned by the four
+ * single-chunk known answers the reference's own test holds
+ * (prover/kernels/tests/test_blake3.cu:94-101) and by multi-chunk known answers of the
+ * official test-vector file quoted in tests/test_oracle.py. */
+static const uint32_t B3_IV[8] = {0x6A09E667u, 0xBB67AE85u, 0x3C6EF372u, 0xA54FF53Au,
+                                  0x510E527Fu, 0x9B05688Cu, 0x1F83D9ABu, 0x5BE0CD19u};
+static const uint8_t B3_PERM[16] = {2, 6, 3, 10, 7, 0, 4, 13, 1, 11, 12, 5, 9, 14, 15, 8};
+enum { B3_CHUNK_START = 1, B3_CHUNK_END = 2, B3_PARENT = 4, B3_ROOT = 8 };
+
+static inline uint32_t rotr32(uint32_t x, int n) { return (x >> n) | (x << (32 - n)); }
+
+static void b3_g(uint32_t *s, int a, int b, int c, int d, uint32_t mx, uint32_t my) {
+    s[a] = s[a] + s[b] + mx; s[d] = rotr32(s[d] ^ s[a], 16);
+    s[c] = s[c] + s[d];      s[b] = rotr32(s[b] ^ s[c], 12);
+    s[a] = s[a] + s[b] + my; s[d] = rotr32(s[d] ^ s[a], 8);
+    s[c] = s[c] + s[d];      s[b] = rotr32(s[b] ^ s[c], 7);
+}
+
+/* out[0..7] = first half of the compression output (the chaining value / digest words) */
+static void b3_compress(const uint32_t cv[8], const uint32_t block[16], u64 counter, uint32_t block_len,
+                        uint32_t flags, uint32_t out[8]) {
+    uint32_t s[16], m[16], t[16];
+    for (int i = 0; i < 8; ++i) s[i] = cv[i];
+    for (int i = 0; i < 4; ++i) s[8 + i] = B3_IV[i];
+    s[12] = (uint32_t)counter; s[13] = (uint32_t)(counter >> 32); s[14] = block_len; s[15] = flags;
+    memcpy(m, block, sizeof m);
+    for (int r = 0; r < 7; ++r) {
+        b3_g(s, 0, 4, 8, 12, m[0], m[1]);   b3_g(s, 1, 5, 9, 13, m[2], m[3]);
+        b3_g(s, 2, 6, 10, 14, m[4], m[5]);  b3_g(s, 3, 7, 11, 15, m[6], m[7]);
+        b3_g(s, 0, 5, 10, 15, m[8], m[9]);  b3_g(s, 1, 6, 11, 12, m[10], m[11]);
+        b3_g(s, 2, 7, 8, 13, m[12], m[13]); b3_g(s, 3, 4, 9, 14, m[14], m[15]);
+        for (int i = 0; i < 16; ++i) t[i] = m[B3_PERM[i]];
+        memcpy(m, t, sizeof m);
+    }
+    for (int i = 0; i < 8; ++i) out[i] = s[i] ^ s[i + 8];
+}
+
+static void b3_load_block(const uint8_t *p, size_t len, uint32_t block[16]) {
+    uint8_t buf[64];
+    memset(buf, 0, 64);
+    memcpy(buf, p, len);
+    for (int i = 0; i < 16; ++i)
+        block[i] = (uint32_t)buf[4 * i] | ((uint32_t)buf[4 * i + 1] << 8) | ((uint32_t)buf[4 * i + 2] << 16) |
+                   ((uint32_t)buf[4 * i + 3] << 24);
+}
+
+/* chaining value of one chunk (<= 1024 bytes); `root` marks a single-chunk message */
+static void b3_chunk_cv(const uint8_t *p, size_t len, u64 chunk_index, int root, uint32_t cv_out[8]) {
+    uint32_t cv[8], block[16];
+    memcpy(cv, B3_IV, sizeof cv);
+    size_t n_blocks = len == 0 ? 1 : (len + 63) / 64;
+    for (size_t b = 0; b < n_blocks; ++b) {
+        size_t off = b * 64, bl = len - off < 64 ? len - off : 64;
+        uint32_t flags = 0;
+        if (b == 0) flags |= B3_CHUNK_START;
+        if (b == n_blocks - 1) flags |= B3_CHUNK_END | (root ? B3_ROOT : 0);
+        b3_load_block(p + off, bl, block);
+        b3_compress(cv, block, chunk_index, (uint32_t)bl, flags, cv);
+    }
+    memcpy(cv_out, cv, sizeof cv);
+}
+
+/* subtree over chunks [first, first + n): left child takes the largest power of two < n */
+static void b3_subtree(const uint8_t *p, size_t len, u64 first_chunk, int root, uint32_t cv_out[8]) {
+    size_t n = len == 0 ? 1 : (len + 1023) / 1024;
+    if (n == 1) { b3_chunk_cv(p, len, first_chunk, root, cv_out); return; }
+    size_t left = 1;
+    while (left * 2 < n) left *= 2;
+    uint32_t block[16];
+    b3_subtree(p, left * 1024, first_chunk, 0, block);
+    b3_subtree(p + left * 1024, len - left * 1024, first_chunk + left, 0, block + 8);
+    b3_compress(B3_IV, block, 0, 64, B3_PARENT | (root ? B3_ROOT : 0), cv_out);
+}
+
+void vo_blake3(const uint8_t *data, size_t len, uint8_t out[32]) {
+    uint32_t cv[8];
+    b3_subtree(data, len, 0, 1, cv);
+    for (int i = 0; i < 8; ++i) {
+        out[4 * i] = (uint8_t)cv[i]; out[4 * i + 1] = (uint8_t)(cv[i] >> 8);
+        out[4 * i + 2] = (uint8_t)(cv[i] >> 16); out[4 * i + 3] = (uint8_t)(cv[i] >> 24);
+    }
+}
+
+/* prover/cuda_primitives.py:796-808 + prover/protocol.py:100-105: digest of every column of a
+ * row-major (m, n) matrix, column bytes = its m values as little-endian 8-byte words */
+void vo_hash_columns(const u64 *mat, size_t m, size_t n, uint8_t *out /* n x 32 */) {
+    #pragma omp parallel
+    {
+        uint8_t *col = (uint8_t *)malloc(m * 8 + 8);
+        #pragma omp for schedule(static)
+        for (long j = 0; j < (long)n; ++j) {
+            for (size_t i = 0; i < m; ++i) {
+                u64 v = mat[i * n + (size_t)j];
+                for (int b = 0; b < 8; ++b) col[i * 8 + b] = (uint8_t)(v >> (8 * b));
+            }
+            vo_blake3(col, m * 8, out + (size_t)j * 32);
+        }
+        free(col);
+    }
+}
+
+/* one Merkle level, layergkr/rs.py:135-146 / prover/cuda_primitives.py:1385-1401:
+ * parent = BLAKE3(left || right); an odd last node is paired with itself.  Returns the
+ * number of parents written. */
+size_t vo_merkle_level(const uint8_t *nodes, size_t n, uint8_t *out) {
+    size_t parents = (n + 1) / 2;
+    #pragma omp parallel for schedule(static)
+    for (long i = 0; i < (long)parents; ++i) {
+        uint8_t buf[64];
+        memcpy(buf, nodes + (size_t)i * 64, 32);
+        memcpy(buf + 32, nodes + ((size_t)(2 * i + 1) < n ? (size_t)(2 * i + 1) : (size_t)(2 * i)) * 32, 32);
+        vo_blake3(buf, 64, out + (size_t)i * 32);
+    }
+    return parents;
+}

@@ -26,6 +26,8 @@ EXPORTS = [
     "vi_coset_lde",
     "vi_kquant_to_field",
     "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval", "vi_sumcheck_prove",
+    "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
+    "vi_merkle_level",
 ]
 
 COIN_FN = ctypes.CFUNCTYPE(c_int, c_int, POINTER(c_uint64), c_int, POINTER(c_uint64), c_void_p)
@@ -82,12 +84,19 @@ def lib():
     L.vi_sumcheck_prove.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int,
                                     COIN_FN, vp, vp, POINTER(u64), POINTER(u64), vp, sz, vp]
     L.vi_sumcheck_prove.restype = c_int
+    L.vi_hash_columns_workspace_bytes.restype = sz
+    L.vi_hash_columns_workspace_bytes.argtypes = [i64, i64]
+    L.vi_hash_columns.argtypes = [vp, i64, i64, i64, vp, vp, sz, vp]
+    L.vi_hash_columns_update.argtypes = [vp, i64, i64, i64, i64, i64, vp, sz, vp]
+    L.vi_hash_columns_finalize.argtypes = [i64, i64, vp, sz, vp, vp]
+    L.vi_merkle_level.argtypes = [vp, i64, vp, vp]
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
                  "vi_ntt_batched", "vi_coset_lde", "vi_kquant_to_field", "vi_sumcheck_eval",
-                 "vi_sumcheck_fold_eval"):
+                 "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
+                 "vi_merkle_level"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

@@ -1,0 +1,234 @@
+// BLAKE3 column hashing and Merkle levels for committed codeword matrices.
+//
+// digest_j = BLAKE3(column j of a row-major (m, n) uint64 matrix as little-endian bytes)
+// (prover/cuda_primitives.py:796-808, prover/protocol.py:100-105); a Merkle parent is
+// BLAKE3(left || right), an odd last node is paired with itself (layergkr/rs.py:135-146).
+//
+// The reference walks a whole column with one thread and keeps BLAKE3's merge stack
+// per column (prover/kernels/blake3_columns.cuh:47-170).  Here the work is split the
+// other way: k_chunk_cvs gives every (1 KiB chunk, column) pair its own thread -- lanes
+// run along the columns, so the eight 8-byte loads of a 64-byte block are each one
+// coalesced 512-byte wavefront access -- and stores the chunk's chaining value;
+// k_merge_level then halves the number of chaining values per launch.  Pairing adjacent
+// nodes and carrying an odd last node up unchanged reproduces BLAKE3's left-full tree,
+// and the last merge carries the ROOT flag.  The chunk stage is therefore a streaming
+// pass over the matrix with as many independent threads as the GPU wants, and it can be
+// fed in row slabs (vi_hash_columns_update) while the codewords are produced.
+#include "common.hpp"
+
+namespace {
+
+typedef uint32_t u32;
+typedef uint64_t u64;
+typedef int64_t i64;
+
+constexpr int BLOCK = 256;
+constexpr u32 CHUNK_START = 1, CHUNK_END = 2, PARENT = 4, ROOT = 8;
+constexpr int ROWS_PER_CHUNK = 128;          // 1024 bytes of 8-byte words
+constexpr int ROWS_PER_BLOCK = 8;            // 64 bytes
+
+__device__ __constant__ const u32 IV[8] = {0x6A09E667u, 0xBB67AE85u, 0x3C6EF372u, 0xA54FF53Au,
+                                           0x510E527Fu, 0x9B05688Cu, 0x1F83D9ABu, 0x5BE0CD19u};
+
+// message word index used at position i of round r (the round permutation applied r times)
+__host__ __device__ constexpr int sched(int r, int i) {
+    constexpr int perm[16] = {2, 6, 3, 10, 7, 0, 4, 13, 1, 11, 12, 5, 9, 14, 15, 8};
+    int idx = i;
+    for (int k = 0; k < r; ++k) idx = perm[idx];
+    return idx;
+}
+
+__device__ __forceinline__ u32 rotr(u32 x, int n) { return __builtin_amdgcn_alignbit(x, x, n); }
+
+#define B3_G(a, b, c, d, mx, my)            \
+    a = a + b + (mx); d = rotr(d ^ a, 16);  \
+    c = c + d;        b = rotr(b ^ c, 12);  \
+    a = a + b + (my); d = rotr(d ^ a, 8);   \
+    c = c + d;        b = rotr(b ^ c, 7);
+
+template <int R>
+__device__ __forceinline__ void b3_round(u32 (&s)[16], const u32 (&m)[16]) {
+    B3_G(s[0], s[4], s[8], s[12], m[sched(R, 0)], m[sched(R, 1)])
+    B3_G(s[1], s[5], s[9], s[13], m[sched(R, 2)], m[sched(R, 3)])
+    B3_G(s[2], s[6], s[10], s[14], m[sched(R, 4)], m[sched(R, 5)])
+    B3_G(s[3], s[7], s[11], s[15], m[sched(R, 6)], m[sched(R, 7)])
+    B3_G(s[0], s[5], s[10], s[15], m[sched(R, 8)], m[sched(R, 9)])
+    B3_G(s[1], s[6], s[11], s[12], m[sched(R, 10)], m[sched(R, 11)])
+    B3_G(s[2], s[7], s[8], s[13], m[sched(R, 12)], m[sched(R, 13)])
+    B3_G(s[3], s[4], s[9], s[14], m[sched(R, 14)], m[sched(R, 15)])
+}
+
+// cv <- first eight words of compress(cv, m, counter, block_len, flags)
+__device__ __forceinline__ void compress(u32 (&cv)[8], const u32 (&m)[16], u64 counter, u32 block_len, u32 flags) {
+    u32 s[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] = cv[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s[8 + i] = IV[i];
+    s[12] = (u32)counter;
+    s[13] = (u32)(counter >> 32);
+    s[14] = block_len;
+    s[15] = flags;
+    b3_round<0>(s, m); b3_round<1>(s, m); b3_round<2>(s, m); b3_round<3>(s, m);
+    b3_round<4>(s, m); b3_round<5>(s, m); b3_round<6>(s, m);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cv[i] = s[i] ^ s[i + 8];
+}
+
+// Chaining value of chunk (chunk0 + blockIdx.y) of every column.
+//   rows          first row of the slab (row pitch `stride` words), slab_rows rows in it
+//   single_root   the whole message is this one chunk: its last block carries ROOT
+// cvs[(chunk0 + c) * n + col] receives 8 words.
+__global__ __launch_bounds__(BLOCK) void k_chunk_cvs(const u64 *__restrict__ rows, i64 slab_rows, i64 n, i64 stride, i64 chunk0,
+                                                     int single_root, u32 *__restrict__ cvs) {
+    const i64 col = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    if (col >= n) return;
+    const i64 c = blockIdx.y;
+    const i64 r0 = c * ROWS_PER_CHUNK;
+    const i64 nrows = (slab_rows - r0 < ROWS_PER_CHUNK) ? (slab_rows - r0) : ROWS_PER_CHUNK;   // >= 0
+    const int n_blocks = nrows == 0 ? 1 : (int)((nrows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK);
+    const u64 *p = rows + r0 * stride + col;
+    u32 cv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cv[i] = IV[i];
+    for (int b = 0; b < n_blocks; ++b) {
+        u32 m[16];
+        const i64 left = nrows - (i64)b * ROWS_PER_BLOCK;
+        const int here = left >= ROWS_PER_BLOCK ? ROWS_PER_BLOCK : (int)left;
+#pragma unroll
+        for (int i = 0; i < ROWS_PER_BLOCK; ++i) {
+            u64 v = i < here ? p[((i64)b * ROWS_PER_BLOCK + i) * stride] : 0;
+            m[2 * i] = (u32)v;
+            m[2 * i + 1] = (u32)(v >> 32);
+        }
+        u32 flags = 0;
+        if (b == 0) flags |= CHUNK_START;
+        if (b == n_blocks - 1) flags |= CHUNK_END | (single_root ? ROOT : 0u);
+        compress(cv, m, (u64)(chunk0 + c), (u32)(here * 8), flags);
+    }
+    u32 *o = cvs + ((chunk0 + c) * n + col) * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = cv[i];
+}
+
+// One level of BLAKE3's internal tree over `count` nodes per column: node pairs (2i, 2i+1)
+// become a parent, an odd last node moves up unchanged.  in/out: [node][col][8 words].
+__global__ __launch_bounds__(BLOCK) void k_merge_level(const u32 *__restrict__ in, i64 count, i64 n, int is_root_level,
+                                                       u32 *__restrict__ out) {
+    const i64 col = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    if (col >= n) return;
+    const i64 i = blockIdx.y;                       // parent index
+    const u32 *l = in + ((2 * i) * n + col) * 8;
+    u32 *o = out + (i * n + col) * 8;
+    if (2 * i + 1 >= count) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o[k] = l[k];
+        return;
+    }
+    const u32 *r = in + ((2 * i + 1) * n + col) * 8;
+    u32 m[16], cv[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { m[k] = l[k]; m[8 + k] = r[k]; cv[k] = IV[k]; }
+    compress(cv, m, 0, 64, PARENT | (is_root_level ? ROOT : 0u));
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = cv[k];
+}
+
+// Merkle level over 32-byte nodes: parent i = BLAKE3(node[2i] || node[2i+1]), the odd last
+// node is paired with itself.  A 64-byte message is one block: CHUNK_START|CHUNK_END|ROOT.
+__global__ __launch_bounds__(BLOCK) void k_merkle_level(const u32 *__restrict__ nodes, i64 count, u32 *__restrict__ out) {
+    const i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    const i64 parents = (count + 1) / 2;
+    if (i >= parents) return;
+    const u32 *l = nodes + (2 * i) * 8;
+    const u32 *r = nodes + ((2 * i + 1 < count) ? (2 * i + 1) : (2 * i)) * 8;
+    u32 m[16], cv[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { m[k] = l[k]; m[8 + k] = r[k]; cv[k] = IV[k]; }
+    compress(cv, m, 0, 64, CHUNK_START | CHUNK_END | ROOT);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) out[i * 8 + k] = cv[k];
+}
+
+inline i64 chunks_of(i64 m) { return m <= 0 ? 1 : (m + ROWS_PER_CHUNK - 1) / ROWS_PER_CHUNK; }
+
+}  // namespace
+
+extern "C" {
+
+size_t vi_hash_columns_workspace_bytes(int64_t m, int64_t n) {
+    if (m < 0 || n <= 0) return 0;
+    // chunk chaining values + one ping-pong level
+    i64 c = chunks_of(m);
+    return (size_t)(c + (c + 1) / 2) * (size_t)n * 32;
+}
+
+int vi_hash_columns_update(const uint64_t *rows, int64_t slab_rows, int64_t n, int64_t row_stride, int64_t chunk0,
+                           int64_t n_chunks_total, void *ws, size_t ws_bytes, void *stream) {
+    if (n <= 0 || slab_rows < 0 || row_stride < n || chunk0 < 0 || n_chunks_total < 1)
+        return vi::fail(VI_EINVAL, "vi_hash_columns_update: bad shape rows=%lld n=%lld stride=%lld", (long long)slab_rows, (long long)n, (long long)row_stride);
+    const i64 slab_chunks = chunks_of(slab_rows);
+    if (chunk0 + slab_chunks > n_chunks_total) return vi::fail(VI_EINVAL, "vi_hash_columns_update: slab exceeds the declared %lld chunks", (long long)n_chunks_total);
+    if (chunk0 + slab_chunks < n_chunks_total && slab_rows % ROWS_PER_CHUNK)
+        return vi::fail(VI_EINVAL, "vi_hash_columns_update: only the last slab may hold a partial 128-row chunk");
+    if (slab_rows == 0 && n_chunks_total > 1) return vi::fail(VI_EINVAL, "vi_hash_columns_update: empty slab of a multi-chunk message");
+    if (slab_rows > 0 && !rows) return vi::fail(VI_EINVAL, "vi_hash_columns_update: null rows");
+    if (!ws || ws_bytes < (size_t)(n_chunks_total + (n_chunks_total + 1) / 2) * (size_t)n * 32)
+        return vi::fail(VI_ENOMEM, "vi_hash_columns_update: workspace too small");
+    if (slab_chunks > 65535) return vi::fail(VI_EINVAL, "vi_hash_columns_update: at most 65535 chunks (8,388,480 rows) per call");
+    dim3 grid((unsigned)((n + BLOCK - 1) / BLOCK), (unsigned)slab_chunks);
+    hipLaunchKernelGGL(k_chunk_cvs, grid, dim3(BLOCK), 0, (hipStream_t)stream, rows, (i64)slab_rows, (i64)n, (i64)row_stride,
+                       (i64)chunk0, n_chunks_total == 1 ? 1 : 0, (u32 *)ws);
+    VI_LAUNCH_CHECK("k_chunk_cvs");
+    return VI_OK;
+}
+
+int vi_hash_columns_finalize(int64_t n, int64_t n_chunks_total, void *ws, size_t ws_bytes, uint8_t *digests, void *stream) {
+    if (n <= 0 || n_chunks_total < 1 || !digests) return vi::fail(VI_EINVAL, "vi_hash_columns_finalize: bad arguments");
+    if (!ws || ws_bytes < (size_t)(n_chunks_total + (n_chunks_total + 1) / 2) * (size_t)n * 32)
+        return vi::fail(VI_ENOMEM, "vi_hash_columns_finalize: workspace too small");
+    hipStream_t s = (hipStream_t)stream;
+    u32 *a = (u32 *)ws;                               // n_chunks_total nodes
+    u32 *b = a + (size_t)n_chunks_total * n * 8;      // ceil(n_chunks_total / 2) nodes
+    i64 count = n_chunks_total;
+    while (count > 1) {
+        const i64 parents = (count + 1) / 2;
+        for (i64 lo = 0; lo < parents; lo += 65535) {             // grid.y limit
+            const i64 cnt = parents - lo < 65535 ? parents - lo : 65535;
+            dim3 grid((unsigned)((n + BLOCK - 1) / BLOCK), (unsigned)cnt);
+            hipLaunchKernelGGL(k_merge_level, grid, dim3(BLOCK), 0, s, (const u32 *)(a + (size_t)(2 * lo) * n * 8), count - 2 * lo,
+                               (i64)n, parents == 1 ? 1 : 0, b + (size_t)lo * n * 8);
+            VI_LAUNCH_CHECK("k_merge_level");
+        }
+        u32 *t = a; a = b; b = t;
+        count = parents;
+    }
+    VI_HIP(hipMemcpyAsync(digests, a, (size_t)n * 32, hipMemcpyDeviceToDevice, s));
+    return VI_OK;
+}
+
+int vi_hash_columns(const uint64_t *mat, int64_t m, int64_t n, int64_t row_stride, uint8_t *digests, void *ws,
+                    size_t ws_bytes, void *stream) {
+    if (m < 0) return vi::fail(VI_EINVAL, "vi_hash_columns: m = %lld", (long long)m);
+    const i64 total = chunks_of(m);
+    for (i64 c0 = 0; c0 < total; c0 += 65535) {
+        const i64 cc = total - c0 < 65535 ? total - c0 : 65535;
+        const i64 r0 = c0 * ROWS_PER_CHUNK;
+        const i64 rows = (c0 + cc == total) ? m - r0 : cc * ROWS_PER_CHUNK;
+        int rc = vi_hash_columns_update(mat ? mat + r0 * row_stride : nullptr, rows, n, row_stride, c0, total, ws, ws_bytes, stream);
+        if (rc) return rc;
+    }
+    return vi_hash_columns_finalize(n, total, ws, ws_bytes, digests, stream);
+}
+
+int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *stream) {
+    if (count < 1 || !nodes || !out) return vi::fail(VI_EINVAL, "vi_merkle_level: bad arguments");
+    if (((uintptr_t)nodes | (uintptr_t)out) & 3) return vi::fail(VI_EINVAL, "vi_merkle_level: nodes must be 4-byte aligned");
+    const i64 parents = (count + 1) / 2;
+    hipLaunchKernelGGL(k_merkle_level, dim3((unsigned)((parents + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, (hipStream_t)stream,
+                       (const u32 *)nodes, (i64)count, (u32 *)out);
+    VI_LAUNCH_CHECK("k_merkle_level");
+    return VI_OK;
+}
+
+}  // extern "C"

@@ -158,6 +158,25 @@ def combine_t(cfg: Config, mat, coeffs: Sequence[int]):
     return cp.gl_matmul(_u64_row(coeffs), mat)
 
 
+def hash_and_tree(cfg: Config, mat):
+    """Column digests and the Merkle tree of a device codeword matrix, both computed on the
+    device (gpu.py:274-288): returns (root bytes, list of (k_i, 32) uint8 level tensors)."""
+    _require_gpu()
+    dig = cp.hash_columns_streamed(mat)
+    root_t, levels_t = cp.merkle_build_blake3(dig)
+    return bytes(root_t.cpu().tolist()), levels_t
+
+
+def levels_to_host(levels_t):
+    """The (small) tree as lists of 32-byte nodes, so that opening paths cost nothing
+    (gpu.py:291-297)."""
+    out = []
+    for lvl in levels_t:
+        raw = lvl.cpu().numpy().tobytes()
+        out.append([raw[32 * r:32 * r + 32] for r in range(lvl.shape[0])])
+    return out
+
+
 def column(mat, col: int):
     """One codeword column back to the host."""
     return [int(v) for v in mat.view(torch.int64)[:, col].contiguous().view(torch.uint64).cpu().tolist()]

@@ -6,15 +6,46 @@ device codewords with the Lagrange definition `protocol.eval_zeta_form` -- whole
 codewords at small geometries, sampled columns at large ones -- and a failing
 gate raises instead of switching to another encoder.
 
-Column hashing and the Merkle tree (rs.py:135-157, BLAKE3) are outside this
-package, so a Commit here carries the codeword matrix and the linear operations on
-it, not a root.
+The commitment itself (rs.py:135-157, 160-252) is the device path of the reference:
+the codeword matrix never leaves the GPU, `gpu.hash_and_tree` hashes its columns and
+builds the Merkle tree there, and only the tree (32 bytes per node) and the opened
+columns come back to the host.
 """
-from typing import List, Sequence
+from typing import List, Sequence, Tuple
 
-from ..prover.protocol import Config, P, eval_zeta_form  # noqa: F401  (re-exported like the reference)
+from ..prover.protocol import (  # noqa: F401  (re-exported like the reference)
+    Config, P, blake3_digest, eval_zeta_form, merkle_leaf, merkle_verify)
 
 Codeword = List[int]
+Path = List[Tuple[bytes, int]]
+
+
+def _b3(a: bytes, b: bytes) -> bytes:
+    return blake3_digest(a + b)
+
+
+def build_tree(leaves: List[bytes]) -> List[List[bytes]]:
+    """Host-side tree over a few leaves (rs.py:135-144): levels[0] = leaves, last level =
+    [root]; an odd node is paired with itself.  The device builds the same tree in
+    cuda_primitives.merkle_build_blake3."""
+    levels = [list(leaves)]
+    while len(levels[-1]) > 1:
+        cur = levels[-1]
+        levels.append([_b3(cur[i], cur[i + 1] if i + 1 < len(cur) else cur[i]) for i in range(0, len(cur), 2)])
+    return levels
+
+
+def merkle_path(levels: List[List[bytes]], idx: int) -> Path:
+    """Opening path of leaf `idx` as (sibling, side) pairs, side 1 = sibling on the right
+    (rs.py:147-157); a missing sibling is the node itself."""
+    path: Path = []
+    for level in levels[:-1]:
+        sib = idx ^ 1
+        if sib >= len(level):
+            sib = idx
+        path.append((level[sib], 1 if (idx & 1) == 0 else 0))
+        idx //= 2
+    return path
 
 _NTT_OK: dict = {}
 
@@ -44,11 +75,21 @@ def encode_row(cfg: Config, message: Sequence[int]) -> Codeword:
 
 
 class Commit:
-    """Reed-Solomon codewords of a set of rows, resident on the device."""
+    """A column-Merkle commitment to Reed-Solomon codewords that stay on the device
+    (the `mat=` branch of rs.py:176-187).  Hashing happens on first use of `root`,
+    `levels` or `open`, so callers that only encode and combine do not pay for it."""
 
     def __init__(self, cfg: Config, mat):
         self.cfg = cfg
         self.mat = mat
+        self._root = None
+        self._levels_dev = None
+        self._levels = None
+
+    def _hash(self):
+        if self._root is None:
+            from . import gpu
+            self._root, self._levels_dev = gpu.hash_and_tree(self.cfg, self.mat)
 
     @classmethod
     def from_messages(cls, cfg: Config, messages) -> "Commit":
@@ -83,4 +124,19 @@ class Commit:
 
     @property
     def root(self) -> bytes:
-        raise NotImplementedError("column hashing / Merkle tree are outside verinf_amd")
+        self._hash()
+        return self._root
+
+    @property
+    def levels(self) -> List[List[bytes]]:
+        if self._levels is None:
+            from . import gpu
+            self._hash()
+            self._levels = gpu.levels_to_host(self._levels_dev)
+        return self._levels
+
+    def open(self, col: int) -> Tuple[List[int], Path]:
+        return self.col_values(col), merkle_path(self.levels, col)
+
+    def check_open(self, col: int, values: List[int], path: Path) -> bool:
+        return merkle_verify(merkle_leaf(values), path, self.root)

@@ -338,3 +338,134 @@ def poly_mul_batched(A, B):
     prod = gl_mul(fa, fb)
     ntt_inverse_batched(prod)
     return prod.view(torch.int64)[:, :out_len].contiguous().view(torch.uint64)
+
+
+# ---- BLAKE3 column hash + Merkle (prover/cuda_primitives.py:1250-1402) ----
+
+_BLAKE3_CHUNK_ROWS = 128          # a BLAKE3 chunk is 1024 bytes = 128 uint64 rows of one column
+
+
+def _n_chunks(n_rows):
+    return max(1, (int(n_rows) + _BLAKE3_CHUNK_ROWS - 1) // _BLAKE3_CHUNK_ROWS)
+
+
+def hash_columns_streamed(matrix):
+    """(m, n) uint64 -> (n, 32) uint8 BLAKE3 column digests
+    (prover/cuda_primitives.py:1252-1254).  No row cap; rows may be strided, the
+    columns of a row must be adjacent."""
+    if not isinstance(matrix, torch.Tensor) or not matrix.is_cuda:
+        raise RuntimeError("matrix must be CUDA")
+    if matrix.dtype != torch.uint64:
+        raise RuntimeError("matrix dtype must be uint64")
+    if matrix.dim() != 2:
+        raise RuntimeError("matrix must be 2D")
+    m, n = int(matrix.shape[0]), int(matrix.shape[1])
+    if n == 0:
+        return torch.empty((0, 32), dtype=torch.uint8, device=matrix.device)
+    if n > 1 and m > 0 and matrix.stride(1) != 1:
+        raise RuntimeError("matrix must be contiguous")
+    stride = int(matrix.stride(0)) if m > 1 else n
+    if stride < n:
+        raise RuntimeError("matrix must be contiguous")
+    L = _lib.lib()
+    out = torch.empty((n, 32), dtype=torch.uint8, device=matrix.device)
+    nbytes = L.vi_hash_columns_workspace_bytes(m, n)
+    ws = _lib.workspace(nbytes, matrix.device, "hash")
+    _lib.check(L.vi_hash_columns(matrix.data_ptr(), m, n, stride, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                 _lib.stream_ptr()))
+    return out
+
+
+class MerkleColumnAccumulator:
+    """Column digests of a tall matrix that arrives in row slabs
+    (prover/cuda_primitives.py:1297-1386): same digests as hash_columns_streamed on
+    the concatenation, without ever holding the whole matrix.
+
+    `n_total_rows` is fixed up front.  update() takes any number of rows; rows
+    short of a 128-row BLAKE3 chunk are kept until a later call completes them.
+    All complete chunks of a slab go to the device in one launch, and the state
+    between calls is the table of chunk chaining values (32 bytes per chunk and
+    column).  Like the reference it wants more than one chunk in total."""
+
+    def __init__(self, n_cols: int, n_total_rows: int):
+        assert n_total_rows > _BLAKE3_CHUNK_ROWS, (
+            "MerkleColumnAccumulator requires multi-BLAKE3-chunk input; "
+            "for <=128 rows use hash_columns_streamed directly")
+        self.n_cols = int(n_cols)
+        self.n_total_rows = int(n_total_rows)
+        self.n_chunks_total = _n_chunks(n_total_rows)
+        L = _lib.lib()
+        nbytes = L.vi_hash_columns_workspace_bytes(self.n_total_rows, self.n_cols)
+        self._states = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        self._chunks_seen = 0
+        self._rows_seen = 0
+        self._partial = None
+
+    def _emit(self, rows):
+        L = _lib.lib()
+        rows = rows if rows.stride(1) == 1 else rows.contiguous()
+        k = int(rows.size(0))
+        _lib.check(L.vi_hash_columns_update(rows.data_ptr(), k, self.n_cols, int(rows.stride(0)) if k > 1 else self.n_cols,
+                                            self._chunks_seen, self.n_chunks_total, self._states.data_ptr(),
+                                            self._states.numel(), _lib.stream_ptr()))
+        self._chunks_seen += _n_chunks(k)
+        self._rows_seen += k
+
+    def update(self, rows):
+        """rows: (k, n_cols) uint64, any k >= 0."""
+        assert rows.dtype == torch.uint64 and rows.is_cuda
+        assert rows.dim() == 2 and rows.size(1) == self.n_cols
+        if self._partial is not None:
+            rows = torch.cat([self._partial, rows])
+            self._partial = None
+        k = int(rows.size(0))
+        if k == 0:
+            return
+        assert self._rows_seen + k <= self.n_total_rows, "more rows than n_total_rows"
+        if self._rows_seen + k == self.n_total_rows:
+            self._emit(rows)                       # the last slab may end in a partial chunk
+            return
+        full = (k // _BLAKE3_CHUNK_ROWS) * _BLAKE3_CHUNK_ROWS
+        if full:
+            self._emit(rows[:full])
+        if full < k:
+            self._partial = rows[full:].clone()
+
+    def finalize(self):
+        """Returns (n_cols, 32) uint8 column digests."""
+        assert self._chunks_seen == self.n_chunks_total, (
+            f"expected {self.n_chunks_total} chunks, saw {self._chunks_seen}"
+            f" (rows_seen={self._rows_seen}/{self.n_total_rows})")
+        L = _lib.lib()
+        out = torch.empty((self.n_cols, 32), dtype=torch.uint8, device=self._states.device)
+        _lib.check(L.vi_hash_columns_finalize(self.n_cols, self.n_chunks_total, self._states.data_ptr(),
+                                              self._states.numel(), out.data_ptr(), _lib.stream_ptr()))
+        return out
+
+
+def merkle_one_level(nodes):
+    """(k, 32) uint8 (or (k, 8) uint32) nodes -> (ceil(k / 2), 32) uint8 parents;
+    an odd last node is paired with itself (layergkr/rs.py:135-144)."""
+    if not nodes.is_cuda or not nodes.is_contiguous():
+        raise RuntimeError("nodes must be CUDA and contiguous")
+    k = int(nodes.size(0))
+    if k < 1 or nodes.numel() * nodes.element_size() != 32 * k:
+        raise RuntimeError("nodes must be (k, 32) uint8")
+    out = torch.empty(((k + 1) // 2, 32), dtype=torch.uint8, device=nodes.device)
+    _lib.check(_lib.lib().vi_merkle_level(nodes.data_ptr(), k, out.data_ptr(), _lib.stream_ptr()))
+    return out
+
+
+def merkle_build_blake3(leaves):
+    """(N, 32) uint8 leaves -> (root: (32,) uint8, levels: list of (k_i, 32) uint8);
+    levels[0] = leaves, levels[-1] = (1, 32) holding the root
+    (prover/cuda_primitives.py:1388-1402)."""
+    assert leaves.dim() == 2 and leaves.size(1) == 32
+    assert leaves.dtype == torch.uint8 and leaves.is_cuda
+    levels = [leaves]
+    cur = leaves.contiguous()
+    while cur.size(0) > 1:
+        cur = merkle_one_level(cur)
+        levels.append(cur)
+    root = levels[-1].view(-1)[:32].clone()
+    return root, levels
