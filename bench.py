@@ -174,14 +174,56 @@ def bench_kquant(torch, steps=20, cpu=True):
     return res
 
 
+def bench_hash(torch, steps=10, cpu=True):
+    """Column digests + Merkle tree of the headline codeword matrix (1024 x 2^18 uint64, 2 GiB):
+    what turns the LDE output into a commitment root."""
+    from verinf_amd.prover import cuda_primitives as cp
+    m, n = 1024, 1 << 18
+    g = torch.Generator(device="cuda").manual_seed(9)
+    mat = torch.randint(-(1 << 63), (1 << 63) - 1, (m, n), generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
+    for _ in range(2):
+        dig = cp.hash_columns_streamed(mat)
+        root, _ = cp.merkle_build_blake3(dig)
+    torch.cuda.synchronize()
+    s, e, e2 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_hash = t_tree = 0.0
+    for _ in range(steps):
+        s.record()
+        dig = cp.hash_columns_streamed(mat)
+        e.record()
+        root, _ = cp.merkle_build_blake3(dig)
+        e2.record()
+        torch.cuda.synchronize()
+        t_hash += s.elapsed_time(e)
+        t_tree += e.elapsed_time(e2)
+    hash_ms, tree_ms = t_hash / steps, t_tree / steps
+    alg = 8 * m * n + 32 * n
+    res = {"matrix": "1024 x 2^18 uint64", "hash_columns_ms": hash_ms, "hash_gbs_algorithmic": alg / hash_ms / 1e6,
+           "frac_of_hbm_peak": alg / hash_ms / 1e6 / HBM_PEAK_GBS, "merkle_tree_2^18_leaves_ms": tree_ms,
+           "root": bytes(root.cpu().tolist()).hex()}
+    if cpu:
+        import numpy as np
+        from oracle import oracle as O
+        cols = 1 << 16                      # 512 MiB sample of the same matrix
+        sub = mat.view(torch.int64)[:, :cols].contiguous().view(torch.uint64).cpu().numpy()
+        O.hash_columns(sub[:, :64].copy())
+        c0 = time.perf_counter()
+        want = O.hash_columns(sub)
+        dt = time.perf_counter() - c0
+        res["cpu_baseline"] = {"value": sub.nbytes / dt / 1e9, "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+                               "sample": f"first {cols} columns of the same matrix, {dt:.2f} s wall",
+                               "bit_exact_vs_gpu": bool(np.array_equal(dig[:cols].cpu().numpy(), want))}
+    return res
+
+
 def bench_layer(torch):
     """Config 5: one Llama-2-7B-shape layer proof core.  Commit = coset LDE of every weight
     and activation row at the production geometry ELL = 8192, K = 2^14, N = 2^16 (a row of
     n_in > 8192 values spans two rows); then the GKR sumchecks: one degree-2 contraction
     per matmul (width next_pow2(n_in), layergkr/full_layer.py:216-224) and one degree-3
-    eq*a*b gate batch over S*d_ff -> 2^24 (layergkr/relations.py:104-124).  Column hashing
-    and the projection seam between the two are outside this package; random field tables
-    stand in for the projected vectors."""
+    eq*a*b gate batch over S*d_ff -> 2^24 (layergkr/relations.py:104-124).  Every committed
+    matrix is hashed by column and gets its Merkle root (layergkr/rs.py:176-187).  Random field
+    tables stand in for the projected vectors of the sumchecks."""
     from verinf_amd.layergkr import gpu
     from verinf_amd.prover import cuda_primitives as cp
     d, dff, S = 4096, 11008, 1000
@@ -214,9 +256,14 @@ def bench_layer(torch):
     r = random.Random(7)
     coins = [r.randrange(P) for _ in range(24)]
 
-    def commit():
+    def commit(hash_too=True):
+        roots = []
         for m in msgs:
-            cp.coset_lde(m, K, N, 7, out=out[: m.shape[0]])
+            code = out[: m.shape[0]]
+            cp.coset_lde(m, K, N, 7, out=code)
+            if hash_too:
+                roots.append(cp.merkle_build_blake3(cp.hash_columns_streamed(code))[0])
+        return roots
 
     def sumchecks():
         for tabs in mm_tabs:
@@ -234,6 +281,10 @@ def bench_layer(torch):
 
     commit(); projections(); sumchecks()         # warm-up (twiddle tables, workspaces)
     torch.cuda.synchronize()
+    tl0 = time.perf_counter()
+    commit(hash_too=False)
+    torch.cuda.synchronize()
+    lde_only_s = time.perf_counter() - tl0
     t0 = time.perf_counter()
     commit()
     torch.cuda.synchronize()
@@ -255,8 +306,9 @@ def bench_layer(torch):
     return {"rows_committed": total_rows, "geometry": "ELL=8192 K=2^14 N=2^16",
             "end_to_end_ms": (t2 - t0) * 1e3,
             "projection_matvec_ms": proj_ms, "projection_matvec_gbs": proj_bytes / proj_ms / 1e6,
-            "commit_lde_ms": (t1 - t0) * 1e3, "commit_lde_gbs_algorithmic": lde_bytes / (t1 - t0) / 1e9,
-            "commit_lde_gelems_per_s": total_rows * N / (t1 - t0) / 1e9,
+            "commit_ms": (t1 - t0) * 1e3, "commit_hash_and_tree_ms": (t1 - t0 - lde_only_s) * 1e3,
+            "commit_lde_ms": lde_only_s * 1e3, "commit_lde_gbs_algorithmic": lde_bytes / lde_only_s / 1e9,
+            "commit_lde_gelems_per_s": total_rows * N / lde_only_s / 1e9,
             "sumchecks_ms": (t2 - t1b) * 1e3,
             "gate_sumcheck_2^24_deg3_ms": (t4 - t3) * 1e3,
             "gate_sumcheck_gbs_algorithmic": 96 * (1 << 24) / (t4 - t3) / 1e9,
@@ -283,7 +335,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
     ap.add_argument("--copy-probe", action="store_true")
     ap.add_argument("--ws-mb", type=int, default=0, help="override the LDE workspace size (MiB); 0 = library default")
-    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer"], default=None,
+    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer", "hash"], default=None,
                     help="run just one of the extra legs and print its JSON (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -304,6 +356,9 @@ def main():
     if args.only == "layer":
         print(json.dumps(bench_layer(torch)))
         return
+    if args.only == "hash":
+        print(json.dumps(bench_hash(torch)))
+        return
 
     lde, msgs, out = bench_lde(torch, args.steps, args.warmup, args.ws_mb)
     cpu = cpu_baseline_lde(torch, msgs, out, args.cpu_rows)
@@ -314,6 +369,8 @@ def main():
         extra["sumcheck_3x2^26_deg3"] = bench_sumcheck(torch)
         torch.cuda.empty_cache()
         extra["kquant_q4k_4096x11008"] = bench_kquant(torch)
+        torch.cuda.empty_cache()
+        extra["blake3_commit_1024x2^18"] = bench_hash(torch)
         torch.cuda.empty_cache()
         extra["llama2_7b_layer"] = bench_layer(torch)
 
