@@ -104,6 +104,23 @@ int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride
                  int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, void *ws,
                  size_t ws_bytes, void *stream);
 
+/* The two halves of the coset LDE for callers that keep the row polynomials, as the production prover
+ * does (prover/core.py:795-802: row_polys = iNTT_K(padded); codewords = _coset_encode_codewords(row_polys)).
+ *
+ * vi_coset_lde_coeffs: values -> coefficients (m rows of K words at `coeffs`, row pitch coeffs_stride >= K)
+ * and, when out is not NULL, on to the codewords exactly as vi_coset_lde.  The coefficients replace
+ * ntt_inverse_batched(padded.clone()) (prover/core.py:797-798); coeffs may equal `in` (same stride) for an
+ * in-place transform.  out == NULL is need_codewords=False (prover/core.py:799-800).
+ *
+ * vi_coset_extend: coefficients (m rows of `width` <= K words, the rest read as zero) -> codewords; replaces
+ * _coset_encode_codewords / _coset_encode_via_coset_ntt (prover/core.py:702-743).
+ * Workspace and chunking as for vi_coset_lde. */
+int vi_coset_lde_coeffs(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K, int64_t N,
+                        uint64_t shift, uint64_t *coeffs, int64_t coeffs_stride, uint64_t *out, int64_t out_stride,
+                        void *ws, size_t ws_bytes, void *stream);
+int vi_coset_extend(const uint64_t *coeffs, int64_t m, int64_t width, int64_t coeffs_stride, int64_t K, int64_t N,
+                    uint64_t shift, uint64_t *out, int64_t out_stride, void *ws, size_t ws_bytes, void *stream);
+
 /* ---- K-quant super-blocks -> field ---------------------------------------------
  * Replaces q4k_to_field / q5k_to_field / q6k_to_field behind kquant_to_field
  * (prover/kquant_cuda.py:60-139, 170-177): raw holds n_blocks super-blocks of
@@ -194,6 +211,15 @@ int vi_hash_columns_update(const uint64_t *rows, int64_t slab_rows, int64_t n, i
 int vi_hash_columns_finalize(int64_t n, int64_t n_chunks_total, void *ws, size_t ws_bytes, uint8_t *digests,
                              void *stream);
 int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *stream);
+
+/* Zero-knowledge pad generator; replaces row_prg / row_prg_indexed (prover/cuda_primitives.py:1262-1294,
+ * kernels :877-930): out[r * out_stride + k] = (BLAKE3(seed[32] || row_le8 || k_le8)[0:8] as a little-endian
+ * word) mod p for r < n_rows, k < slack, with row = row_indices[r] if row_indices is not NULL, else the
+ * 32-bit sum (uint32)(row_offset + r) as in the reference's contiguous variant.  seed is a device pointer.
+ * out_stride >= slack lets the pad be written straight into columns [ELL, K) of the padded message
+ * matrix (prover/core.py:783-794) without an intermediate tensor. */
+int vi_row_prg(const uint8_t *seed, const uint64_t *row_indices, int64_t row_offset, int64_t n_rows, int64_t slack,
+               uint64_t *out, int64_t out_stride, void *stream);
 
 #ifdef __cplusplus
 }

@@ -70,6 +70,7 @@ def lib():
         L.vo_hash_columns.argtypes = [u64p, c_size_t, c_size_t, u8p]
         L.vo_merkle_level.restype = c_size_t
         L.vo_merkle_level.argtypes = [u8p, c_size_t, u8p]
+        L.vo_row_prg.argtypes = [u8p, u64p, c_uint64, c_size_t, c_size_t, u64p]
         _lib = L
     return _lib
 
@@ -205,6 +206,20 @@ def merkle_level(nodes: np.ndarray) -> np.ndarray:
     out = np.empty(((k + 1) // 2, 32), dtype=np.uint8)
     got = lib().vo_merkle_level(_p8(nodes), k, _p8(out))
     assert got == out.shape[0]
+    return out
+
+
+def row_prg(seed: bytes, row_offset: int, n_rows: int, slack: int, row_indices=None) -> np.ndarray:
+    """(n_rows, slack) pad words: le64(BLAKE3(seed || row_le8 || k_le8)[:8]) mod p."""
+    assert len(seed) == 32
+    sd = np.frombuffer(bytes(seed), dtype=np.uint8).copy()
+    idx = None
+    if row_indices is not None:
+        idx = np.ascontiguousarray(row_indices, dtype=np.uint64)
+        n_rows = idx.size
+    out = np.empty((n_rows, slack), dtype=np.uint64)
+    if n_rows and slack:
+        lib().vo_row_prg(_p8(sd), _p64(idx) if idx is not None else None, int(row_offset) & ((1 << 64) - 1), n_rows, slack, _p64(out))
     return out
 
 

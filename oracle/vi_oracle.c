@@ -533,3 +533,23 @@ size_t vo_merkle_level(const uint8_t *nodes, size_t n, uint8_t *out) {
     }
     return parents;
 }
+
+/* prover/cuda_primitives.py:877-930 (k_row_prg / k_row_prg_indexed):
+ * out[r][k] = le64(BLAKE3(seed || row_le8 || k_le8)[0:8]) mod p; row = row_indices[r], or
+ * (uint32)(row_offset + r) when row_indices is NULL (the contiguous kernel counts rows in uint32). */
+void vo_row_prg(const uint8_t seed[32], const u64 *row_indices, u64 row_offset, size_t n_rows, size_t slack, u64 *out) {
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < (long)n_rows; ++r) {
+        uint8_t msg[48], dig[32];
+        memcpy(msg, seed, 32);
+        u64 row = row_indices ? row_indices[r] : (u64)(uint32_t)((uint32_t)row_offset + (uint32_t)r);
+        for (int b = 0; b < 8; ++b) msg[32 + b] = (uint8_t)(row >> (8 * b));
+        for (size_t k = 0; k < slack; ++k) {
+            for (int b = 0; b < 8; ++b) msg[40 + b] = (uint8_t)((u64)k >> (8 * b));
+            vo_blake3(msg, 48, dig);
+            u64 raw = 0;
+            for (int b = 7; b >= 0; --b) raw = (raw << 8) | dig[b];
+            out[(size_t)r * slack + k] = raw % GL_P;
+        }
+    }
+}

@@ -115,4 +115,18 @@ int emu_coset_lde(const u64 *in, long m, long w, long in_stride, int logK, int l
     delete of;
     return (int)passes.size();
 }
+// mode 0: values -> coeffs (+ out if not null); mode 1: coefficients -> out
+int emu_coset_lde_ex(const u64 *in, long m, long w, long in_stride, int logK, int logN, u64 shift,
+                     u64 *coeffs, long coeffs_stride, u64 *out, int in_is_coeffs) {
+    Owned *oi = make_owned(logK, 1), *of = make_owned(logK, 0);
+    std::vector<u64> pre = make_coset_pre(logK, logN, shift);
+    std::vector<u64> ws((size_t)lde_ws_elems(logK, logN, m));
+    std::vector<PassArgs> passes;
+    build_lde_passes(oi->T, of->T, pre.data(), logN, in, w, in_stride, out, (i64)1 << logN, ws.data(), m,
+                     passes, coeffs, coeffs_stride, in_is_coeffs != 0);
+    for (auto &A : passes) run_pass(A);
+    delete oi;
+    delete of;
+    return (int)passes.size();
+}
 }

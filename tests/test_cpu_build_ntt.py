@@ -31,6 +31,7 @@ def emu():
     L.emu_set_fast.argtypes = [c_int]
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
+    L.emu_coset_lde_ex.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p, c_long, u64p, c_int]
     return L
 
 
@@ -104,3 +105,43 @@ def test_lde_strided_input_and_other_shift(emu):
     got = np.zeros((6, 256), dtype=np.uint64)
     emu.emu_coset_lde(_p(big), 6, 40, 100, 6, 8, 11, _p(got))
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("logK,logN,m,w", [(5, 6, 4, 16), (9, 10, 3, 256), (12, 14, 2, 4096), (13, 15, 2, 5000),
+                                           (14, 16, 1, 8192), (4, 7, 5, 11)])
+def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w):
+    """The two halves of the pipeline: values -> (coefficients, codewords), coefficients only,
+    in place, and coefficients -> codewords."""
+    K, N = 1 << logK, 1 << logN
+    msgs = _rand((m, w), 300 + logK)
+    want = O.coset_lde_rows(msgs, K, N, 7)
+    padded = np.zeros((m, K), dtype=np.uint64)
+    padded[:, :w] = msgs
+    want_c = O.ntt_rows(padded, inverse=True)
+    for fast in (1, 0):
+        emu.emu_set_fast(fast)
+        pitch = K + 3
+        co = np.zeros((m, pitch), dtype=np.uint64)
+        got = np.zeros((m, N), dtype=np.uint64)
+        emu.emu_coset_lde_ex(_p(msgs), m, w, w, logK, logN, 7, _p(co), pitch, _p(got), 0)
+        assert np.array_equal(co[:, :K], want_c) and not co[:, K:].any()
+        assert np.array_equal(got, want)
+        co2 = np.zeros((m, K), dtype=np.uint64)
+        emu.emu_coset_lde_ex(_p(msgs), m, w, w, logK, logN, 7, _p(co2), K, None, 0)      # coefficients only
+        assert np.array_equal(co2, want_c)
+        inpl = padded.copy()
+        emu.emu_coset_lde_ex(_p(inpl), m, K, K, logK, logN, 7, _p(inpl), K, None, 0)       # in place
+        assert np.array_equal(inpl, want_c)
+        got2 = np.zeros((m, N), dtype=np.uint64)
+        emu.emu_coset_lde_ex(_p(want_c), m, K, K, logK, logN, 7, None, 0, _p(got2), 1)      # from coefficients
+        assert np.array_equal(got2, want)
+        # low-degree coefficients: only the first K/2 are given, the rest read as zero
+        half = np.ascontiguousarray(want_c[:, : K // 2])
+        full = np.zeros((m, K), dtype=np.uint64)
+        full[:, : K // 2] = half
+        got3 = np.zeros((m, N), dtype=np.uint64)
+        emu.emu_coset_lde_ex(_p(half), m, K // 2, K // 2, logK, logN, 7, None, 0, _p(got3), 1)
+        got4 = np.zeros((m, N), dtype=np.uint64)
+        emu.emu_coset_lde_ex(_p(full), m, K, K, logK, logN, 7, None, 0, _p(got4), 1)
+        assert np.array_equal(got3, got4)
+    emu.emu_set_fast(1)

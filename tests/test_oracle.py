@@ -332,3 +332,22 @@ def test_merkle_levels_and_paths_verify():
             if path:
                 bad = [(bytes(32), path[0][1])] + path[1:]
                 assert not merkle_verify(host[0][idx], bad, root)
+
+
+def test_row_prg_is_the_stated_hash():
+    """Definition spelled out with the independent host hash: first 8 digest bytes, little
+    endian, mod p, of seed || row_le8 || k_le8; rows count in uint32 in the contiguous form."""
+    from verinf_amd.prover.protocol import blake3_digest
+    seed = bytes(range(7, 39))
+    out = O.row_prg(seed, 5, 3, 4)
+    for r in range(3):
+        for k in range(4):
+            d = blake3_digest(seed + (5 + r).to_bytes(8, "little") + k.to_bytes(8, "little"))
+            assert int(out[r, k]) == int.from_bytes(d[:8], "little") % P
+    idx = np.array([0, 5, (1 << 40) + 3], dtype=np.uint64)
+    ind = O.row_prg(seed, 0, 0, 2, row_indices=idx)
+    assert np.array_equal(ind[1], out[0, :2])
+    d = blake3_digest(seed + ((1 << 40) + 3).to_bytes(8, "little") + (1).to_bytes(8, "little"))
+    assert int(ind[2, 1]) == int.from_bytes(d[:8], "little") % P
+    wrap = O.row_prg(seed, (1 << 32) - 1, 2, 1)          # row (2^32 - 1) + 1 wraps to 0
+    assert np.array_equal(wrap[1], O.row_prg(seed, 0, 1, 1)[0])

@@ -23,11 +23,11 @@ EXPORTS = [
     "vi_gl_matmul_workspace_bytes", "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
     "vi_ntt_workspace_bytes", "vi_ntt_batched",
     "vi_coset_lde_workspace_bytes", "vi_coset_lde_min_workspace_bytes", "vi_coset_lde_launches",
-    "vi_coset_lde",
+    "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend",
     "vi_kquant_to_field",
     "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval", "vi_sumcheck_prove",
     "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
-    "vi_merkle_level",
+    "vi_merkle_level", "vi_row_prg",
 ]
 
 COIN_FN = ctypes.CFUNCTYPE(c_int, c_int, POINTER(c_uint64), c_int, POINTER(c_uint64), c_void_p)
@@ -75,6 +75,8 @@ def lib():
     L.vi_coset_lde_launches.restype = i64
     L.vi_coset_lde_launches.argtypes = [i64, i64, i64, sz]
     L.vi_coset_lde.argtypes = [vp, i64, i64, i64, i64, i64, u64, vp, i64, vp, sz, vp]
+    L.vi_coset_lde_coeffs.argtypes = [vp, i64, i64, i64, i64, i64, u64, vp, i64, vp, i64, vp, sz, vp]
+    L.vi_coset_extend.argtypes = [vp, i64, i64, i64, i64, i64, u64, vp, i64, vp, sz, vp]
     L.vi_kquant_to_field.argtypes = [c_int, vp, i64, c_double, vp, vp]
     L.vi_sumcheck_workspace_bytes.restype = sz
     L.vi_sumcheck_workspace_bytes.argtypes = []
@@ -90,13 +92,14 @@ def lib():
     L.vi_hash_columns_update.argtypes = [vp, i64, i64, i64, i64, i64, vp, sz, vp]
     L.vi_hash_columns_finalize.argtypes = [i64, i64, vp, sz, vp, vp]
     L.vi_merkle_level.argtypes = [vp, i64, vp, vp]
+    L.vi_row_prg.argtypes = [vp, vp, i64, i64, i64, vp, i64, vp]
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
-                 "vi_ntt_batched", "vi_coset_lde", "vi_kquant_to_field", "vi_sumcheck_eval",
+                 "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_sumcheck_eval",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
-                 "vi_merkle_level"):
+                 "vi_merkle_level", "vi_row_prg"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

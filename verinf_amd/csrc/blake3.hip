@@ -150,6 +150,30 @@ __global__ __launch_bounds__(BLOCK) void k_merkle_level(const u32 *__restrict__ 
     for (int k = 0; k < 8; ++k) out[i * 8 + k] = cv[k];
 }
 
+// Zero-knowledge pad generator (prover/cuda_primitives.py:870-930, k_row_prg / k_row_prg_indexed):
+//   out[r][k] = (first 8 bytes of BLAKE3(seed[32] || row_le8 || k_le8), little-endian) mod p.
+// The 48-byte message is a single block, so a value costs one compression, of which only the
+// first two output words are used.  One thread per value, consecutive threads along k, so
+// that stores are coalesced; the reference gives a whole row to one thread.
+// row = row_indices[r] when row_indices is given, else the 32-bit sum row_offset + r (the
+// reference's contiguous variant computes the row number in uint32).
+__global__ __launch_bounds__(BLOCK) void k_row_prg(const u32 *__restrict__ seed, const u64 *__restrict__ row_indices, u32 row_offset,
+                                                   i64 n_rows, i64 slack, u64 *__restrict__ out, i64 out_stride) {
+    const i64 g = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    if (g >= n_rows * slack) return;
+    const i64 r = g / slack, k = g - r * slack;
+    const u64 row = row_indices ? row_indices[r] : (u64)(u32)(row_offset + (u32)r);
+    u32 m[16], cv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { m[i] = seed[i]; cv[i] = IV[i]; }
+    m[8] = (u32)row; m[9] = (u32)(row >> 32);
+    m[10] = (u32)k;  m[11] = (u32)((u64)k >> 32);
+    m[12] = m[13] = m[14] = m[15] = 0;
+    compress(cv, m, 0, 48, CHUNK_START | CHUNK_END | ROOT);
+    const u64 raw = ((u64)cv[1] << 32) | cv[0];
+    out[r * out_stride + k] = raw >= 0xFFFFFFFF00000001ull ? raw - 0xFFFFFFFF00000001ull : raw;
+}
+
 inline i64 chunks_of(i64 m) { return m <= 0 ? 1 : (m + ROWS_PER_CHUNK - 1) / ROWS_PER_CHUNK; }
 
 }  // namespace
@@ -228,6 +252,21 @@ int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *str
     hipLaunchKernelGGL(k_merkle_level, dim3((unsigned)((parents + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, (hipStream_t)stream,
                        (const u32 *)nodes, (i64)count, (u32 *)out);
     VI_LAUNCH_CHECK("k_merkle_level");
+    return VI_OK;
+}
+
+int vi_row_prg(const uint8_t *seed, const uint64_t *row_indices, int64_t row_offset, int64_t n_rows, int64_t slack,
+               uint64_t *out, int64_t out_stride, void *stream) {
+    if (n_rows < 0 || slack < 0 || out_stride < slack) return vi::fail(VI_EINVAL, "vi_row_prg: bad shape n_rows=%lld slack=%lld out_stride=%lld", (long long)n_rows, (long long)slack, (long long)out_stride);
+    if (n_rows == 0 || slack == 0) return VI_OK;
+    if (!seed || !out) return vi::fail(VI_EINVAL, "vi_row_prg: null pointer");
+    if ((uintptr_t)seed & 3) return vi::fail(VI_EINVAL, "vi_row_prg: seed must be 4-byte aligned");
+    const i64 total = n_rows * slack;
+    const i64 blocks = (total + BLOCK - 1) / BLOCK;
+    if (blocks > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "vi_row_prg: %lld values exceed one launch", (long long)total);
+    hipLaunchKernelGGL(k_row_prg, dim3((unsigned)blocks), dim3(BLOCK), 0, (hipStream_t)stream, (const u32 *)seed, row_indices,
+                       (u32)row_offset, (i64)n_rows, (i64)slack, out, (i64)out_stride);
+    VI_LAUNCH_CHECK("k_row_prg");
     return VI_OK;
 }
 

@@ -252,23 +252,26 @@ int64_t vi_coset_lde_launches(int64_t m, int64_t K, int64_t N, size_t ws_bytes) 
     return ((m + chunk - 1) / chunk) * 2 * split_digits(vi::ilog2(K)).p;   // balancing keeps the chunk count
 }
 
-int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
-                 int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, void *ws,
-                 size_t ws_bytes, void *stream) {
+namespace {
+
+// values (or coefficients) -> optional coefficients -> optional codewords, chunked over rows
+int coset_lde_impl(const char *who, const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
+                   int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, uint64_t *coeffs,
+                   int64_t coeffs_stride, bool in_is_coeffs, void *ws, size_t ws_bytes, void *stream) {
     if (!vi::is_pow2(K) || !vi::is_pow2(N) || K < 2 || N < K || N > ((int64_t)1 << 32))
-        return vi::fail(VI_EINVAL, "vi_coset_lde: need powers of two with 2 <= K <= N <= 2^32, got K=%lld N=%lld",
+        return vi::fail(VI_EINVAL, "%s: need powers of two with 2 <= K <= N <= 2^32, got K=%lld N=%lld", who,
                         (long long)K, (long long)N);
-    if (m < 0 || width < 0 || width > K || in_stride < width || out_stride < N)
-        return vi::fail(VI_EINVAL, "vi_coset_lde: bad shape m=%lld width=%lld in_stride=%lld out_stride=%lld",
-                        (long long)m, (long long)width, (long long)in_stride, (long long)out_stride);
-    if (shift == 0 || shift >= gl::P) return vi::fail(VI_EINVAL, "vi_coset_lde: shift must be in [1, p)");
+    if (m < 0 || width < 0 || width > K || in_stride < width || (out && out_stride < N) || (coeffs && coeffs_stride < K))
+        return vi::fail(VI_EINVAL, "%s: bad shape m=%lld width=%lld in_stride=%lld out_stride=%lld coeffs_stride=%lld", who,
+                        (long long)m, (long long)width, (long long)in_stride, (long long)out_stride, (long long)coeffs_stride);
+    if (shift == 0 || shift >= gl::P) return vi::fail(VI_EINVAL, "%s: shift must be in [1, p)", who);
     if (m == 0) return VI_OK;
-    if (!in || !out) return vi::fail(VI_EINVAL, "vi_coset_lde: null pointer");
+    if (!in || (!out && !coeffs)) return vi::fail(VI_EINVAL, "%s: null pointer", who);
     const int logK = vi::ilog2(K), logN = vi::ilog2(N);
     size_t one = (size_t)lde_ws_elems(logK, logN, 1) * sizeof(u64);
     i64 chunk = (i64)(ws_bytes / one);
     if (!ws || chunk < 1)
-        return vi::fail(VI_ENOMEM, "vi_coset_lde: workspace of %zu bytes is below the one-row minimum %zu", ws_bytes, one);
+        return vi::fail(VI_ENOMEM, "%s: workspace of %zu bytes is below the one-row minimum %zu", who, ws_bytes, one);
     if (chunk > m) chunk = m;
     if (chunk > max_rows_per_launch(logN)) chunk = max_rows_per_launch(logN);
     chunk = (m + ((m + chunk - 1) / chunk) - 1) / ((m + chunk - 1) / chunk);   // same chunk count, even sizes
@@ -281,12 +284,40 @@ int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride
     for (i64 lo = 0; lo < m; lo += chunk) {
         i64 cnt = (m - lo < chunk) ? (m - lo) : chunk;
         std::vector<PassArgs> passes;
-        build_lde_passes(*Ti, *Tf, pre, logN, in + lo * in_stride, width, in_stride, out + lo * out_stride,
-                         out_stride, (u64 *)ws, cnt, passes);
+        build_lde_passes(*Ti, *Tf, pre, logN, in + lo * in_stride, width, in_stride, out ? out + lo * out_stride : nullptr,
+                         out_stride, (u64 *)ws, cnt, passes, coeffs ? coeffs + lo * coeffs_stride : nullptr, coeffs_stride,
+                         in_is_coeffs);
         rc = launch_passes(passes, (hipStream_t)stream);
         if (rc) return rc;
     }
     return VI_OK;
+}
+
+}  // namespace
+
+int vi_coset_lde(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
+                 int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, void *ws,
+                 size_t ws_bytes, void *stream) {
+    if (m > 0 && !out) return vi::fail(VI_EINVAL, "vi_coset_lde: null pointer");
+    return coset_lde_impl("vi_coset_lde", in, m, width, in_stride, K, N, shift, out, out_stride, nullptr, 0, false, ws,
+                          ws_bytes, stream);
+}
+
+int vi_coset_lde_coeffs(const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K, int64_t N,
+                        uint64_t shift, uint64_t *coeffs, int64_t coeffs_stride, uint64_t *out, int64_t out_stride,
+                        void *ws, size_t ws_bytes, void *stream) {
+    if (m > 0 && !coeffs) return vi::fail(VI_EINVAL, "vi_coset_lde_coeffs: null coeffs");
+    if (coeffs == in && coeffs_stride != in_stride)
+        return vi::fail(VI_EINVAL, "vi_coset_lde_coeffs: in-place use needs equal strides");
+    return coset_lde_impl("vi_coset_lde_coeffs", in, m, width, in_stride, K, N, shift, out, out_stride, coeffs,
+                          coeffs_stride, false, ws, ws_bytes, stream);
+}
+
+int vi_coset_extend(const uint64_t *coeffs, int64_t m, int64_t width, int64_t coeffs_stride, int64_t K, int64_t N,
+                    uint64_t shift, uint64_t *out, int64_t out_stride, void *ws, size_t ws_bytes, void *stream) {
+    if (m > 0 && !out) return vi::fail(VI_EINVAL, "vi_coset_extend: null pointer");
+    return coset_lde_impl("vi_coset_extend", coeffs, m, width, coeffs_stride, K, N, shift, out, out_stride, nullptr, 0,
+                          true, ws, ws_bytes, stream);
 }
 
 }  // extern "C"

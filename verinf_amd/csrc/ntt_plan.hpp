@@ -167,23 +167,30 @@ inline i64 lde_ws_elems(int logK, int logN, i64 m) {
     return split_digits(logK).p == 1 ? m * K : m * K * (1 + rho);
 }
 
+// in -> [inverse passes] -> coefficients -> [forward passes over rho cosets] -> out.
+// The coefficients live in the workspace unless the caller wants them (coeffs != nullptr: the
+// last inverse pass writes them there, row pitch coeffs_stride).  in_is_coeffs skips the
+// inverse passes: `in` already holds coefficients (width w, the rest zero).
 inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre, int logN,
                              const u64 *in, i64 w, i64 in_stride, u64 *out, i64 out_stride,
-                             u64 *ws, i64 m, std::vector<PassArgs> &passes) {
+                             u64 *ws, i64 m, std::vector<PassArgs> &passes,
+                             u64 *coeffs = nullptr, i64 coeffs_stride = 0, bool in_is_coeffs = false) {
     const int logK = Ti.logn, log_rho = logN - logK, p = Ti.sp.p;
     const i64 K = (i64)1 << logK;
-    u64 *C = ws, *S = ws + m * K;
+    u64 *C = coeffs ? coeffs : ws, *S = ws + m * K;
+    const i64 c_stride = coeffs ? coeffs_stride : K;
     // inverse: in -> S (plane 0) -> C
-    for (int q = 0; q < p; ++q) {
+    for (int q = 0; q < p && !in_is_coeffs; ++q) {
         PassArgs A = base_pass(Ti, q, m);
         A.src = (q == 0) ? in : S;
         A.canon_src = (q == 0);
         A.src_row_stride = (q == 0) ? in_stride : K;
         A.src_width = (q == 0) ? w : K;
         A.dst = A.is_final ? C : S;
-        A.dst_row_stride = K;
+        A.dst_row_stride = A.is_final ? c_stride : K;
         passes.push_back(A);
     }
+    if (!out) return;
     // forward over rho cosets
     for (int q = 0; q < p; ++q) {
         bool first = (q == 0), last = (q == p - 1);
@@ -191,8 +198,9 @@ inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre,
         A.log_rho = (first || last) ? log_rho : 0;     // middle passes see rho*m plain rows
         A.loop_cosets = first && !last;
         A.pre = first ? pre : nullptr;
-        A.src = first ? C : S;
-        A.src_row_stride = K;
+        A.src = first ? (in_is_coeffs ? in : C) : S;
+        A.src_row_stride = first ? (in_is_coeffs ? in_stride : c_stride) : K;
+        if (first && in_is_coeffs) { A.src_width = w; A.canon_src = 1; }
         A.src_coset_stride = first ? 0 : m * K;
         A.dst = last ? out : S;
         A.dst_row_stride = last ? out_stride : K;

@@ -170,18 +170,13 @@ def ntt_inverse_batched(rows):
 
 
 # ---- Reed-Solomon ------------------------------------------------------------------
-def coset_lde(messages, k_deg, n_lig, shift=GLOBAL_G, out=None):
-    """(m, w <= K) values at the K-th roots of unity -> (m, N) codewords on the coset
-    shift * <w_N>, in one fused pipeline: inverse NTT_K, coefficient twist, zero
-    extension and forward transform (the recipe of layergkr/gpu.py:141-203 and
-    prover/core.py:721-743, 798).  Rows may be a strided view with unit column
-    stride, so `buf[:, :ELL]` needs no copy."""
+def _lde_args(messages, k_deg, n_lig, what="messages"):
     if not isinstance(messages, torch.Tensor) or not messages.is_cuda:
-        raise RuntimeError("messages must be CUDA")
+        raise RuntimeError(f"{what} must be CUDA")
     if messages.dtype != torch.uint64:
-        raise RuntimeError("messages dtype must be uint64")
+        raise RuntimeError(f"{what} dtype must be uint64")
     if messages.dim() != 2:
-        raise RuntimeError("coset_lde expects (m, width)")
+        raise RuntimeError(f"expected (m, width) {what}")
     k_deg, n_lig = int(k_deg), int(n_lig)
     m, w = int(messages.shape[0]), int(messages.shape[1])
     if not (_is_pow2(k_deg) and k_deg >= 2):
@@ -189,18 +184,32 @@ def coset_lde(messages, k_deg, n_lig, shift=GLOBAL_G, out=None):
     if not (_is_pow2(n_lig) and n_lig >= k_deg):
         raise RuntimeError("n_lig must be a power of 2 >= k_deg")
     if w > k_deg:
-        raise RuntimeError("messages' second dim must be <= k_deg")
+        raise RuntimeError(f"{what}' second dim must be <= k_deg")
     if m and w and messages.stride(1) != 1:
-        raise RuntimeError("messages must have unit column stride")
+        raise RuntimeError(f"{what} must have unit column stride")
     in_stride = int(messages.stride(0)) if (m > 1 and w) else max(w, 1)
     if in_stride < w:
-        raise RuntimeError("messages rows overlap")
+        raise RuntimeError(f"{what} rows overlap")
+    return k_deg, n_lig, m, w, in_stride
+
+
+def _lde_out(out, m, n_lig, device):
     if out is None:
-        out = torch.empty((m, n_lig), dtype=torch.uint64, device=messages.device)
-    else:
-        _check_u64(out, "out")
-        if tuple(out.shape) != (m, n_lig):
-            raise RuntimeError("out must be (m, n_lig)")
+        return torch.empty((m, n_lig), dtype=torch.uint64, device=device)
+    _check_u64(out, "out")
+    if tuple(out.shape) != (m, n_lig):
+        raise RuntimeError("out must be (m, n_lig)")
+    return out
+
+
+def coset_lde(messages, k_deg, n_lig, shift=GLOBAL_G, out=None):
+    """(m, w <= K) values at the K-th roots of unity -> (m, N) codewords on the coset
+    shift * <w_N>, in one fused pipeline: inverse NTT_K, coefficient twist, zero
+    extension and forward transform (the recipe of layergkr/gpu.py:141-203 and
+    prover/core.py:721-743, 798).  Rows may be a strided view with unit column
+    stride, so `buf[:, :ELL]` needs no copy."""
+    k_deg, n_lig, m, w, in_stride = _lde_args(messages, k_deg, n_lig)
+    out = _lde_out(out, m, n_lig, messages.device)
     if m == 0:
         return out
     if w == 0:                      # an empty message is the zero polynomial
@@ -210,6 +219,48 @@ def coset_lde(messages, k_deg, n_lig, shift=GLOBAL_G, out=None):
         ws = _lib.workspace(L.vi_coset_lde_workspace_bytes(m, k_deg, n_lig), messages.device, "lde")
         _lib.check(L.vi_coset_lde(messages.data_ptr(), m, w, in_stride, k_deg, n_lig, int(shift) % P,
                                   out.data_ptr(), n_lig, ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    return out
+
+
+def coset_lde_with_coeffs(messages, k_deg, n_lig, shift=GLOBAL_G, need_codewords=True, out=None):
+    """As coset_lde, but also returns the row polynomials the pipeline passes through:
+    (coeffs (m, K), codewords (m, N) or None).  One call stands for
+    `row_polys = padded.clone(); ntt_inverse_batched(row_polys); _coset_encode_codewords(row_polys)`
+    (prover/core.py:795-802); need_codewords=False stops after the coefficients."""
+    k_deg, n_lig, m, w, in_stride = _lde_args(messages, k_deg, n_lig)
+    coeffs = torch.empty((m, k_deg), dtype=torch.uint64, device=messages.device)
+    out = _lde_out(out, m, n_lig, messages.device) if need_codewords else None
+    if m == 0:
+        return coeffs, out
+    if w == 0:
+        coeffs.view(torch.int64).zero_()
+        if out is not None:
+            out.view(torch.int64).zero_()
+        return coeffs, out
+    L = _lib.lib()
+    with torch.cuda.device(messages.device):
+        ws = _lib.workspace(L.vi_coset_lde_workspace_bytes(m, k_deg, n_lig), messages.device, "lde")
+        _lib.check(L.vi_coset_lde_coeffs(messages.data_ptr(), m, w, in_stride, k_deg, n_lig, int(shift) % P,
+                                         coeffs.data_ptr(), k_deg, out.data_ptr() if out is not None else None, n_lig,
+                                         ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    return coeffs, out
+
+
+def coset_extend(coeffs, k_deg, n_lig, shift=GLOBAL_G, out=None):
+    """(m, w <= K) polynomial coefficients -> (m, N) evaluations on shift * <w_N>: the
+    twist, zero extension and forward transform of prover/core.py:721-743 (and its
+    cosets formulation :702-718) without the `(m, N)` staging buffer."""
+    k_deg, n_lig, m, w, in_stride = _lde_args(coeffs, k_deg, n_lig, "coeffs")
+    out = _lde_out(out, m, n_lig, coeffs.device)
+    if m == 0:
+        return out
+    if w == 0:
+        return out.view(torch.int64).zero_().view(torch.uint64)
+    L = _lib.lib()
+    with torch.cuda.device(coeffs.device):
+        ws = _lib.workspace(L.vi_coset_lde_workspace_bytes(m, k_deg, n_lig), coeffs.device, "lde")
+        _lib.check(L.vi_coset_extend(coeffs.data_ptr(), m, w, in_stride, k_deg, n_lig, int(shift) % P,
+                                     out.data_ptr(), n_lig, ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
     return out
 
 
@@ -441,6 +492,60 @@ class MerkleColumnAccumulator:
         _lib.check(L.vi_hash_columns_finalize(self.n_cols, self.n_chunks_total, self._states.data_ptr(),
                                               self._states.numel(), out.data_ptr(), _lib.stream_ptr()))
         return out
+
+
+# ---- ZK pad generator (prover/cuda_primitives.py:1262-1294) ----
+
+def _check_seed(master_seed):
+    assert isinstance(master_seed, torch.Tensor)
+    if master_seed.dtype != torch.uint8:
+        raise RuntimeError("master_seed must be uint8")
+    if master_seed.numel() != 32:
+        raise RuntimeError("master_seed must be 32 bytes")
+    if not master_seed.is_cuda:
+        raise RuntimeError("master_seed must be on CUDA")
+    if not master_seed.is_contiguous():
+        raise RuntimeError("master_seed must be contiguous")
+
+
+def _row_prg(master_seed, row_indices, row_offset, n_rows, slack, out):
+    if n_rows and slack:
+        _lib.check(_lib.lib().vi_row_prg(master_seed.data_ptr(), row_indices.data_ptr() if row_indices is not None else None,
+                                         int(row_offset), n_rows, slack, out.data_ptr(),
+                                         int(out.stride(0)) if n_rows > 1 else max(slack, int(out.stride(0))),
+                                         _lib.stream_ptr()))
+    return out
+
+
+def row_prg(master_seed, row_offset, n_rows, slack_per_row, out=None):
+    """(n_rows, slack_per_row) uint64 with
+    out[r, k] = BLAKE3(master_seed || (row_offset + r)_le8 || k_le8)[0:8] mod P
+    (prover/cuda_primitives.py:1262-1286).  `out` may be a column slice of a wider
+    matrix (unit column stride), e.g. `padded[:, ELL:]`, which is then filled in place."""
+    _check_seed(master_seed)
+    n_rows, slack = int(n_rows), int(slack_per_row)
+    if n_rows < 0 or slack < 0:
+        raise RuntimeError("n_rows and slack_per_row must be >= 0")
+    if out is None:
+        out = torch.empty((n_rows, slack), dtype=torch.uint64, device=master_seed.device)
+    else:
+        if out.dtype != torch.uint64 or not out.is_cuda or tuple(out.shape) != (n_rows, slack):
+            raise RuntimeError("out must be a (n_rows, slack_per_row) CUDA uint64 tensor")
+        if n_rows and slack and (out.stride(1) != 1 or (n_rows > 1 and out.stride(0) < slack)):
+            raise RuntimeError("out must have unit column stride and non-overlapping rows")
+    return _row_prg(master_seed, None, row_offset, n_rows, slack, out)
+
+
+def row_prg_indexed(master_seed, row_indices, slack_per_row):
+    """row_prg for a list of absolute row indices (cuda uint64 tensor), one launch
+    (prover/cuda_primitives.py:1289-1294)."""
+    _check_seed(master_seed)
+    if (not isinstance(row_indices, torch.Tensor) or row_indices.dtype != torch.uint64 or not row_indices.is_cuda
+            or not row_indices.is_contiguous()):
+        raise RuntimeError("row_indices must be a contiguous CUDA uint64 tensor")
+    n_rows, slack = int(row_indices.numel()), int(slack_per_row)
+    out = torch.empty((n_rows, slack), dtype=torch.uint64, device=master_seed.device)
+    return _row_prg(master_seed, row_indices, 0, n_rows, slack, out)
 
 
 def merkle_one_level(nodes):
