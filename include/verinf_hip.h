@@ -221,6 +221,24 @@ int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *str
 int vi_row_prg(const uint8_t *seed, const uint64_t *row_indices, int64_t row_offset, int64_t n_rows, int64_t slack,
                uint64_t *out, int64_t out_stride, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Multilinear helpers around the sumchecks.  A point z is a HOST array of n_vars <= 32 words (reduced
+ * mod p by the callee).
+ *
+ * vi_eq_vector replaces eq_vector (layergkr/logup.py:61-69) for device consumers:
+ *   out[i] = prod_j (bit(i, pos_j) ? z_j : 1 - z_j), 2^n_vars words,
+ * with pos_j = j when msb_first == 0 -- z_0 on the least significant index bit, which is what the
+ * reference's doubling loop produces -- and pos_j = n_vars - 1 - j when msb_first != 0, the variable
+ * order of mle_eval and of the sumcheck folds.
+ * vi_mle_eval replaces mle_eval (layergkr/sumcheck.py:40-48) for device tables: out[t] = the
+ * multilinear extension of row t of `tables` (n_tables rows of 2^n_vars words, pitch row_stride)
+ * at z (z_0 on the most significant bit), one pass per table; out is a device array of n_tables words.
+ * Workspace: vi_mle_eval_workspace_bytes(n_tables) = 8 KiB per table. */
+int vi_eq_vector(const uint64_t *z, int n_vars, int msb_first, uint64_t *out, void *stream);
+size_t vi_mle_eval_workspace_bytes(int64_t n_tables);
+int vi_mle_eval(const uint64_t *tables, int64_t n_tables, int64_t row_stride, const uint64_t *z, int n_vars,
+                uint64_t *out, void *ws, size_t ws_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

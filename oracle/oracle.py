@@ -71,6 +71,7 @@ def lib():
         L.vo_merkle_level.restype = c_size_t
         L.vo_merkle_level.argtypes = [u8p, c_size_t, u8p]
         L.vo_row_prg.argtypes = [u8p, u64p, c_uint64, c_size_t, c_size_t, u64p]
+        L.vo_eq_vector.argtypes = [u64p, c_int, u64p]
         _lib = L
     return _lib
 
@@ -221,6 +222,22 @@ def row_prg(seed: bytes, row_offset: int, n_rows: int, slack: int, row_indices=N
     if n_rows and slack:
         lib().vo_row_prg(_p8(sd), _p64(idx) if idx is not None else None, int(row_offset) & ((1 << 64) - 1), n_rows, slack, _p64(out))
     return out
+
+
+def eq_vector(z) -> np.ndarray:
+    """layergkr/logup.py:61-69: 2^n words, z[0] on the least significant index bit."""
+    zz = np.array([int(v) % P for v in z], dtype=np.uint64)
+    out = np.empty(1 << len(zz), dtype=np.uint64)
+    lib().vo_eq_vector(_p64(zz) if len(zz) else None, len(zz), _p64(out))
+    return out
+
+
+def mle_eval(values: np.ndarray, point) -> int:
+    """layergkr/sumcheck.py:40-48 by repeated vo_fold, point[0] on the most significant bit."""
+    cur = np.ascontiguousarray(values, dtype=np.uint64) % np.uint64(P)
+    for r in point:
+        cur = fold(cur, int(r) % P)
+    return int(cur[0])
 
 
 def merkle_levels(leaves: np.ndarray):

@@ -553,3 +553,20 @@ void vo_row_prg(const uint8_t seed[32], const u64 *row_indices, u64 row_offset, 
         }
     }
 }
+
+/* layergkr/logup.py:61-69 -- eq(z, .) over the hypercube by doubling, most-significant variable
+ * first: out <- [v (1 - z_i)] ++ [v z_i].  out holds 2^n words. */
+void vo_eq_vector(const u64 *z, int n, u64 *out) {
+    size_t len = 1;
+    out[0] = 1;
+    for (int i = 0; i < n; ++i) {
+        u64 zi = z[i] % GL_P, om = vo_sub(1, zi);
+        /* the old entries become the low half, their z-multiples the high half */
+        for (size_t k = 0; k < len; ++k) {
+            u64 v = out[k];
+            out[len + k] = vo_mul(v, zi);
+            out[k] = vo_mul(v, om);
+        }
+        len *= 2;
+    }
+}

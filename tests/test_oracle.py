@@ -351,3 +351,39 @@ def test_row_prg_is_the_stated_hash():
     assert int(ind[2, 1]) == int.from_bytes(d[:8], "little") % P
     wrap = O.row_prg(seed, (1 << 32) - 1, 2, 1)          # row (2^32 - 1) + 1 wraps to 0
     assert np.array_equal(wrap[1], O.row_prg(seed, 0, 1, 1)[0])
+
+
+# ---- multilinear helpers ---------------------------------------------------------------
+def test_eq_vector_product_formula_and_invariants():
+    rng = random.Random(21)
+    for n in [0, 1, 2, 3, 5, 9]:
+        z = [rng.randrange(P) for _ in range(n)]
+        eq = O.eq_vector(z)
+        assert eq.shape == (1 << n,)
+        # closed form, z[j] on index bit j (what the reference's doubling loop yields)
+        for i in rng.sample(range(1 << n), min(1 << n, 12)):
+            want = 1
+            for j in range(n):
+                want = want * (z[j] if (i >> j) & 1 else (1 - z[j])) % P
+            assert int(eq[i]) == want
+        assert sum(int(v) for v in eq) % P == 1          # a partition of unity
+    # at a Boolean point eq is the indicator of that index
+    bits = [1, 0, 1, 1]
+    eq = O.eq_vector(bits)
+    idx = sum(b << j for j, b in enumerate(bits))
+    assert [int(v) for v in eq] == [1 if i == idx else 0 for i in range(16)]
+
+
+def test_mle_eval_matches_definition():
+    rng = random.Random(22)
+    for n in [1, 3, 6]:
+        f = np.array([rng.randrange(P) for _ in range(1 << n)], dtype=np.uint64)
+        pt = [rng.randrange(P) for _ in range(n)]
+        got = O.mle_eval(f, pt)
+        assert got == O.py_mle_eval([int(v) for v in f], pt)
+        # = <f, eq> with the point reversed (mle_eval counts variables from the top bit)
+        eq = O.eq_vector(pt[::-1])
+        assert got == sum(int(a) * int(b) for a, b in zip(f, eq)) % P
+        # Boolean points read the table
+        i = rng.randrange(1 << n)
+        assert O.mle_eval(f, [(i >> (n - 1 - j)) & 1 for j in range(n)]) == int(f[i])

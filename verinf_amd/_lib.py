@@ -28,6 +28,7 @@ EXPORTS = [
     "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval", "vi_sumcheck_prove",
     "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
     "vi_merkle_level", "vi_row_prg",
+    "vi_eq_vector", "vi_mle_eval_workspace_bytes", "vi_mle_eval",
 ]
 
 COIN_FN = ctypes.CFUNCTYPE(c_int, c_int, POINTER(c_uint64), c_int, POINTER(c_uint64), c_void_p)
@@ -93,13 +94,17 @@ def lib():
     L.vi_hash_columns_finalize.argtypes = [i64, i64, vp, sz, vp, vp]
     L.vi_merkle_level.argtypes = [vp, i64, vp, vp]
     L.vi_row_prg.argtypes = [vp, vp, i64, i64, i64, vp, i64, vp]
+    L.vi_eq_vector.argtypes = [POINTER(u64), c_int, c_int, vp, vp]
+    L.vi_mle_eval_workspace_bytes.restype = sz
+    L.vi_mle_eval_workspace_bytes.argtypes = [i64]
+    L.vi_mle_eval.argtypes = [vp, i64, i64, POINTER(u64), c_int, vp, vp, sz, vp]
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
                  "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_sumcheck_eval",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
-                 "vi_merkle_level", "vi_row_prg"):
+                 "vi_merkle_level", "vi_row_prg", "vi_eq_vector", "vi_mle_eval"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

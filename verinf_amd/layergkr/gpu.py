@@ -182,6 +182,47 @@ def column(mat, col: int):
     return [int(v) for v in mat.view(torch.int64)[:, col].contiguous().view(torch.uint64).cpu().tolist()]
 
 
+# ---- multilinear helpers ---------------------------------------------------------------
+def _point(z):
+    arr = (ctypes.c_uint64 * max(len(z), 1))(*[int(v) % P for v in z])
+    return arr
+
+
+def eq_vector_t(z: Sequence[int], msb_first: bool = False):
+    """eq(z, .) over the hypercube as a device tensor of 2^len(z) field elements, built on
+    the device.  Default order is that of the reference's eq_vector (layergkr/logup.py:61-69,
+    z[0] on the least significant index bit), so the tensor can stand in for its list as a
+    sumcheck factor; msb_first=True gives the variable order of mle_eval / fold_t."""
+    _require_gpu()
+    n = len(z)
+    if n > 32:
+        raise RuntimeError("eq_vector_t: at most 32 variables")
+    out = torch.empty(1 << n, dtype=torch.uint64, device="cuda")
+    _lib.check(_lib.lib().vi_eq_vector(_point(z), n, 1 if msb_first else 0, out.data_ptr(), _lib.stream_ptr()))
+    return out
+
+
+def mle_eval_t(tables, point: Sequence[int]):
+    """Multilinear extension of a device table (or of every row of a (k, 2^n) matrix) at
+    `point`, point[0] on the most significant index bit as in layergkr/sumcheck.py:40-48.
+    One streaming pass per table; returns an int (1-D input) or a list of ints."""
+    _require_gpu()
+    cp._check_u64(tables, "tables")
+    n = len(point)
+    one = tables.dim() == 1
+    mat = tables.view(1, -1) if one else tables
+    if mat.dim() != 2 or int(mat.shape[1]) != (1 << n):
+        raise RuntimeError(f"mle_eval_t: tables of length {tuple(tables.shape)} do not match {n} variables")
+    k = int(mat.shape[0])
+    out = torch.empty(max(k, 1), dtype=torch.uint64, device=tables.device)
+    L = _lib.lib()
+    ws = _lib.workspace(L.vi_mle_eval_workspace_bytes(k), tables.device, "mle")
+    _lib.check(L.vi_mle_eval(mat.data_ptr(), k, 1 << n, _point(point), n, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                             _lib.stream_ptr()))
+    vals = [int(v) for v in out[:k].cpu().tolist()]
+    return vals[0] if one else vals
+
+
 # ---- sumcheck ------------------------------------------------------------------------
 def gl_sum(t):
     """Field sum of a uint64 device tensor -> 1-element device tensor."""
