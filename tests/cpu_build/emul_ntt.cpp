@@ -91,6 +91,7 @@ u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
 u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
 u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }
 u64 emu_mul_pow2(u64 x, unsigned s) { return gl::mul_pow2(x, s); }
+u64 emu_inv(u64 x) { return gl::inv(x); }
 
 int emu_ntt_batched(u64 *buf, long m, int logn, int inverse) {
     Owned *o = make_owned(logn, inverse);

@@ -27,6 +27,8 @@ def emu():
         f.restype = c_uint64
         f.argtypes = [c_uint64, c_uint64]
     L.emu_mul_pow2.restype = c_uint64
+    L.emu_inv.restype = c_uint64
+    L.emu_inv.argtypes = [c_uint64]
     L.emu_mul_pow2.argtypes = [c_uint64, c_uint]
     L.emu_set_fast.argtypes = [c_int]
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
@@ -59,6 +61,17 @@ def test_device_field_functions(emu):
     for a in edge[:9] + [r.randrange(P) for _ in range(100)]:
         for s in range(96):
             assert emu.emu_mul_pow2(a, s) == a * (1 << s) % P, (a, s)
+
+
+def test_device_inverse_chain(emu):
+    """The fixed addition chain for x^(p-2): x * inv(x) = 1, inv(0) = 0, non-canonical words
+    invert as their residues."""
+    rng = random.Random(4)
+    for x in [1, 2, P - 1, P - 2, 1 << 32, (1 << 32) - 1, 7] + [rng.randrange(1, P) for _ in range(200)]:
+        assert emu.emu_inv(x) == pow(x, P - 2, P), x
+    assert emu.emu_inv(0) == 0
+    assert emu.emu_inv(P) == 0
+    assert emu.emu_inv(P + 5) == pow(5, P - 2, P)
 
 
 @pytest.mark.parametrize("logn,m", [(1, 3), (2, 5), (4, 300), (5, 9), (6, 7), (7, 70), (8, 33), (10, 5), (12, 3),

@@ -114,3 +114,24 @@ def test_gl_sum_and_fold_t():
     got = gpu.fold_t(to_dev(f), torch.tensor([r], dtype=torch.uint64).cuda())
     assert np.array_equal(to_np(got), O.fold(f, r))
     assert np.array_equal(to_np(gpu.fold_t(to_dev(f), r)), O.fold(f, r))
+
+
+@pytest.mark.parametrize("n", [1, 2, 7, 8, 9, 63, 64, 65, 1000, 4099, 1 << 16, (1 << 20) + 3])
+def test_inverse_of_arrays_with_zeros_and_ragged_lengths(cp, n):
+    """The batched inverse shares one inversion among eight elements: every length class
+    (fewer than eight, not a multiple of eight), zeros anywhere (0 -> 0 as the Fermat power
+    gives) and non-canonical words."""
+    a = rand_field((n,), 40 + n)
+    rng = np.random.default_rng(n)
+    a[rng.integers(0, n, max(1, n // 50))] = 0
+    if n > 4:
+        a[3] = np.uint64(P)                          # = 0 mod p
+        a[4] = np.uint64(P + 6)                      # = 6 mod p
+    got = to_np(cp.gl_inv_batched(to_dev(a)))
+    idx = list(range(min(n, 40))) + [int(i) for i in rng.integers(0, n, 60)] + [n - 1]
+    for i in idx:
+        x = int(a[i]) % P
+        assert int(got[i]) == (pow(x, P - 2, P) if x else 0), i
+    red = to_dev(a % np.uint64(P))
+    prod = to_np(cp.gl_mul(red, to_dev(got)))
+    assert np.array_equal(prod, (to_np(red) != 0).astype(np.uint64))

@@ -54,6 +54,41 @@ __global__ __launch_bounds__(BLOCK) void k_unop(int op, const u64 *a, u64 arg, u
     }
 }
 
+// Inverses of a whole array by Montgomery's trick in registers (the batching of
+// layergkr/field.py:84-101 at the scale of one thread): a thread takes INV_E elements, one
+// from each of INV_E equal slabs of the array so that a wavefront's accesses stay contiguous,
+// multiplies them up, inverts the product once (74 multiplications) and peels the single
+// inverses off with two multiplications each.  Zeros are taken out of the product and map
+// to zero, so every output equals the Fermat power a^(p-2) of the reference kernel
+// (prover/cuda_primitives.py:289-303).
+constexpr int INV_E = 8;
+
+__global__ __launch_bounds__(BLOCK) void k_inv_batched(const u64 *a, u64 *out, i64 n, i64 groups) {
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 g = (i64)blockIdx.x * BLOCK + threadIdx.x; g < groups; g += stride) {
+        u64 x[INV_E], pre[INV_E];
+        unsigned zero = 0;
+#pragma unroll
+        for (int j = 0; j < INV_E; ++j) {
+            const i64 i = (i64)j * groups + g;
+            u64 v = i < n ? gl::canon(a[i]) : 1;
+            if (v == 0) { zero |= 1u << j; v = 1; }
+            x[j] = v;
+        }
+        pre[0] = x[0];
+#pragma unroll
+        for (int j = 1; j < INV_E; ++j) pre[j] = gl::mul(pre[j - 1], x[j]);
+        u64 acc = gl::inv(pre[INV_E - 1]);
+#pragma unroll
+        for (int j = INV_E - 1; j >= 0; --j) {
+            const u64 r = j ? gl::mul(acc, pre[j - 1]) : acc;
+            if (j) acc = gl::mul(acc, x[j]);
+            const i64 i = (i64)j * groups + g;
+            if (i < n) out[i] = (zero >> j) & 1 ? 0 : r;
+        }
+    }
+}
+
 __global__ __launch_bounds__(BLOCK) void k_axpy(u64 *y, u64 alpha, const u64 *x, i64 n) {
     i64 stride = (i64)gridDim.x * BLOCK;
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) y[i] = gl::add(y[i], gl::mul(alpha, x[i]));
@@ -151,7 +186,12 @@ int vi_gl_unop(int op, const uint64_t *a, uint64_t arg, uint64_t *out, int64_t n
     if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_unop: n = %lld", (long long)n);
     if (n == 0) return VI_OK;
     if (!a || !out) return vi::fail(VI_EINVAL, "vi_gl_unop: null pointer");
-    if (op == 2) { op = 1; arg = gl::P - 2; }
+    if (op == 2) {
+        const i64 groups = (n + INV_E - 1) / INV_E;
+        hipLaunchKernelGGL(k_inv_batched, dim3(grid_for(groups)), dim3(BLOCK), 0, (hipStream_t)stream, a, out, (i64)n, groups);
+        VI_LAUNCH_CHECK("k_inv_batched");
+        return VI_OK;
+    }
     hipLaunchKernelGGL(k_unop, dim3(grid_for(n)), dim3(BLOCK), 0, (hipStream_t)stream, op, a, (u64)arg, out, (i64)n);
     VI_LAUNCH_CHECK("k_unop");
     return VI_OK;

@@ -127,6 +127,27 @@ VI_HD u64 pow(u64 base, u64 e) {
     return r;
 }
 
+VI_HD u64 sqr_n(u64 x, int n) {
+    for (int i = 0; i < n; ++i) x = mul(x, x);
+    return x;
+}
+
+// x^(p-2) by a fixed addition chain: p - 2 = (2^31 - 1) * 2^33 + (2^32 - 1), and x^(2^k - 1)
+// doubles its k with k squarings and one product.  64 squarings + 10 products instead of the
+// 63 + 62 of square-and-multiply; 0 -> 0 like the Fermat power.
+VI_HD u64 inv(u64 x) {
+    u64 a2 = mul(sqr_n(x, 1), x);            // 2^2 - 1
+    u64 a4 = mul(sqr_n(a2, 2), a2);
+    u64 a8 = mul(sqr_n(a4, 4), a4);
+    u64 a16 = mul(sqr_n(a8, 8), a8);
+    u64 a24 = mul(sqr_n(a16, 8), a8);
+    u64 a28 = mul(sqr_n(a24, 4), a4);
+    u64 a30 = mul(sqr_n(a28, 2), a2);
+    u64 a31 = mul(sqr_n(a30, 1), x);         // 2^31 - 1
+    u64 a32 = mul(sqr_n(a31, 1), x);         // 2^32 - 1
+    return mul(sqr_n(a31, 33), a32);
+}
+
 // canonical x times 2^s for 0 <= s < 96, as shifts: the 64-bit value moved left by
 // s bits occupies at most three 32-bit limbs L[q..q+2] (s = 32q + r) of
 //   L0 + L1*phi + L2*phi^2 + L3*phi^3 + L4*phi^4,  phi = 2^32,

@@ -98,8 +98,9 @@ def gl_inv(a):
 
 
 def gl_inv_batched(a):
-    """Inverse of every element of a 1-D tensor (one Fermat power per lane, as the
-    reference does since cuda_primitives.py:289-303)."""
+    """Inverse of every element of a 1-D tensor, 0 -> 0, the values of the reference's
+    per-lane Fermat power (cuda_primitives.py:289-303); computed eight elements to one
+    inversion with Montgomery's trick in registers."""
     _check_u64(a, "a")
     if a.dim() != 1:
         raise RuntimeError("gl_inv_batched: 1-D input only")
