@@ -8,7 +8,7 @@
  * Every function restates, in plain scalar C, the algorithm of a reference file
  * (cited per function as path:line under the upstream tree).  The restatement is
  * deliberately the slow textbook form; independent pins (closed forms, brute
- * force, invariants) live in tests/test_oracle_*.py.
+ * force, invariants, published known answers) live in tests/test_oracle.py.
  *
  * Parity status (what pins each function):
  *   vo_add/vo_sub/vo_mul/vo_pow/vo_inv  pinned: Python big-int (a op b) % p, edge set
@@ -21,6 +21,20 @@
  *                                       numpy restatement and closed-form cases; agreement with the
  *                                       third-party gguf-py 0.19.0 dequantiser is PARITY UNPINNED
  *                                       (package and model file are not available offline).
+ *   vo_blake3                           pinned: the reference's four known answers
+ *                                       (prover/kernels/tests/test_blake3.cu:94-101) + nine published
+ *                                       multi-chunk vectors; cross-checked against a second, level-wise
+ *                                       implementation on random lengths.  The algorithm is the BLAKE3
+ *                                       specification's (the reference takes it from the blake3 1.0.9 wheel
+ *                                       and from prover/kernels/blake3_*.cuh); restated here as the recursive
+ *                                       left-full tree.
+ *   vo_hash_columns                     pinned: equals vo_blake3 of the packed column (prover/protocol.py:100-104)
+ *   vo_merkle_level                     pinned: BLAKE3(left || right) spelled out, odd node doubled, paths verify
+ *   vo_row_prg                          pinned: the stated hash of seed || row || k with the second BLAKE3
+ *                                       implementation, incl. the uint32 row wrap of the contiguous form.
+ *                                       The reference itself notes it has no CPU twin of this kernel.
+ *   vo_eq_vector                        pinned: product formula in Python ints, sums to 1, Boolean points
+ *   (mle_eval = repeated vo_fold)       pinned: pure-Python fold, <f, eq>, Boolean points read the table
  */
 #include <stdint.h>
 #include <stddef.h>

@@ -37,6 +37,7 @@ struct Desc {
     unsigned char fidx[VI_SC_MAX_FACTORS];
     int n_tables, n_terms, deg;
     int coeff_at_end;                       // single term: apply its coefficient in the final reduction
+    int product;                            // one term whose factors are exactly the n_tables tables, once each
     int skip1;                              // S(1) is not summed: it is claim - S(0) (the round's known total)
     u64 claim;                              // S(0) + S(1) when skip1
 };
@@ -55,7 +56,10 @@ __device__ __forceinline__ u64 wave_sum(u64 v) {
 // loads per table and index, so two indices are kept in flight to cover HBM latency.
 // `direct`: a single-workgroup launch writes the finished samples itself (small rounds
 // need no second launch).
-template <int NT, int MODE, int U>
+// PROD: the sum is a single product of all NT tables (a matmul contraction, eq * a * b, the
+// three-factor benchmark instance): the term interpreter below -- scalar loads of the term
+// description and a select chain per factor -- gives way to a fully unrolled product.
+template <int NT, int MODE, int U, bool PROD>
 __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial, u64 *out,
                                                  u64 scale, int direct) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
@@ -73,7 +77,7 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         if (i >= count) continue;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            if (t < D.n_tables) {
+            if (PROD || t < D.n_tables) {
                 const u64 *f = D.src[t];
                 if (MODE == 0) {
                     lo_u[u][t] = f[i];
@@ -101,7 +105,23 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         u64 cur[NT], dif[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-            if (t < D.n_tables) { cur[t] = lo[t]; dif[t] = gl::sub(hi[t], lo[t]); }
+            if (PROD || t < D.n_tables) { cur[t] = lo[t]; dif[t] = gl::sub(hi[t], lo[t]); }
+        if (PROD) {
+#pragma unroll
+            for (int x = 0; x <= NT; ++x) {
+                if (!(x == 1 && D.skip1)) {
+                    u64 prod = cur[0];
+#pragma unroll
+                    for (int t = 1; t < NT; ++t) prod = (t + 1 < NT) ? gl::mul_lazy(prod, cur[t]) : gl::mul(prod, cur[t]);
+                    acc[x] = gl::addc(acc[x], NT == 1 ? gl::canon(prod) : prod);
+                }
+                if (x < NT) {
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) cur[t] = gl::addc(cur[t], dif[t]);
+                }
+            }
+            continue;
+        }
         for (int x = 0; x <= D.deg; ++x) {
             if (!(D.skip1 && x == 1)) {
                 u64 sx = 0;
@@ -237,6 +257,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
     D.n_terms = 0;
     D.deg = 0;
     D.coeff_at_end = 0;
+    D.product = 0;
     D.skip1 = 0;
     D.claim = 0;
     if (!need_terms) return VI_OK;
@@ -257,6 +278,11 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         D.fidx[j] = (unsigned char)factor_idx[j];
     }
     D.coeff_at_end = (n_terms == 1);
+    if (n_terms == 1 && term_off[1] == n_tables && n_tables <= 4) {
+        unsigned seen = 0;
+        for (int j = 0; j < n_tables; ++j) seen |= 1u << factor_idx[j];
+        D.product = (seen == (1u << n_tables) - 1);
+    }
     return VI_OK;
 }
 
@@ -283,12 +309,19 @@ int resident_blocks(K kernel) {
     return nb > MAX_BLOCKS ? MAX_BLOCKS : nb;
 }
 
+template <int NT, int MODE, int U, bool PROD>
+int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
+    static const int cap = resident_blocks(k_round<NT, MODE, U, PROD>);     // per instantiation, first use
+    if (nb > cap) nb = cap;
+    hipLaunchKernelGGL((k_round<NT, MODE, U, PROD>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    return nb;
+}
+
 template <int NT, int MODE, int U>
 int launch_k(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
-    static const int cap = resident_blocks(k_round<NT, MODE, U>);     // per instantiation, first use
-    if (nb > cap) nb = cap;
-    hipLaunchKernelGGL((k_round<NT, MODE, U>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
-    return nb;
+    if (MODE != 1 && NT <= 4 && D.product && D.n_tables == NT)
+        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4)>(D, half, r, partial, nb, out, scale, direct, s);
+    return launch_kp<NT, MODE, U, false>(D, half, r, partial, nb, out, scale, direct, s);
 }
 
 template <int MODE, int U>
