@@ -28,6 +28,12 @@ P = (1 << 64) - (1 << 32) + 1
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 
+# HBM bytes per k_ntt_fast launch of the default LDE leg, averaged over the 16 launches of a step:
+# FETCH_SIZE and WRITE_SIZE read by rocprofv3 in two counter runs of this script (5.55 GB read +
+# 6.01 GB written per step), each scaled by what the same counter reads for a 1 GiB device copy.
+LDE_TRAFFIC_BYTES_PER_LAUNCH = 722.6e6
+
+
 def _events(torch):
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
@@ -393,7 +399,9 @@ def main():
         "config": {"workload": "coset LDE 1024 rows x 2^16 -> 2^18, shift 7 (BASELINE configs[1])",
                    "rows": 1024, "K": 1 << 16, "N": 1 << 18},
         "roofline": {"bound": "hbm", "achieved": lde["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": LDE_TRAFFIC_BYTES_PER_LAUNCH,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a copy probe "
+                                       "(x2.000 / x1.000); not re-measured in this run",
                      "kernel": "k_ntt_fast", "launches_per_step": lde["launches_per_step"],
                      "avg_launch_us": lde["kernel_avg_us"],
                      "algorithmic_bytes_per_launch": lde["alg_bytes_per_launch"]},
