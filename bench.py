@@ -166,6 +166,22 @@ def bench_kquant(torch, steps=20, cpu=True):
     ms = s.elapsed_time(e) / steps
     res = {"ms": ms, "weights_per_s": nb * 256 / (ms * 1e-3), "gbs_algorithmic": nb * 2192 / (ms * 1e-3) / 1e9,
            "frac_of_hbm_peak": nb * 2192 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    for qt, bb in (("Q5_K", 176), ("Q6_K", 210)):                     # same weight count in the other two layouts
+        other = torch.randint(0, 256, (nb, bb), generator=g, dtype=torch.uint8, device="cuda")
+        if qt == "Q6_K":
+            other[:, 208:210] = hd.reshape(nb, 4)[:, :2]
+        else:
+            other[:, 0:4] = hd.reshape(nb, 4)
+        kq.kquant_to_field(other, qt, 4096)
+        torch.cuda.synchronize()
+        s.record()
+        for _ in range(steps):
+            kq.kquant_to_field(other, qt, 4096)
+        e.record()
+        torch.cuda.synchronize()
+        t = s.elapsed_time(e) / steps
+        res[qt.lower() + "_ms"] = t
+        res[qt.lower() + "_gbs_algorithmic"] = nb * (bb + 2048) / (t * 1e-3) / 1e9
     if cpu:
         # C oracle (scalar byte map, OpenMP over blocks) on the whole matrix, compared bit for bit
         import numpy as np

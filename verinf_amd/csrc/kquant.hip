@@ -13,8 +13,10 @@
 // wave), and issues two 16-byte stores, so each store instruction writes 1 KiB of
 // consecutive output.  The reference uses one thread per weight with byte loads.
 //
-// k_generic: one thread per weight, byte loads, any alignment (Q5_K, Q6_K, and
-// Q4_K buffers that are not 4-byte aligned).
+// k_q5k / k_q6k: the same wavefront-per-super-block scheme for the other two layouts.
+//
+// k_generic: one thread per weight, byte loads, any alignment (buffers whose base is not
+// aligned for the wavefront kernels).
 #include "common.hpp"
 #include "gl_field.hpp"
 
@@ -77,6 +79,64 @@ __global__ __launch_bounds__(BLOCK) void k_q4k(const unsigned char *__restrict__
     }
 }
 
+// Q5_K (176 B: d, dmin, 12 scale bytes, 32 bytes of fifth bits, 128 quant bytes): as k_q4k, plus
+// one 16-bit load of the fifth-bit bytes of weights (2l, 2l+1) mod 32; bit s belongs to sub-block s.
+__global__ __launch_bounds__(BLOCK) void k_q5k(const unsigned char *__restrict__ raw, u64 *__restrict__ out, i64 n_blocks, double S) {
+    const int lane = threadIdx.x & 63;
+    const i64 wave = ((i64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const i64 n_waves = ((i64)gridDim.x * BLOCK) >> 6;
+    for (i64 b = wave; b < n_blocks; b += n_waves) {
+        const unsigned char *p = raw + b * 176;
+        const u32 *hdr = (const u32 *)p;
+        u32 h = hdr[0], w0 = hdr[1], w1 = hdr[2], w2 = hdr[3];
+        float d = half_bits_to_float(h & 0xFFFF), dmin = half_bits_to_float(h >> 16);
+        int s = lane >> 4;
+        int nib = 4 * (s & 1);
+        const u32 qh = *(const unsigned short *)(p + 16 + ((2 * lane) & 31));
+        const unsigned short *qs = (const unsigned short *)(p + 48 + (lane >> 5) * 32 + ((2 * lane) & 31));
+        u32 qa = qs[0], qb = qs[32];
+        u32 sc, mn;
+        ulonglong2 r;
+        scale_min(w0, w1, w2, s, sc, mn);
+        r.x = to_field(dequant(d, dmin, sc, mn, ((qa >> nib) & 0xF) | (((qh >> s) & 1) << 4)), S);
+        r.y = to_field(dequant(d, dmin, sc, mn, ((qa >> (8 + nib)) & 0xF) | (((qh >> (8 + s)) & 1) << 4)), S);
+        ulonglong2 *o = (ulonglong2 *)(out + b * 256);
+        o[lane] = r;
+        scale_min(w0, w1, w2, s + 4, sc, mn);
+        r.x = to_field(dequant(d, dmin, sc, mn, ((qb >> nib) & 0xF) | (((qh >> (s + 4)) & 1) << 4)), S);
+        r.y = to_field(dequant(d, dmin, sc, mn, ((qb >> (8 + nib)) & 0xF) | (((qh >> (12 + s)) & 1) << 4)), S);
+        o[64 + lane] = r;
+    }
+}
+
+// Q6_K (210 B: 128 low-nibble bytes, 64 bytes of two-bit highs, 16 int8 scales, d).  210 is not a
+// multiple of four, so a block is only 2-byte aligned: 16-bit loads throughout.  Lane l decodes
+// weights {2l, 2l+1} of each 128-weight half.
+__global__ __launch_bounds__(BLOCK) void k_q6k(const unsigned char *__restrict__ raw, u64 *__restrict__ out, i64 n_blocks, double S) {
+    const int lane = threadIdx.x & 63;
+    const i64 wave = ((i64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
+    const i64 n_waves = ((i64)gridDim.x * BLOCK) >> 6;
+    for (i64 b = wave; b < n_blocks; b += n_waves) {
+        const unsigned char *p = raw + b * 210;
+        const float d = half_bits_to_float(*(const unsigned short *)(p + 208));
+        const int nib = 4 * (lane >> 5), two = 2 * ((lane >> 4) & 3);
+        ulonglong2 *o = (ulonglong2 *)(out + b * 256);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const u32 ql = *(const unsigned short *)(p + half * 64 + ((2 * lane) & 63));
+            const u32 qh = *(const unsigned short *)(p + 128 + half * 32 + ((2 * lane) & 31));
+            const int sc = (int)(signed char)p[192 + half * 8 + (lane >> 3)];
+            const float ds = __fmul_rn(d, (float)sc);
+            const int q0 = (int)(((ql >> nib) & 0xF) | (((qh >> two) & 3) << 4)) - 32;
+            const int q1 = (int)(((ql >> (8 + nib)) & 0xF) | (((qh >> (8 + two)) & 3) << 4)) - 32;
+            ulonglong2 r;
+            r.x = to_field(__fmul_rn(ds, (float)q0), S);
+            r.y = to_field(__fmul_rn(ds, (float)q1), S);
+            o[half * 64 + lane] = r;
+        }
+    }
+}
+
 template <int QT>
 __global__ __launch_bounds__(BLOCK) void k_generic(const unsigned char *__restrict__ raw, u64 *__restrict__ out, i64 n, double S) {
     i64 stride = (i64)gridDim.x * BLOCK;
@@ -128,9 +188,14 @@ extern "C" int vi_kquant_to_field(int qtype, const uint8_t *raw, int64_t n_block
     if (!raw || !out) return vi::fail(VI_EINVAL, "vi_kquant_to_field: null pointer");
     hipStream_t s = (hipStream_t)stream;
     const i64 n = n_blocks * 256;
-    if (qtype == 4 && ((uintptr_t)raw & 3) == 0 && ((uintptr_t)out & 15) == 0) {
-        unsigned g = grid_cap((n_blocks + 3) / 4, 256 * 32);
-        hipLaunchKernelGGL(k_q4k, dim3(g), dim3(BLOCK), 0, s, raw, out, (i64)n_blocks, S);
+    const bool out16 = ((uintptr_t)out & 15) == 0;
+    const unsigned gw = grid_cap((n_blocks + 3) / 4, 256 * 32);        // one wavefront per super-block
+    if (qtype == 4 && ((uintptr_t)raw & 3) == 0 && out16) {
+        hipLaunchKernelGGL(k_q4k, dim3(gw), dim3(BLOCK), 0, s, raw, out, (i64)n_blocks, S);
+    } else if (qtype == 5 && ((uintptr_t)raw & 3) == 0 && out16) {
+        hipLaunchKernelGGL(k_q5k, dim3(gw), dim3(BLOCK), 0, s, raw, out, (i64)n_blocks, S);
+    } else if (qtype == 6 && ((uintptr_t)raw & 1) == 0 && out16) {
+        hipLaunchKernelGGL(k_q6k, dim3(gw), dim3(BLOCK), 0, s, raw, out, (i64)n_blocks, S);
     } else {
         unsigned g = grid_cap((n + BLOCK - 1) / BLOCK, 256 * 32);
         if (qtype == 4) hipLaunchKernelGGL(k_generic<4>, dim3(g), dim3(BLOCK), 0, s, raw, out, n, S);
