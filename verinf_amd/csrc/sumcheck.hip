@@ -133,10 +133,7 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
                     const int j1 = D.term_off[k + 1];
                     for (int j = D.term_off[k]; j < j1; ++j) {
                         int t = D.fidx[j];
-                        u64 v = 0;
-#pragma unroll
-                        for (int u = 0; u < NT; ++u)
-                            if (u == t) v = cur[u];
+                        u64 v = cur[t];
                         prod = first ? v : (j + 1 < j1 ? gl::mul_lazy(prod, v) : gl::mul(prod, v));
                         first = false;
                     }
