@@ -8,15 +8,18 @@ Kept, with the reference's names and argument meaning:
   prove_terms_gpu(terms, coin, field_p, mask, mu0)   gpu.py:350-410
   MAX_GRID_ROWS, _chunk_rows, _coset_powers     gpu.py:33-61, 128-138
 
+  hash_and_tree(cfg, mat), levels_to_host       gpu.py:274-297
+  linear_combination, combine_t, column         gpu.py:113-122, 301-315
+
 What changes underneath: encode is ONE fused library call (no (rows, N) zero
 buffer, no expanded gamma powers, no per-chunk copies), and a sumcheck round is
-one fused kernel plus a single-block reduction instead of ~(deg+1)*(4*factors +
-log n) elementwise launches; the only host synchronisation per round is the
-read-back of the deg+1 samples that the verifier coin needs.
+one fused launch instead of ~(deg+1)*(4*factors + log n) elementwise launches; the
+only host wait per round is for the deg+1 samples that the verifier coin needs.
 
-`linear_combination` and `combine_t` (gpu.py:113-122, 301-308) run on `gl_matmul`.
-The dense Lagrange-matrix encoders (`encode_batch[_t]`) and the BLAKE3 `hash_and_tree` of
-the reference module are outside this package (the NTT encoder is the one encoder here).
+Added for device consumers: eq_vector_t, mle_eval_t (the reference's eq_vector /
+mle_eval work on Python lists).  The dense Lagrange-matrix encoders
+(`encode_batch[_t]`) of the reference module are not provided: the NTT encoder is
+the one encoder here.
 """
 import ctypes
 from typing import Optional, Sequence
