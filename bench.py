@@ -62,17 +62,22 @@ def bench_lde(torch, steps, warmup, ws_mb=0):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    s, e = _events(torch)
-    s.record()
-    for _ in range(steps):
+    # one event pair around the K timed steps (the reported figure) and an event after every step,
+    # on the stream the kernels run on, for the spread between steps
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    marks[0].record()
+    for i in range(steps):
         step()
-    e.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
-    ms = s.elapsed_time(e) / steps
+    ms = marks[0].elapsed_time(marks[steps]) / steps
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    q = lambda f: per_step[min(steps - 1, int(f * steps))]
     launches = int(L.vi_coset_lde_launches(m, K, N, ws_bytes))
     alg_bytes = 8 * (K + N) * m                       # compulsory traffic of one step
     res = {
         "ms_per_step": ms,
+        "ms_per_step_median": q(0.5), "ms_per_step_iqr": [q(0.25), q(0.75)],
         "elems_per_s": m * N / (ms * 1e-3),
         "launches_per_step": launches,
         "kernel_avg_us": ms * 1e3 / launches,
@@ -407,6 +412,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": lde["ms_per_step"],
+        "ms_per_step_median": lde["ms_per_step_median"],
+        "ms_per_step_iqr": lde["ms_per_step_iqr"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
