@@ -135,3 +135,13 @@ def test_host_verifier_accepts_oracle_proofs_and_rejects_tampering():
     assert tp.take(2) == [1, 2]
     with pytest.raises(RuntimeError):
         tp.take(2)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build runs on one GPU; bench.py says so instead of starting ranks."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0
+    assert "ONE GPU" in res.stderr
