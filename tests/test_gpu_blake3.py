@@ -142,7 +142,6 @@ def test_full_size_properties(cp):
     root, levels = cp.merkle_build_blake3(dig)
     assert len(levels) == 19 and levels[-1].shape == (1, 32)
     # a path read off the device tree verifies on the host
-    from verinf_amd.layergkr import gpu as lg, rs
     from verinf_amd.prover.protocol import merkle_verify
     idx = 123457
     path = []
