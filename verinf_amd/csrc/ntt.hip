@@ -53,14 +53,24 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     //  * a loop over the cosets inside one workgroup: every address becomes loop-invariant,
     //    ~50 more live registers, spills;
     //  * persistent workgroups prefetching the next tile into a second register buffer: -3 %;
+    //  * two tiles per workgroup with both tiles' loads issued up front: -6 % (128 registers, spills);
     //  * workgroup ids laid out so that the cosets of a tile share an XCD and its L2 (ids 8
     //    apart): fetch traffic of the pass drops from 537 to 134 MB per 256 rows, run time
     //    rises 2.6 % -- the pass is bound by integer VALU issue, not by HBM.
     const int t = blockIdx.y;
-    for (int i = tid; i < (16 << A2); i += NTHREADS) twi[i] = A.twi[i];
-    __syncthreads();
     u64 reg[16];
     fast_load<A2>(A, tile, tid, reg);
+    if (!A.is_final) {
+        // strided pass: a wavefront uses only the table rows of its own n2 values (at most 64 words), so each
+        // wavefront fills just those and no workgroup barrier is needed before stage 1
+        const int lt = TILE_LOG - A.a;
+        const int lane = tid & 63, first = ((tid & ~63) >> lt) * 16, count = lt >= 6 ? 16 : (16 << (6 - lt));
+        if (lane < count) twi[first + lane] = A.twi[first + lane];
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        for (int i = tid; i < (16 << A2); i += NTHREADS) twi[i] = A.twi[i];
+        __syncthreads();
+    }
     fast_stage1<A2, INV>(A, tile, tid, t, reg, twi, lds);
     __syncthreads();
     fast_stage2<A2, INV>(A, tile, tid, t, lds);
