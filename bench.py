@@ -278,7 +278,7 @@ def bench_layer(torch):
     for name, (n_rows, n_in) in acts.items():
         msgs += rows_of(n_rows, n_in, -(1 << 15), 1 << 15)
     total_rows = sum(int(m.shape[0]) for m in msgs)
-    out = torch.empty((max(int(m.shape[0]) for m in msgs), N), dtype=torch.uint64, device="cuda")
+    codes = [torch.empty((int(m.shape[0]), N), dtype=torch.uint64, device="cuda") for m in msgs]    # 31 GB of codewords stay resident
     widths = [1 << 12] * 6 + [1 << 14]
     mm_tabs = [[rand_field(torch, (w,), 100 + 2 * i), rand_field(torch, (w,), 101 + 2 * i)] for i, w in enumerate(widths)]
     gate_tabs = [rand_field(torch, (1 << 24,), 200 + j) for j in range(3)]
@@ -287,8 +287,7 @@ def bench_layer(torch):
 
     def commit(hash_too=True):
         roots = []
-        for m in msgs:
-            code = out[: m.shape[0]]
+        for m, code in zip(msgs, codes):
             cp.coset_lde(m, K, N, 7, out=code)
             if hash_too:
                 roots.append(cp.merkle_build_blake3(cp.hash_columns_streamed(code))[0])
@@ -303,10 +302,10 @@ def bench_layer(torch):
     chis = [rand_field(torch, (1, int(m.shape[0])), 300 + i) for i, m in enumerate(msgs[:n_w])]
 
     def projections():
-        """chi^T W per weight block: the (1 x n_out) @ (n_out x width) seam product of
-        layergkr/projection.py:150-167; streams every committed weight message once."""
-        for chi, m in zip(chis, msgs[:n_w]):
-            cp.gl_matmul(chi, m)
+        """chi^T C per committed weight block: the (1 x rows) @ (rows x N) combination of
+        layergkr/gpu.py:301-308 / projection.py:150-167; streams every weight codeword once."""
+        for chi, code in zip(chis, codes[:n_w]):
+            cp.gl_matmul(chi, code)
 
     commit(); projections(); sumchecks()         # warm-up (twiddle tables, workspaces)
     torch.cuda.synchronize()
@@ -322,7 +321,7 @@ def bench_layer(torch):
     torch.cuda.synchronize()
     tp = time.perf_counter()
     proj_ms = (tp - t1) * 1e3
-    proj_bytes = sum(int(m.numel()) * 8 for m in msgs[:n_w])
+    proj_bytes = sum(int(c.numel()) * 8 for c in codes[:n_w])
     t1b = time.perf_counter()
     sumchecks()
     torch.cuda.synchronize()
