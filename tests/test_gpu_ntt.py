@@ -135,7 +135,8 @@ def test_lde_golden(cp, golden_dir):
 @pytest.mark.parametrize("logK,logN,m,w", [(1, 1, 3, 2), (1, 3, 3, 1), (3, 5, 700, 8), (5, 6, 4, 16), (7, 8, 9, 64),
                                            (9, 10, 3, 256), (10, 10, 3, 1000), (4, 7, 5, 11), (12, 14, 16, 4096),
                                            (13, 15, 5, 5000), (14, 16, 9, 8192), (16, 18, 5, 65536),
-                                           (16, 17, 3, 40000), (17, 19, 2, 1 << 17)])
+                                           (16, 17, 3, 40000), (17, 19, 2, 1 << 17), (18, 20, 2, 200000), (20, 22, 1, 1 << 20),
+                                           (8, 14, 3, 256), (12, 18, 2, 4000)])
 def test_lde_matches_oracle(cp, logK, logN, m, w):
     msgs = rand_field((m, w), 200 + logK)
     got = cp.coset_lde(to_dev(msgs), 1 << logK, 1 << logN, 7)
@@ -229,3 +230,40 @@ def test_lde_full_baseline_shape_properties(cp):
         cp.ntt_inverse_batched(blk)
         assert not bool(blk.view(torch.int64)[:, K:].any())
     del out
+
+
+def test_two_host_threads_on_their_own_streams(cp):
+    """The library keeps per-device table caches behind a mutex and no other shared state: two
+    host threads, each with its own stream and workspace, transform different data at the same
+    time (first use of two table sizes included) and both results are bit-exact."""
+    import threading
+    from verinf_amd import _lib
+    L = _lib.lib()
+    jobs = [(1 << 11, 1 << 13, 300, 31), (1 << 15, 1 << 17, 40, 32)]       # sizes no other test has warmed up
+    results, errors = {}, []
+
+    def work(i, K, N, m, seed):
+        try:
+            st = torch.cuda.Stream()
+            msgs = rand_field((m, K), seed)
+            with torch.cuda.stream(st):
+                dev = to_dev(msgs)
+                out = torch.empty((m, N), dtype=torch.uint64, device="cuda")
+                ws = torch.empty(L.vi_coset_lde_workspace_bytes(m, K, N), dtype=torch.uint8, device="cuda")
+                for _ in range(3):
+                    _lib.check(L.vi_coset_lde(dev.data_ptr(), m, K, K, K, N, 7, out.data_ptr(), N, ws.data_ptr(),
+                                              ws.numel(), st.cuda_stream))
+                st.synchronize()
+                results[i] = (msgs, to_np(out), K, N)
+        except Exception as exc:            # surfaced in the main thread
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(i,) + j) for i, j in enumerate(jobs)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for msgs, got, K, N in results.values():
+        rows = [0, msgs.shape[0] - 1]
+        assert np.array_equal(got[rows], O.coset_lde_rows(np.ascontiguousarray(msgs[rows]), K, N, 7))
