@@ -145,3 +145,45 @@ def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode != 0
     assert "ONE GPU" in res.stderr
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """include/verinf_hip.h is a C header (no C++ or torch types): it compiles as C99 and as C++,
+    and a C program that includes it links against the library and can call the entry points
+    that need no device (version string, workspace queries, argument validation)."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    hdr = os.path.join(root, "include", "verinf_hip.h")
+    lib = os.path.join(root, "verinf_amd", "libverinf_hip.so")
+    if not os.path.exists(lib):
+        from verinf_amd.build import build
+        build()
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c", hdr])
+    subprocess.check_call(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", hdr])
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "verinf_hip.h"
+int main(void) {
+    if (!vi_version() || !strlen(vi_version())) return 1;
+    if (vi_coset_lde_workspace_bytes(1024, 65536, 262144) == 0) return 2;
+    if (vi_coset_lde_min_workspace_bytes(65536, 262144) != (size_t)(65536 + 262144) * 8) return 3;
+    if (vi_hash_columns_workspace_bytes(1024, 262144) != (size_t)(8 + 4) * 262144 * 32) return 4;
+    if (vi_sumcheck_workspace_bytes() == 0 || vi_mle_eval_workspace_bytes(3) != 3 * 8192) return 5;
+    /* bad arguments are refused before anything touches a device */
+    static uint64_t dummy[4];     /* never dereferenced: K = 12 is refused first */
+    if (vi_coset_lde(dummy, 4, 3, 3, 12, 48, 7, dummy, 48, 0, 0, 0) != VI_EINVAL) return 6;
+    if (!strstr(vi_last_error(), "powers of two")) return 7;
+    if (vi_kquant_to_field(8, 0, 1, 4096.0, 0, 0) != VI_EINVAL) return 8;
+    if (vi_row_prg(0, 0, 0, 4, 4, 0, 2, 0) != VI_EINVAL) return 9;
+    puts(vi_version());
+    return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    hip_lib_dir = "/opt/rocm/lib"
+    subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(root, "include"), str(src), "-o", str(exe), lib,
+                           "-Wl,-rpath," + os.path.dirname(lib), "-Wl,-rpath," + hip_lib_dir, "-L" + hip_lib_dir, "-lamdhip64"])
+    res = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert res.returncode == 0, (res.returncode, res.stdout, res.stderr)
