@@ -76,24 +76,41 @@ __device__ __forceinline__ u64 block_sum(u64 v, u64 *lds4) {
     return r;
 }
 
-// partial[row * gridDim.x + block] = sum over this block's share of f_row[i] * eq[i]
+// partial[row * gridDim.x + block] = sum over this block's share of f_row[i] * eq[i], for the up to TB
+// tables row = blockIdx.y * TB + 0 .. TB-1: the eq entries of an index are computed once and used for all
+// of them.
+constexpr int TB = 4;
+
 template <int JB>
 __global__ __launch_bounds__(BLOCK) void k_mle_partial(const Point pt, int n, const u64 *__restrict__ tables, i64 row_stride,
-                                                       u64 *__restrict__ partial) {
+                                                       int n_tables, u64 *__restrict__ partial) {
     __shared__ u64 lds4[BLOCK / 64];
     const i64 threads = (i64)1 << (n - JB);
-    const u64 *f = tables + (i64)blockIdx.y * row_stride;
-    u64 acc = 0;
-    for (i64 g = (i64)blockIdx.x * BLOCK + threadIdx.x; g < threads; g += (i64)gridDim.x * BLOCK) {
-        u64 e[1 << JB], v[1 << JB];
+    const int row0 = blockIdx.y * TB;
+    const int rows = n_tables - row0 < TB ? n_tables - row0 : TB;
+    u64 acc[TB];
 #pragma unroll
-        for (int j = 0; j < (1 << JB); ++j) v[j] = f[((i64)j << (n - JB)) | g];
+    for (int r = 0; r < TB; ++r) acc[r] = 0;
+    for (i64 g = (i64)blockIdx.x * BLOCK + threadIdx.x; g < threads; g += (i64)gridDim.x * BLOCK) {
+        u64 e[1 << JB];
         eq_entries<JB>(pt, n, g, e);
 #pragma unroll
-        for (int j = 0; j < (1 << JB); ++j) acc = gl::add(acc, gl::mul(e[j], v[j]));
+        for (int r = 0; r < TB; ++r) {
+            if (r < rows) {
+                const u64 *f = tables + (i64)(row0 + r) * row_stride;
+                u64 v[1 << JB];
+#pragma unroll
+                for (int j = 0; j < (1 << JB); ++j) v[j] = f[((i64)j << (n - JB)) | g];
+#pragma unroll
+                for (int j = 0; j < (1 << JB); ++j) acc[r] = gl::add(acc[r], gl::mul(e[j], v[j]));
+            }
+        }
     }
-    const u64 r = block_sum(acc, lds4);
-    if (threadIdx.x == 0) partial[(i64)blockIdx.y * gridDim.x + blockIdx.x] = r;
+#pragma unroll
+    for (int r = 0; r < TB; ++r) {
+        const u64 s = block_sum(acc[r], lds4);
+        if (threadIdx.x == 0 && r < rows) partial[(i64)(row0 + r) * gridDim.x + blockIdx.x] = s;
+    }
 }
 
 __global__ __launch_bounds__(BLOCK) void k_mle_final(const u64 *__restrict__ partial, int nb, u64 *__restrict__ out) {
@@ -153,15 +170,15 @@ int vi_mle_eval(const uint64_t *tables, int64_t n_tables, int64_t row_stride, co
     const i64 threads = (i64)1 << (n_vars - jb);
     i64 nb = (threads + BLOCK - 1) / BLOCK;
     if (nb > PARTIAL_BLOCKS) nb = PARTIAL_BLOCKS;
-    const dim3 grid((unsigned)nb, (unsigned)n_tables), block(BLOCK);
+    const dim3 grid((unsigned)nb, (unsigned)((n_tables + TB - 1) / TB)), block(BLOCK);
     hipStream_t s = (hipStream_t)stream;
     u64 *partial = (u64 *)ws;
     switch (jb) {
-        case 0: hipLaunchKernelGGL(k_mle_partial<0>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, partial); break;
-        case 1: hipLaunchKernelGGL(k_mle_partial<1>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, partial); break;
-        case 2: hipLaunchKernelGGL(k_mle_partial<2>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, partial); break;
-        case 3: hipLaunchKernelGGL(k_mle_partial<3>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, partial); break;
-        default: hipLaunchKernelGGL(k_mle_partial<4>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, partial); break;
+        case 0: hipLaunchKernelGGL(k_mle_partial<0>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, (int)n_tables, partial); break;
+        case 1: hipLaunchKernelGGL(k_mle_partial<1>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, (int)n_tables, partial); break;
+        case 2: hipLaunchKernelGGL(k_mle_partial<2>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, (int)n_tables, partial); break;
+        case 3: hipLaunchKernelGGL(k_mle_partial<3>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, (int)n_tables, partial); break;
+        default: hipLaunchKernelGGL(k_mle_partial<4>, grid, block, 0, s, pt, n_vars, tables, (i64)row_stride, (int)n_tables, partial); break;
     }
     VI_LAUNCH_CHECK("k_mle_partial");
     hipLaunchKernelGGL(k_mle_final, dim3((unsigned)n_tables), block, 0, s, (const u64 *)partial, (int)nb, out);
