@@ -188,3 +188,35 @@ def test_fold_eval_in_place_c_abi(mods):
         assert np.array_equal(to_np(t)[: 1 << 11], f)
     _, samples, _ = O.sumcheck_prove(folded, [(1, [0, 1, 2])], [0] * 11)
     assert [int(x) for x in out.cpu().tolist()] == samples[0]
+
+
+def test_verifier_accepts_and_rejects_device_table_proofs(mods):
+    """prove_terms / verify_terms on device tensors at a size where host lists are out of the
+    question (2^20): the verifier's terminal check evaluates the tables on the device.  A shared
+    factor, two terms, then a tampered sample and a tampered table."""
+    gpu, sc = mods
+    v = 20
+    eq = gpu.eq_vector_t([random.Random(3).randrange(P) for _ in range(v)])
+    a, b, c = (to_dev(rand_field((1 << v,), 60 + i)) for i in range(3))
+    terms = [(5, [eq, a, b]), (P - 2, [eq, c])]
+    coins = [random.Random(4).randrange(P) for _ in range(v)]
+    proof = sc.prove_terms(terms, lambda i: coins[i])
+    ok, why = sc.verify_terms(proof, terms, lambda i: coins[i])
+    assert ok, why
+    # the claim is the sum the terms define
+    want = (5 * int(gpu.gl_sum(cp_mul(cp_mul(eq, a), b)).cpu().item()) - 2 * int(gpu.gl_sum(cp_mul(eq, c)).cpu().item())) % P
+    assert proof.claim == want
+    bad = sc.SumcheckProof(**{**proof.__dict__})
+    bad.round_polys = [list(s) for s in proof.round_polys]
+    x, y = bad.round_polys[7][2]
+    bad.round_polys[7][2] = (x, (y + 1) % P)
+    assert not sc.verify_terms(bad, terms, lambda i: coins[i])[0]
+    c2 = c.clone()
+    c2.view(torch.int64)[12345] += 1
+    ok, why = sc.verify_terms(proof, [(5, [eq, a, b]), (P - 2, [eq, c2])], lambda i: coins[i])
+    assert not ok and "terminal" in why
+
+
+def cp_mul(x, y):
+    from verinf_amd.prover import cuda_primitives as cp
+    return cp.gl_mul(x, y)

@@ -146,8 +146,17 @@ def prove(factors: Sequence[Sequence[int]], coin: Callable[[int], int],
     return prove_terms([(1, list(factors))], coin, tape, mu0)
 
 
-def _host_values(f):
-    return [int(v) for v in f.cpu().tolist()] if hasattr(f, "shape") else f
+def _terminal_value(f, point, cache):
+    """f~(point) for a factor given as a Python list (host fold, layergkr/sumcheck.py:40-48) or as a
+    device table (one device pass); a table object shared by several terms is evaluated once."""
+    key = id(f)
+    if key not in cache:
+        if hasattr(f, "shape"):
+            from . import gpu
+            cache[key] = gpu.mle_eval_t(f.reshape(-1), point)
+        else:
+            cache[key] = mle_eval(f, point)
+    return cache[key]
 
 
 def verify_terms(proof: SumcheckProof, terms: Sequence[Term],
@@ -164,11 +173,11 @@ def verify_terms(proof: SumcheckProof, terms: Sequence[Term],
         if r != proof.challenges[rnd]:
             return False, f"round {rnd}: challenge mismatch"
         running = _lagrange_interpolate(samples, r)
-    terminal = 0
+    terminal, seen = 0, {}
     for c, fs in terms:
         prod = c % FIELD_P
         for f in fs:
-            prod = prod * mle_eval(_host_values(f), proof.final_point) % FIELD_P
+            prod = prod * _terminal_value(f, proof.final_point, seen) % FIELD_P
         terminal += prod
     terminal %= FIELD_P
     if proof.masked:
