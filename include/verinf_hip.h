@@ -239,6 +239,29 @@ size_t vi_mle_eval_workspace_bytes(int64_t n_tables);
 int vi_mle_eval(const uint64_t *tables, int64_t n_tables, int64_t row_stride, const uint64_t *z, int n_vars,
                 uint64_t *out, void *ws, size_t ws_bytes, void *stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * The remaining field primitives of the production prover that sit next to the path.
+ *
+ * vi_challenge replaces challenge_vec / challenge_at (prover/cuda_primitives.py:551-592, 1233-1248):
+ *   out[i] = challenge(seed, cid_i, label) = le128(BLAKE3(seed[32] || label || cid_le8)[0:16]) mod p
+ * (prover/protocol.py:127-135) with cid_i = cids[i], or i when cids is NULL.  seed (32 bytes, 4-byte aligned) and
+ * label (label_len <= 8 bytes) are device pointers.
+ *
+ * vi_gl_spmv replaces gl_spmv / gl_spmv_challenged (prover/cuda_primitives.py:512-548, prover/kernels/gl_spmv.cuh):
+ *   y[i] = sum over p in [row_ptr[i], row_ptr[i+1]) of values[p] * x[col_idx[p]]   (CSR, all words uint64),
+ * and with x == NULL the combiner entry is challenge(seed, col_idx[p], label) computed in place.
+ *
+ * vi_lookup_multiplicities replaces lookup_multiplicities[_into] and its range form
+ * (prover/cuda_primitives.py:1008-1052, prover/kernels/gl_extras.cuh:118-150): mult[j] += 1 for every i whose
+ * x[i] equals table[j] (the first such j); values not in the table count nowhere.  table_is_range != 0 promises
+ * table[j] == j, which makes the search an index.  mult accumulates: zero it for a fresh histogram. */
+int vi_challenge(const uint8_t *seed, const uint8_t *label, int label_len, const uint64_t *cids, int64_t n, uint64_t *out,
+                 void *stream);
+int vi_gl_spmv(const uint64_t *values, const uint64_t *col_idx, const uint64_t *row_ptr, int64_t n_rows, int64_t nnz,
+               const uint64_t *x, const uint8_t *seed, const uint8_t *label, int label_len, uint64_t *y, void *stream);
+int vi_lookup_multiplicities(const uint64_t *x, int64_t n_x, const uint64_t *table, int64_t n_table, int table_is_range,
+                             uint64_t *mult, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -72,6 +72,9 @@ def lib():
         L.vo_merkle_level.argtypes = [u8p, c_size_t, u8p]
         L.vo_row_prg.argtypes = [u8p, u64p, c_uint64, c_size_t, c_size_t, u64p]
         L.vo_eq_vector.argtypes = [u64p, c_int, u64p]
+        L.vo_challenge_vec.argtypes = [u8p, u8p, c_int, u64p, c_size_t, u64p]
+        L.vo_spmv.argtypes = [u64p, u64p, u64p, c_size_t, u64p, u8p, u8p, c_int, u64p]
+        L.vo_lookup_multiplicities.argtypes = [u64p, c_size_t, u64p, c_size_t, u64p]
         _lib = L
     return _lib
 
@@ -238,6 +241,42 @@ def mle_eval(values: np.ndarray, point) -> int:
     for r in point:
         cur = fold(cur, int(r) % P)
     return int(cur[0])
+
+
+def _bytes8(b: bytes):
+    return np.frombuffer(bytes(b) + b"\x00", dtype=np.uint8).copy()
+
+
+def challenge_vec(seed: bytes, label: bytes, n: int = 0, cids=None) -> np.ndarray:
+    """challenge(seed, cid, label) for cid = 0..n-1 or for the given cids (prover/protocol.py:127-135)."""
+    assert len(seed) == 32 and len(label) <= 8
+    idx = None if cids is None else np.ascontiguousarray(cids, dtype=np.uint64)
+    n = n if idx is None else idx.size
+    out = np.empty(n, dtype=np.uint64)
+    if n:
+        lib().vo_challenge_vec(_p8(_bytes8(seed)), _p8(_bytes8(label)), len(label), _p64(idx) if idx is not None else None, n, _p64(out))
+    return out
+
+
+def spmv(values, col_idx, row_ptr, x=None, seed: bytes = b"", label: bytes = b"") -> np.ndarray:
+    """CSR matrix times x over the field; x = None uses the challenged combiner of (seed, label)."""
+    values, col_idx, row_ptr = (np.ascontiguousarray(a, dtype=np.uint64) for a in (values, col_idx, row_ptr))
+    n_rows = row_ptr.size - 1
+    y = np.zeros(max(n_rows, 0), dtype=np.uint64)
+    if n_rows > 0:
+        xv = None if x is None else np.ascontiguousarray(x, dtype=np.uint64)
+        pad = np.zeros(1, dtype=np.uint64)
+        lib().vo_spmv(_p64(values if values.size else pad), _p64(col_idx if col_idx.size else pad), _p64(row_ptr), n_rows,
+                      _p64(xv) if xv is not None else None, _p8(_bytes8(seed.ljust(32, b"\0"))), _p8(_bytes8(label)), len(label), _p64(y))
+    return y
+
+
+def lookup_multiplicities(x, table) -> np.ndarray:
+    x, table = np.ascontiguousarray(x, dtype=np.uint64), np.ascontiguousarray(table, dtype=np.uint64)
+    mult = np.zeros(table.size, dtype=np.uint64)
+    if x.size and table.size:
+        lib().vo_lookup_multiplicities(_p64(x), x.size, _p64(table), table.size, _p64(mult))
+    return mult
 
 
 def merkle_levels(leaves: np.ndarray):

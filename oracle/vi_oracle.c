@@ -33,6 +33,8 @@
  *   vo_row_prg                          pinned: the stated hash of seed || row || k with the second BLAKE3
  *                                       implementation, incl. the uint32 row wrap of the contiguous form.
  *                                       The reference itself notes it has no CPU twin of this kernel.
+ *   vo_challenge / vo_challenge_vec     pinned: the PRF of prover/protocol.py:127-135 spelled out with the second BLAKE3
+ *   vo_spmv, vo_lookup_multiplicities   pinned: Python big-int row sums; hand-counted histogram (duplicate table entry)
  *   vo_eq_vector                        pinned: product formula in Python ints, sums to 1, Boolean points
  *   (mle_eval = repeated vo_fold)       pinned: pure-Python fold, <f, eq>, Boolean points read the table
  */
@@ -583,4 +585,42 @@ void vo_eq_vector(const u64 *z, int n, u64 *out) {
         }
         len *= 2;
     }
+}
+
+/* prover/protocol.py:127-135: le128(BLAKE3(seed || label || cid_le8)[0:16]) mod p */
+u64 vo_challenge(const uint8_t seed[32], const uint8_t *label, int label_len, u64 cid) {
+    uint8_t msg[48], dig[32];
+    memcpy(msg, seed, 32);
+    if (label_len > 0) memcpy(msg + 32, label, (size_t)label_len);
+    for (int b = 0; b < 8; ++b) msg[32 + label_len + b] = (uint8_t)(cid >> (8 * b));
+    vo_blake3(msg, (size_t)(40 + label_len), dig);
+    u128 v = 0;
+    for (int b = 15; b >= 0; --b) v = (v << 8) | dig[b];
+    return (u64)(v % GL_P);
+}
+
+void vo_challenge_vec(const uint8_t seed[32], const uint8_t *label, int label_len, const u64 *cids, size_t n, u64 *out) {
+    #pragma omp parallel for schedule(static)
+    for (long i = 0; i < (long)n; ++i) out[i] = vo_challenge(seed, label, label_len, cids ? cids[i] : (u64)i);
+}
+
+/* prover/kernels/gl_spmv.cuh:25-41, 72-92: CSR row dot products; x == NULL means the challenged combiner */
+void vo_spmv(const u64 *values, const u64 *col_idx, const u64 *row_ptr, size_t n_rows, const u64 *x,
+             const uint8_t *seed, const uint8_t *label, int label_len, u64 *y) {
+    #pragma omp parallel for schedule(dynamic, 64)
+    for (long i = 0; i < (long)n_rows; ++i) {
+        u64 s = 0;
+        for (u64 p = row_ptr[i]; p < row_ptr[i + 1]; ++p) {
+            u64 xv = x ? x[col_idx[p]] % GL_P : vo_challenge(seed, label, label_len, col_idx[p]);
+            s = vo_add(s, vo_mul(values[p] % GL_P, xv));
+        }
+        y[i] = s;
+    }
+}
+
+/* prover/kernels/gl_extras.cuh:118-150: mult[j] += 1 for the first j with table[j] == x[i] */
+void vo_lookup_multiplicities(const u64 *x, size_t n_x, const u64 *table, size_t n_table, u64 *mult) {
+    for (size_t i = 0; i < n_x; ++i)
+        for (size_t j = 0; j < n_table; ++j)
+            if (table[j] == x[i]) { mult[j] += 1; break; }
 }

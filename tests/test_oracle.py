@@ -387,3 +387,42 @@ def test_mle_eval_matches_definition():
         # Boolean points read the table
         i = rng.randrange(1 << n)
         assert O.mle_eval(f, [(i >> (n - 1 - j)) & 1 for j in range(n)]) == int(f[i])
+
+
+# ---- combiner challenge, CSR matvec, multiplicities --------------------------------------
+def test_challenge_is_the_stated_prf():
+    from verinf_amd.prover.protocol import blake3_digest
+    seed = bytes((5 * i + 1) % 256 for i in range(32))
+    for label in (b"", b"lin", b"irs", b"quad", b"12345678"):
+        got = O.challenge_vec(seed, label, 5)
+        for i in range(5):
+            d = blake3_digest(seed + label + i.to_bytes(8, "little"))
+            assert int(got[i]) == int.from_bytes(d[:16], "little") % P
+        cids = [7, 1 << 40, (1 << 64) - 1]
+        at = O.challenge_vec(seed, label, cids=cids)
+        for c, v in zip(cids, at):
+            d = blake3_digest(seed + label + c.to_bytes(8, "little"))
+            assert int(v) == int.from_bytes(d[:16], "little") % P
+
+
+def test_spmv_and_multiplicities_match_python():
+    rng = random.Random(31)
+    n_rows, n_cols = 40, 90
+    rows = [[(rng.randrange(n_cols), rng.randrange(P)) for _ in range(rng.randrange(0, 9))] for _ in range(n_rows)]
+    row_ptr, col, val = [0], [], []
+    for r in rows:
+        for c, v in r:
+            col.append(c); val.append(v)
+        row_ptr.append(len(col))
+    x = [rng.randrange(P) for _ in range(n_cols)]
+    got = O.spmv(np.array(val, dtype=np.uint64), np.array(col, dtype=np.uint64), np.array(row_ptr, dtype=np.uint64),
+                 np.array(x, dtype=np.uint64))
+    assert [int(v) for v in got] == [sum(v * x[c] for c, v in r) % P for r in rows]
+    seed = bytes(range(32))
+    r_vec = O.challenge_vec(seed, b"lin", n_cols)
+    got_c = O.spmv(np.array(val, dtype=np.uint64), np.array(col, dtype=np.uint64), np.array(row_ptr, dtype=np.uint64),
+                   None, seed, b"lin")
+    assert [int(v) for v in got_c] == [sum(v * int(r_vec[c]) for c, v in r) % P for r in rows]
+    table = [3, 9, 4, 9, 100]                       # a duplicate entry: the first one collects
+    xs = [9, 9, 3, 5, 100, 4, 4, 4, 77]
+    assert [int(v) for v in O.lookup_multiplicities(xs, table)] == [1, 2, 3, 0, 1]

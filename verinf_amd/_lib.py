@@ -29,6 +29,7 @@ EXPORTS = [
     "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
     "vi_merkle_level", "vi_row_prg",
     "vi_eq_vector", "vi_mle_eval_workspace_bytes", "vi_mle_eval",
+    "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities",
 ]
 
 COIN_FN = ctypes.CFUNCTYPE(c_int, c_int, POINTER(c_uint64), c_int, POINTER(c_uint64), c_void_p)
@@ -94,6 +95,9 @@ def lib():
     L.vi_hash_columns_finalize.argtypes = [i64, i64, vp, sz, vp, vp]
     L.vi_merkle_level.argtypes = [vp, i64, vp, vp]
     L.vi_row_prg.argtypes = [vp, vp, i64, i64, i64, vp, i64, vp]
+    L.vi_challenge.argtypes = [vp, vp, c_int, vp, i64, vp, vp]
+    L.vi_gl_spmv.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, c_int, vp, vp]
+    L.vi_lookup_multiplicities.argtypes = [vp, i64, vp, i64, c_int, vp, vp]
     L.vi_eq_vector.argtypes = [POINTER(u64), c_int, c_int, vp, vp]
     L.vi_mle_eval_workspace_bytes.restype = sz
     L.vi_mle_eval_workspace_bytes.argtypes = [i64]
@@ -104,7 +108,8 @@ def lib():
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
                  "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_sumcheck_eval",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
-                 "vi_merkle_level", "vi_row_prg", "vi_eq_vector", "vi_mle_eval"):
+                 "vi_merkle_level", "vi_row_prg", "vi_eq_vector", "vi_mle_eval",
+                 "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

@@ -15,6 +15,7 @@
 // pass over the matrix with as many independent threads as the GPU wants, and it can be
 // fed in row slabs (vi_hash_columns_update) while the codewords are produced.
 #include "common.hpp"
+#include "gl_field.hpp"
 
 namespace {
 
@@ -174,6 +175,100 @@ __global__ __launch_bounds__(BLOCK) void k_row_prg(const u32 *__restrict__ seed,
     out[r * out_stride + k] = raw >= 0xFFFFFFFF00000001ull ? raw - 0xFFFFFFFF00000001ull : raw;
 }
 
+// The test-combiner challenge of the protocol (prover/protocol.py:127-135, device twin
+// prover/kernels/gl_spmv.cuh:46-70):
+//   challenge(seed, cid, label) = le128(BLAKE3(seed[32] || label || cid_le8)[0:16]) mod p.
+// label has at most 8 bytes, so the message is one block; `tail` holds label || cid packed into
+// the 16 bytes that follow the seed.
+struct ChallengeKey {
+    u32 seed[8];
+    int label_len;
+    u64 label;                 // label bytes as a little-endian integer
+};
+
+__device__ __forceinline__ ChallengeKey load_key(const u32 *__restrict__ seed, const unsigned char *__restrict__ label, int label_len) {
+    ChallengeKey k;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) k.seed[i] = seed[i];
+    k.label_len = label_len;
+    k.label = 0;
+    for (int i = 0; i < label_len; ++i) k.label |= (u64)label[i] << (8 * i);
+    return k;
+}
+
+__device__ __forceinline__ u64 challenge(const ChallengeKey &k, u64 cid) {
+    u32 m[16], cv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { m[i] = k.seed[i]; cv[i] = IV[i]; }
+    const int sh = 8 * k.label_len;                      // 0 .. 64 bits of label before the cid
+    const u64 lo = sh == 64 ? k.label : (k.label | (cid << sh));
+    const u64 hi = sh == 0 ? 0 : (sh == 64 ? cid : (cid >> (64 - sh)));
+    m[8] = (u32)lo;  m[9] = (u32)(lo >> 32);
+    m[10] = (u32)hi; m[11] = (u32)(hi >> 32);
+    m[12] = m[13] = m[14] = m[15] = 0;
+    compress(cv, m, 0, (u32)(40 + k.label_len), CHUNK_START | CHUNK_END | ROOT);
+    return gl::reduce128(((u64)cv[1] << 32) | cv[0], ((u64)cv[3] << 32) | cv[2]);
+}
+
+// out[i] = challenge(seed, cids ? cids[i] : i, label)      (challenge_vec / challenge_at)
+__global__ __launch_bounds__(BLOCK) void k_challenge(const u32 *__restrict__ seed, const unsigned char *__restrict__ label, int label_len,
+                                                     const u64 *__restrict__ cids, i64 n, u64 *__restrict__ out) {
+    const ChallengeKey key = load_key(seed, label, label_len);
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) out[i] = challenge(key, cids ? cids[i] : (u64)i);
+}
+
+// CSR matrix times vector over the field (prover/kernels/gl_spmv.cuh:25-41, 72-92):
+//   y[i] = sum_{p in row i} values[p] * x[col_idx[p]],   x[c] = challenge(seed, c, label) when x is null.
+// WAVE = false: one thread per row (rows of a few entries).  WAVE = true: one wavefront per row, lanes
+// stride over the row so that values and column indices are read coalesced, then a shuffle reduction.
+template <bool WAVE>
+__global__ __launch_bounds__(BLOCK) void k_spmv(const u64 *__restrict__ values, const u64 *__restrict__ col_idx,
+                                                const u64 *__restrict__ row_ptr, const u64 *__restrict__ x, const u32 *__restrict__ seed,
+                                                const unsigned char *__restrict__ label, int label_len, i64 n_rows,
+                                                u64 *__restrict__ y) {
+    ChallengeKey key;
+    if (!x) key = load_key(seed, label, label_len);
+    const i64 gid = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    const i64 n_workers = ((i64)gridDim.x * BLOCK) >> (WAVE ? 6 : 0);
+    const int lane = WAVE ? (threadIdx.x & 63) : 0;
+    for (i64 row = WAVE ? (gid >> 6) : gid; row < n_rows; row += n_workers) {
+        const u64 start = row_ptr[row], end = row_ptr[row + 1];
+        u64 acc = 0;
+        for (u64 p = start + lane; p < end; p += WAVE ? 64 : 1) {
+            const u64 c = col_idx[p];
+            acc = gl::add(acc, gl::mul(values[p], x ? x[c] : challenge(key, c)));
+        }
+        if (WAVE) {
+            for (int off = 32; off > 0; off >>= 1) acc = gl::add(acc, __shfl_xor(acc, off, 64));
+            if (lane == 0) y[row] = acc;
+        } else {
+            y[row] = acc;
+        }
+    }
+}
+
+// LogUp multiplicities (prover/kernels/gl_extras.cuh:118-150): mult[j] += 1 for the first j with
+// table[j] == x[i]; values that are not in the table count nowhere.  t_len_range > 0 says the
+// table is literally 0 .. t_len_range-1, so x[i] is its own index.
+__global__ __launch_bounds__(BLOCK) void k_lookup_mult(const u64 *__restrict__ x, i64 n_x, const u64 *__restrict__ table, i64 n_table,
+                                                       i64 t_len_range, unsigned long long *__restrict__ mult) {
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n_x; i += stride) {
+        const u64 xi = x[i];
+        if (t_len_range > 0) {
+            if (xi < (u64)t_len_range) atomicAdd(&mult[xi], 1ULL);
+            continue;
+        }
+        for (i64 j = 0; j < n_table; ++j) {
+            if (table[j] == xi) {
+                atomicAdd(&mult[j], 1ULL);
+                break;
+            }
+        }
+    }
+}
+
 inline i64 chunks_of(i64 m) { return m <= 0 ? 1 : (m + ROWS_PER_CHUNK - 1) / ROWS_PER_CHUNK; }
 
 }  // namespace
@@ -267,6 +362,63 @@ int vi_row_prg(const uint8_t *seed, const uint64_t *row_indices, int64_t row_off
     hipLaunchKernelGGL(k_row_prg, dim3((unsigned)blocks), dim3(BLOCK), 0, (hipStream_t)stream, (const u32 *)seed, row_indices,
                        (u32)row_offset, (i64)n_rows, (i64)slack, out, (i64)out_stride);
     VI_LAUNCH_CHECK("k_row_prg");
+    return VI_OK;
+}
+
+namespace {
+int check_key(const char *who, const uint8_t *seed, const uint8_t *label, int label_len) {
+    if (!seed || ((uintptr_t)seed & 3)) return vi::fail(VI_EINVAL, "%s: seed must be a 4-byte aligned device pointer", who);
+    if (label_len < 0 || label_len > 8 || (label_len > 0 && !label)) return vi::fail(VI_EINVAL, "%s: label of %d bytes (0 .. 8)", who, label_len);
+    return VI_OK;
+}
+inline unsigned capped_grid(i64 work_items) {
+    i64 b = (work_items + BLOCK - 1) / BLOCK;
+    return (unsigned)(b < 1 ? 1 : (b > 256 * 32 ? 256 * 32 : b));
+}
+}  // namespace
+
+int vi_challenge(const uint8_t *seed, const uint8_t *label, int label_len, const uint64_t *cids, int64_t n, uint64_t *out,
+                 void *stream) {
+    int rc = check_key("vi_challenge", seed, label, label_len);
+    if (rc) return rc;
+    if (n < 0) return vi::fail(VI_EINVAL, "vi_challenge: n = %lld", (long long)n);
+    if (n == 0) return VI_OK;
+    if (!out) return vi::fail(VI_EINVAL, "vi_challenge: null out");
+    hipLaunchKernelGGL(k_challenge, dim3(capped_grid(n)), dim3(BLOCK), 0, (hipStream_t)stream, (const u32 *)seed, label, label_len,
+                       cids, (i64)n, out);
+    VI_LAUNCH_CHECK("k_challenge");
+    return VI_OK;
+}
+
+int vi_gl_spmv(const uint64_t *values, const uint64_t *col_idx, const uint64_t *row_ptr, int64_t n_rows, int64_t nnz,
+               const uint64_t *x, const uint8_t *seed, const uint8_t *label, int label_len, uint64_t *y, void *stream) {
+    if (n_rows < 0 || nnz < 0) return vi::fail(VI_EINVAL, "vi_gl_spmv: n_rows = %lld, nnz = %lld", (long long)n_rows, (long long)nnz);
+    if (!x) {
+        int rc = check_key("vi_gl_spmv", seed, label, label_len);
+        if (rc) return rc;
+    }
+    if (n_rows == 0) return VI_OK;
+    if (!row_ptr || !y || (nnz > 0 && (!values || !col_idx))) return vi::fail(VI_EINVAL, "vi_gl_spmv: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (nnz / n_rows >= 32) {
+        hipLaunchKernelGGL(k_spmv<true>, dim3(capped_grid(n_rows * 64)), dim3(BLOCK), 0, s, values, col_idx, row_ptr, x, (const u32 *)seed,
+                           label, label_len, (i64)n_rows, y);
+    } else {
+        hipLaunchKernelGGL(k_spmv<false>, dim3(capped_grid(n_rows)), dim3(BLOCK), 0, s, values, col_idx, row_ptr, x, (const u32 *)seed,
+                           label, label_len, (i64)n_rows, y);
+    }
+    VI_LAUNCH_CHECK("k_spmv");
+    return VI_OK;
+}
+
+int vi_lookup_multiplicities(const uint64_t *x, int64_t n_x, const uint64_t *table, int64_t n_table, int table_is_range,
+                             uint64_t *mult, void *stream) {
+    if (n_x < 0 || n_table < 0) return vi::fail(VI_EINVAL, "vi_lookup_multiplicities: n_x = %lld, n_table = %lld", (long long)n_x, (long long)n_table);
+    if (n_x == 0 || n_table == 0) return VI_OK;
+    if (!x || !mult || (!table_is_range && !table)) return vi::fail(VI_EINVAL, "vi_lookup_multiplicities: null pointer");
+    hipLaunchKernelGGL(k_lookup_mult, dim3(capped_grid(n_x)), dim3(BLOCK), 0, (hipStream_t)stream, x, (i64)n_x, table, (i64)n_table,
+                       (i64)(table_is_range ? n_table : 0), (unsigned long long *)mult);
+    VI_LAUNCH_CHECK("k_lookup_mult");
     return VI_OK;
 }
 

@@ -575,3 +575,122 @@ def merkle_build_blake3(leaves):
         levels.append(cur)
     root = levels[-1].view(-1)[:32].clone()
     return root, levels
+
+
+# ---- combiner challenges, CSR matvec, LogUp multiplicities (prover/cuda_primitives.py:512-592, 1008-1052) ----
+
+def _check_key(seed, label):
+    if not (isinstance(seed, torch.Tensor) and seed.is_cuda and seed.dtype == torch.uint8 and seed.numel() == 32
+            and seed.is_contiguous()):
+        raise RuntimeError("seed must be a 32-byte CUDA uint8 tensor")
+    if not (isinstance(label, torch.Tensor) and label.is_cuda and label.dtype == torch.uint8 and label.numel() <= 8
+            and label.is_contiguous()):
+        raise RuntimeError("label must be a CUDA uint8 tensor of <= 8 bytes")
+
+
+def challenge_at(seed, label, cids):
+    """challenge(seed, cid, label) for an arbitrary cid tensor (uint64, any shape):
+    int.from_bytes(BLAKE3(seed || label || cid_le8)[:16], "little") % P
+    (prover/cuda_primitives.py:1233-1237, prover/protocol.py:127-135)."""
+    _check_key(seed, label)
+    if not (isinstance(cids, torch.Tensor) and cids.is_cuda and cids.dtype == torch.uint64):
+        raise RuntimeError("cids must be a CUDA uint64 tensor")
+    cc = cids.contiguous()
+    n = int(cc.numel())
+    if n >= (1 << 31):
+        raise RuntimeError("challenge_at: too many cids")
+    out = torch.empty_like(cc)
+    if n:
+        _lib.check(_lib.lib().vi_challenge(seed.data_ptr(), label.data_ptr(), int(label.numel()), cc.data_ptr(), n,
+                                           out.data_ptr(), _lib.stream_ptr()))
+    return out
+
+
+def challenge_vec(seed, label, n):
+    """r[i] = challenge(seed, i, label) for i in [0, n) on the device
+    (prover/cuda_primitives.py:1240-1248)."""
+    n = int(n)
+    if n == 0:
+        return torch.empty(0, dtype=torch.uint64, device="cuda")
+    _check_key(seed, label)
+    if n < 0 or n >= (1 << 31):
+        raise RuntimeError("challenge_vec n must be in [0, 2^31)")
+    out = torch.empty(n, dtype=torch.uint64, device=seed.device)
+    _lib.check(_lib.lib().vi_challenge(seed.data_ptr(), label.data_ptr(), int(label.numel()), None, n, out.data_ptr(),
+                                       _lib.stream_ptr()))
+    return out
+
+
+def _spmv(values, col_idx, row_ptr, n_rows, x, seed, label):
+    for t, name in ((values, "values"), (col_idx, "col_idx"), (row_ptr, "row_ptr")):
+        _check_u64(t, name)
+        if t.dim() != 1:
+            raise RuntimeError(f"{name} must be 1-D")
+    n_rows = int(n_rows)
+    if int(row_ptr.size(0)) != n_rows + 1:
+        raise RuntimeError("row_ptr length must be n_rows + 1")
+    if int(values.numel()) != int(col_idx.numel()):
+        raise RuntimeError("values and col_idx must have one entry per non-zero")
+    y = torch.empty(n_rows, dtype=torch.uint64, device=values.device)
+    if n_rows:
+        _lib.check(_lib.lib().vi_gl_spmv(values.data_ptr(), col_idx.data_ptr(), row_ptr.data_ptr(), n_rows, int(values.numel()),
+                                         x.data_ptr() if x is not None else None,
+                                         seed.data_ptr() if seed is not None else None,
+                                         label.data_ptr() if label is not None else None,
+                                         int(label.numel()) if label is not None else 0, y.data_ptr(), _lib.stream_ptr()))
+    return y
+
+
+def gl_spmv(values, col_idx, row_ptr, x, n_rows):
+    """CSR mod-P matvec; row_ptr length must be n_rows + 1 (prover/cuda_primitives.py:1192-1194)."""
+    _check_u64(x, "x")
+    if x.dim() != 1:
+        raise RuntimeError("x must be 1-D")
+    return _spmv(values, col_idx, row_ptr, n_rows, x, None, None)
+
+
+def gl_spmv_challenged(values, col_idx, row_ptr, seed, label, n_rows):
+    """CSR mod-P matvec whose combiner x[cid] = challenge(seed, cid, label) is computed in place
+    (prover/cuda_primitives.py:1197-1202)."""
+    _check_key(seed, label)
+    return _spmv(values, col_idx, row_ptr, n_rows, None, seed, label)
+
+
+_range_table_cache: dict = {}
+
+
+def _is_range_table(table):
+    """One probe per table tensor: is table[i] == i for all i?  Cached by storage address and
+    length, as the reference does (tables are immutable once built, cuda_primitives.py:1411-1423)."""
+    key = (table.data_ptr(), table.numel())
+    if key not in _range_table_cache:
+        ref = torch.arange(table.numel(), dtype=torch.int64, device=table.device).view(torch.uint64)
+        _range_table_cache[key] = bool(torch.equal(table, ref))
+    return _range_table_cache[key]
+
+
+def lookup_multiplicities_into(x, table, mult, label=""):
+    """In-place mult[j] += #{i : x[i] == table[j]}; values outside the table count nowhere
+    (prover/cuda_primitives.py:1431-1446).  A table that is literally 0 .. T-1 is indexed directly."""
+    _check_u64(x, "x")
+    _check_u64(table, "table")
+    _check_u64(mult, "mult")
+    if x.dim() != 1 or table.dim() != 1 or mult.dim() != 1:
+        raise RuntimeError("x, table and mult must be 1-D")
+    if mult.numel() != table.numel():
+        raise RuntimeError("mult length must match table")
+    if x.numel() == 0 or table.numel() == 0:
+        return
+    _lib.check(_lib.lib().vi_lookup_multiplicities(x.data_ptr(), int(x.numel()), table.data_ptr(), int(table.numel()),
+                                                   1 if _is_range_table(table) else 0, mult.data_ptr(), _lib.stream_ptr()))
+
+
+def lookup_multiplicities(x, table):
+    """Per-table-entry multiplicity histogram (prover/cuda_primitives.py:1426-1428)."""
+    _check_u64(x, "x")
+    _check_u64(table, "table")
+    mult = torch.zeros(int(table.numel()), dtype=torch.int64, device=table.device).view(torch.uint64)
+    if x.dim() != 1 or table.dim() != 1:
+        raise RuntimeError("x and table must be 1-D")
+    lookup_multiplicities_into(x, table, mult)
+    return mult
