@@ -1,17 +1,24 @@
-"""Drop-in for the field / NTT / Reed-Solomon part of the reference's
-`prover/cuda_primitives.py` on MI355X.
+"""Drop-in for the reference's `prover/cuda_primitives.py` on MI355X.
 
 Same public names, argument conventions and error behaviour
-(prover/cuda_primitives.py:1-41, 198-456, 1086-1183): every function works on
-contiguous `torch.uint64` tensors that live on the GPU ("cuda" is ROCm's device
-name in PyTorch), binary ops want equal shapes and return a new tensor, the NTTs
-are in place and return None, violations raise RuntimeError.  Underneath, each
-call is one ctypes hop into libverinf_hip.so on torch's current stream; nothing
-is JIT-compiled and there is no CPU fallback.
+(prover/cuda_primitives.py:1-41, 198-1446): every function works on contiguous
+`torch.uint64` (hashes: `torch.uint8`) tensors that live on the GPU ("cuda" is
+ROCm's device name in PyTorch), binary ops want equal shapes and return a new
+tensor, the NTTs are in place and return None, violations raise RuntimeError.
+Underneath, each call is one ctypes hop into libverinf_hip.so on torch's current
+stream; nothing is JIT-compiled and there is no CPU fallback.
+
+Covered: field ops, NTTs, Reed-Solomon / coset encoding, polynomial helpers,
+gl_matmul / gl_matvec / gl_spmv[_challenged], challenge_vec / challenge_at,
+hash_columns_streamed / MerkleColumnAccumulator / merkle_build_blake3, row_prg[_indexed],
+lookup_multiplicities[_into].  Not provided: the `interp_band*` family.
 
 Additions over the reference surface:
   coset_lde(messages, k_deg, n_lig, shift)   the fused iNTT -> twist -> zero-extend -> NTT
+  coset_lde_with_coeffs(...)                 the same, also returning the row polynomials
+  coset_extend(coeffs, k_deg, n_lig, shift)  coefficients -> coset evaluations
   gl_mul_bcast(a, b_row)                     a * (b_row broadcast over rows) without materialising it
+  row_prg(..., out=)                         the pad written straight into a column slice
 """
 import torch
 
