@@ -29,9 +29,9 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 
 # HBM bytes per k_ntt_fast launch of the default LDE leg, averaged over the 16 launches of a step:
-# FETCH_SIZE and WRITE_SIZE read by rocprofv3 in two counter runs of this script (5.55 GB read +
+# FETCH_SIZE and WRITE_SIZE read by rocprofv3 in two counter runs of this script (5.48 GB read +
 # 6.01 GB written per step), each scaled by what the same counter reads for a 1 GiB device copy.
-LDE_TRAFFIC_BYTES_PER_LAUNCH = 722.6e6
+LDE_TRAFFIC_BYTES_PER_LAUNCH = 718.2e6
 
 
 def _events(torch):
