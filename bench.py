@@ -28,10 +28,11 @@ P = (1 << 64) - (1 << 32) + 1
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 
-# HBM bytes per k_ntt_fast launch of the default LDE leg, averaged over the 16 launches of a step:
-# FETCH_SIZE and WRITE_SIZE read by rocprofv3 in two counter runs of this script (5.48 GB read +
-# 6.01 GB written per step), each scaled by what the same counter reads for a 1 GiB device copy.
-LDE_TRAFFIC_BYTES_PER_LAUNCH = 718.2e6
+# HBM bytes of one step of the default LDE leg (all k_ntt_fast launches of the step together): FETCH_SIZE and
+# WRITE_SIZE read by rocprofv3 in two counter runs of this script (5.48 GB read + 6.01 GB written per step),
+# each scaled by what the same counter reads for a 1 GiB device copy.  roofline.traffic is this figure divided
+# by the launches of a step, like roofline.achieved.
+LDE_TRAFFIC_BYTES_PER_STEP = 11.49e9
 
 
 def _events(torch):
@@ -436,7 +437,7 @@ def main():
         "config": {"workload": "coset LDE 1024 rows x 2^16 -> 2^18, shift 7 (BASELINE configs[1])",
                    "rows": 1024, "K": 1 << 16, "N": 1 << 18},
         "roofline": {"bound": "hbm", "achieved": lde["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": LDE_TRAFFIC_BYTES_PER_LAUNCH,
+                     "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": LDE_TRAFFIC_BYTES_PER_STEP / lde["launches_per_step"],
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a copy probe "
                                        "(x2.000 / x1.000); not re-measured in this run",
                      "kernel": "k_ntt_fast", "launches_per_step": lde["launches_per_step"],

@@ -254,10 +254,10 @@ size_t vi_coset_lde_min_workspace_bytes(int64_t K, int64_t N) {
 size_t vi_coset_lde_workspace_bytes(int64_t m, int64_t K, int64_t N) {
     size_t one = vi_coset_lde_min_workspace_bytes(K, N);
     if (!one || m <= 0) return 0;
-    // The passes are bound by integer VALU work, not by HBM, so what matters is that a
-    // launch holds many workgroups per CU (no partially filled last round): measured on
-    // 1024 x 2^16 -> 2^18, 20 / 80 / 320 / 640 MiB of scratch give 9.7 / 4.5 / 3.8 / 3.7 ms.
-    const size_t target = (size_t)640 << 20;
+    // A launch should hold many workgroups per CU (no partially filled last round) and the chunk count should be
+    // low: measured on 1024 x 2^16 -> 2^18, 80 / 160 / 320 / 640 / 1280 / 2560 MiB of scratch give
+    // 4.87 / 4.09 / 3.85 / 3.64 / 3.57 / 3.63 ms.  1.25 GiB is small change next to 288 GB of HBM.
+    const size_t target = (size_t)1280 << 20;
     size_t rows = target / one;
     if (rows < 8) rows = 8;
     if ((int64_t)rows > m) rows = (size_t)m;
