@@ -174,10 +174,14 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, const u
             const int sh = A.is_final ? 0 : A.logR;
             const int t = A.is_final ? R.t : t_loop;
             const u64 *pre = A.pre + ((i64)t << A.logn) + R.idx_base;
+            // all sixteen multipliers are requested at once (they arrive while the data loads are still in flight)
+            u64 pw[16];
+#pragma unroll
+            for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[(i64)((n1 << A2) + n2) << sh];
 #pragma unroll
             for (int g = 0; g < 16; g += 4) {
 #pragma unroll
-                for (int n1 = g; n1 < g + 4; ++n1) x[n1] = gl::mul(x[n1], pre[(i64)((n1 << A2) + n2) << sh]);
+                for (int n1 = g; n1 < g + 4; ++n1) x[n1] = gl::mul(x[n1], pw[n1]);
                 VI_SCHED_FENCE();
             }
         }
@@ -211,6 +215,12 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
     for (int i = 0; i < 16 / E2; ++i) {
         const int k1 = (tid + i * NTHREADS) >> lt;
         u64 x[E2];
+        // the inter-pass twiddles are requested before the LDS reads and the transform, which then cover their latency
+        u64 tw[E2];
+        if (!A.is_final && R.valid) {
+#pragma unroll
+            for (int k2 = 0; k2 < E2; ++k2) tw[k2] = A.tw[((i64)(k1 + 16 * k2) << A.logR) + R.tw_base];
+        }
 #pragma unroll
         for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
         VI_SCHED_FENCE();
@@ -222,7 +232,7 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
             const i64 k = k1 + 16 * k2;
             u64 v = x[k2];
             if (!A.is_final) {
-                v = gl::mul(v, A.tw[(k << A.logR) + R.tw_base]);
+                v = gl::mul(v, tw[k2]);
                 VI_STREAM_STORE(&A.dst[(i64)t_loop * A.dst_coset_stride + R.dst_base + (k << A.logR)], v);
             } else {
                 if (A.scale != 1) v = gl::mul(v, A.scale);
