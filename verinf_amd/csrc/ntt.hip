@@ -51,9 +51,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     __shared__ u64 lds[TILE + (16 << A2)];
     __shared__ u64 twi[16 << A2];
     const int tid = threadIdx.x;
-    const i64 tile = blockIdx.x;
-    // blockIdx.y = coset of a pass that expands one source tile into rho cosets; each of
-    // the rho workgroups of a tile re-reads it.  Measured alternatives, all slower:
+    // A pass that expands one source tile into rho cosets runs rho workgroups per tile, the coset being the low
+    // bits of the workgroup id, so that the workgroups that read the same coefficients run at about the same time
+    // (3.394 vs 3.420 ms against the coset as grid.y); each of them re-reads the tile.  Measured alternatives, all slower:
     //  * a loop over the cosets inside one workgroup: every address becomes loop-invariant,
     //    ~50 more live registers, spills;
     //  * persistent workgroups prefetching the next tile into a second register buffer: -3 %;
@@ -61,7 +61,10 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     //  * workgroup ids laid out so that the cosets of a tile share an XCD and its L2 (ids 8
     //    apart): fetch traffic of the pass drops from 537 to 134 MB per 256 rows, run time
     //    rises 2.6 % -- the pass is bound by integer VALU issue, not by HBM.
-    const int t = blockIdx.y;
+    const bool expand = !A.is_final && A.loop_cosets;
+    const i64 tile = expand ? (i64)(blockIdx.x >> A.log_rho) : (i64)blockIdx.x;
+    const i64 n_tiles = expand ? (i64)(gridDim.x >> A.log_rho) : (i64)gridDim.x;
+    const int t = expand ? (int)(blockIdx.x & ((1u << A.log_rho) - 1)) : 0;
     u64 reg[16];
     fast_load<A2>(A, tile, tid, reg);
     // Warm the L2 for a workgroup that will run on this XCD a little later: after its own loads (loads return in
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     // later loads that tile finds it in the L2 instead of waiting on HBM.  Measured on 1024 x 2^16 -> 2^18 with
     // streaming stores: no touch 3.96 ms, distance 256 / 384 / 448 / 512 / 768 / 1024 tiles -> 3.75 / 3.63 / 3.56 /
     // 3.58 / 3.79 / 3.87 ms (about 1024 workgroups are resident; further ahead and the lines are evicted before use).
-    const u64 touched = fast_touch<A2>(A, tile + TOUCH_AHEAD, (i64)gridDim.x, tid);
+    const u64 touched = fast_touch<A2>(A, tile + (expand ? (TOUCH_AHEAD >> A.log_rho) : TOUCH_AHEAD), n_tiles, tid);
     if (!A.is_final) {
         // strided pass: a wavefront uses only the table rows of its own n2 values (at most 64 words), so each
         // wavefront fills just those and no workgroup barrier is needed before stage 1
@@ -185,7 +188,7 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
         if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
         dim3 grid((unsigned)tiles), block(NTHREADS);
         if (fast_ok(A.a) && A.twi) {
-            if (!A.is_final && A.loop_cosets) grid.y = 1u << A.log_rho;
+            if (!A.is_final && A.loop_cosets) grid.x <<= A.log_rho;       // tiles * rho <= 2^31 by max_rows_per_launch
             switch ((A.a - FAST_A1) * 2 + (A.inverse ? 1 : 0)) {
                 case 2: hipLaunchKernelGGL((k_ntt_fast<1, false>), grid, block, 0, s, A); break;
                 case 3: hipLaunchKernelGGL((k_ntt_fast<1, true>), grid, block, 0, s, A); break;
