@@ -1,0 +1,93 @@
+"""GPU parity on seeded random shapes: the same bit-exact comparisons as the targeted tests, over
+combinations of sizes, widths, pitches and row counts that nobody picked by hand."""
+import random
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+from oracle import oracle as O  # noqa: E402
+from tests.gpu_util import P, rand_field, to_dev, to_np  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def cp():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from verinf_amd.prover import cuda_primitives
+    return cuda_primitives
+
+
+def test_lde_random_geometries(cp):
+    rng = random.Random(2024)
+    for case in range(40):
+        logK = rng.randint(1, 15)
+        logN = rng.randint(logK, min(logK + 5, 17))
+        K, N = 1 << logK, 1 << logN
+        m = rng.choice([1, 2, 3, 5, 17, 64, 130]) if logN <= 14 else rng.choice([1, 2, 3, 5])
+        w = rng.choice([K, rng.randint(1, K), max(1, K // 2)])
+        pitch = w + rng.choice([0, 0, 1, 7, 64])
+        shift = rng.choice([7, 1, rng.randrange(2, P)])
+        big = rand_field((m, pitch), 1000 + case)
+        view = to_dev(big).view(torch.int64)[:, :w].view(torch.uint64)
+        want = O.coset_lde_rows(np.ascontiguousarray(big[:, :w]), K, N, shift)
+        got = cp.coset_lde(view, K, N, shift)
+        assert np.array_equal(to_np(got), want), (case, logK, logN, m, w, pitch, shift)
+        co, code = cp.coset_lde_with_coeffs(view, K, N, shift)
+        assert torch.equal(code, got), (case, "with_coeffs")
+        assert torch.equal(cp.coset_extend(co, K, N, shift), got), (case, "extend")
+
+
+def test_ntt_random_sizes_round_trip_and_oracle(cp):
+    rng = random.Random(7)
+    for case in range(25):
+        logn = rng.randint(1, 18)
+        m = rng.choice([1, 2, 3, 9, 33]) if logn <= 15 else rng.choice([1, 2])
+        a = rand_field((m, 1 << logn), 2000 + case)
+        rows = to_dev(a)
+        cp.ntt_forward_batched(rows)
+        assert np.array_equal(to_np(rows), O.ntt_rows(a)), (case, logn, m)
+        cp.ntt_inverse_batched(rows)
+        assert np.array_equal(to_np(rows), a), (case, logn, m, "inverse")
+
+
+def test_hash_random_shapes_and_slabs(cp):
+    rng = random.Random(11)
+    for case in range(30):
+        m = rng.choice([1, 2, 127, 128, 129, 255, 256, 257, rng.randint(1, 3000)])
+        n = rng.choice([1, 2, 63, 64, 65, 255, 256, 257, rng.randint(1, 1500)])
+        pitch = n + rng.choice([0, 0, 3, 64])
+        big = rand_field((m, pitch), 3000 + case)
+        dev = to_dev(big).view(torch.int64)[:, :n].view(torch.uint64)
+        want = O.hash_columns(np.ascontiguousarray(big[:, :n]))
+        assert np.array_equal(to_np(cp.hash_columns_streamed(dev)), want), (case, m, n, pitch)
+        if m > 128:
+            acc = cp.MerkleColumnAccumulator(n, m)
+            r = 0
+            while r < m:
+                k = min(m - r, rng.choice([1, 50, 128, 129, 300, 1024]))
+                acc.update(dev[r:r + k])
+                r += k
+            assert np.array_equal(to_np(acc.finalize()), want), (case, m, n, "accumulator")
+        root, levels = cp.merkle_build_blake3(to_dev(want))
+        assert to_np(root).tobytes() == O.merkle_levels(want)[-1][0].tobytes(), (case, "root")
+
+
+def test_sumcheck_random_term_structures():
+    from verinf_amd.layergkr import gpu
+    rng = random.Random(5)
+    for case in range(25):
+        v = rng.randint(1, 14)
+        n_tables = rng.randint(1, 12)
+        n_terms = rng.randint(1, 5)
+        terms_idx = [(rng.randrange(P), [rng.randrange(n_tables) for _ in range(rng.randint(1, 4))]) for _ in range(n_terms)]
+        tabs = [rand_field((1 << v,), 4000 + 20 * case + j) for j in range(n_tables)]
+        dev = [to_dev(t) for t in tabs]
+        coins = [rng.randrange(P) for _ in range(v)]
+        claim, polys, chal, _ = gpu.prove_terms_gpu([(c, [dev[i] for i in idx]) for c, idx in terms_idx], lambda i: coins[i], P)
+        want_claim, want_samples, _ = O.sumcheck_prove(tabs, terms_idx, coins)
+        deg = max(len(idx) for _, idx in terms_idx)
+        assert claim == want_claim, (case, v, terms_idx)
+        assert [[y for _, y in s] for s in polys] == [list(s[: deg + 1]) for s in want_samples], (case, v, terms_idx)
+        assert chal == coins
