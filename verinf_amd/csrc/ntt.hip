@@ -58,13 +58,18 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     //    ~50 more live registers, spills;
     //  * persistent workgroups prefetching the next tile into a second register buffer: -3 %;
     //  * two tiles per workgroup with both tiles' loads issued up front: -6 % (128 registers, spills);
-    //  * workgroup ids laid out so that the cosets of a tile share an XCD and its L2 (ids 8
-    //    apart): fetch traffic of the pass drops from 537 to 134 MB per 256 rows, run time
-    //    rises 2.6 % -- the pass is bound by integer VALU issue, not by HBM.
     const bool expand = !A.is_final && A.loop_cosets;
-    const i64 tile = expand ? (i64)(blockIdx.x >> A.log_rho) : (i64)blockIdx.x;
     const i64 n_tiles = expand ? (i64)(gridDim.x >> A.log_rho) : (i64)gridDim.x;
-    const int t = expand ? (int)(blockIdx.x & ((1u << A.log_rho) - 1)) : 0;
+    i64 tile = expand ? (i64)(blockIdx.x >> A.log_rho) : (i64)blockIdx.x;
+    int t = expand ? (int)(blockIdx.x & ((1u << A.log_rho) - 1)) : 0;
+    if (expand && (n_tiles & 7) == 0) {
+        // Workgroup ids are dealt to the 8 XCDs in turn.  Taking the XCD from the low three id bits and (tile, coset)
+        // from the rest puts the rho workgroups of a tile on consecutive slots of ONE XCD, so that all but the first
+        // find the coefficients in that XCD's L2 (3.46-3.50 vs 3.49-3.53 ms).  A bijection of [0, 8 * n_tiles/8 * rho).
+        const u32 xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        t = (int)(slot & ((1u << A.log_rho) - 1));
+        tile = (i64)(slot >> A.log_rho) * 8 + xcd;
+    }
     u64 reg[16];
     fast_load<A2>(A, tile, tid, reg);
     // Warm the L2 for a workgroup that will run on this XCD a little later: after its own loads (loads return in
