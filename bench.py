@@ -29,10 +29,10 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 
 # HBM bytes of one step of the default LDE leg (all k_ntt_fast launches of the step together): FETCH_SIZE and
-# WRITE_SIZE read by rocprofv3 in two counter runs of this script (5.48 GB read + 6.01 GB written per step),
+# WRITE_SIZE read by rocprofv3 in two counter runs of this script (3.80 GB read + 5.77 GB written per step),
 # each scaled by what the same counter reads for a 1 GiB device copy.  roofline.traffic is this figure divided
 # by the launches of a step, like roofline.achieved.
-LDE_TRAFFIC_BYTES_PER_STEP = 11.49e9
+LDE_TRAFFIC_BYTES_PER_STEP = 9.57e9
 
 
 def _events(torch):
