@@ -3,12 +3,12 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 One "step" = one pass of the hot path over one batch of synthetic input: the coset
-low-degree extension of 1024 seeded rows of 2^16 field elements to 2^18 (BASELINE
-configs[1]), input and output resident in HBM.  Prints ONE JSON line with the
+low-degree extension of 1024 seeded rows of 2^16 field elements to 2^18 (the second of the
+benchmark configurations), input and output resident in HBM.  Prints ONE JSON line with the
 metric (output elements per second), the roofline of the dominant kernel and a CPU
 baseline (the C oracle on the host cores, bounded sample, same inputs, outputs
-compared bit for bit with the GPU's).  The sumcheck (config 4) and K-quant
-(config 3) rates of the same run are reported under "extra".
+compared bit for bit with the GPU's).  The sumcheck, K-quant, column-hash and
+Llama-2-7B-layer legs of the same run are reported under "extra".
 
     python bench.py --copy-probe      plain device copy of known size (calibrates the
                                       FETCH_SIZE / WRITE_SIZE counters, see profiles/)

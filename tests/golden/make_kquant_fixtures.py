@@ -7,7 +7,7 @@ evaluated with `fractions.Fraction` and rounded to binary32 by an explicit
 round-to-nearest-even routine, so the fixture depends on no floating-point
 hardware, on no numpy, on the C oracle or on upstream code.
 
-Blocks: seeded random blocks in the shape BASELINE config 3 names (scale/quant
+Blocks: seeded random blocks in the shape of the K-quant benchmark workload (scale/quant
 bytes uniform, d and dmin = fp16(|N(0, 0.01)|)), plus hand-made blocks that hit
 d = 0, fp16 subnormals, the largest fp16, exact-integer cases and exact .5 ties.
 

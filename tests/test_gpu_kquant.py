@@ -25,7 +25,7 @@ def kq():
 
 
 def synth_blocks(qtype, nb, seed):
-    """BASELINE config 3 recipe: scale / quant bytes uniform, d and dmin = fp16(|N(0, 0.01)|)."""
+    """The K-quant benchmark recipe: scale / quant bytes uniform, d and dmin = fp16(|N(0, 0.01)|)."""
     rng = np.random.default_rng(seed)
     bb = O.BLOCK_BYTES[qtype]
     raw = rng.integers(0, 256, size=(nb, bb), dtype=np.uint8)
@@ -81,7 +81,7 @@ def test_kquant_errors(kq):
 
 
 def test_kquant_baseline_shape(kq):
-    """BASELINE config 3: a 4096 x 11008 Q4_K matrix (176,128 super-blocks), whole output
+    """The K-quant benchmark workload: a 4096 x 11008 Q4_K matrix (176,128 super-blocks), whole output
     against the C oracle."""
     nb = 4096 * 11008 // 256
     raw = synth_blocks("Q4_K", nb, 3)

@@ -52,7 +52,7 @@ def test_batched_ntt_matches_oracle(cp, logn, m):
 
 
 def test_config1_plumbing(cp):
-    """BASELINE config 1: 16 x 2^12 (seed 0), forward, inverse, then LDE to 2^14 with shift 7."""
+    """The small plumbing workload: 16 x 2^12 (seed 0), forward, inverse, then LDE to 2^14 with shift 7."""
     a = rand_field((16, 1 << 12), 0)
     rows = to_dev(a)
     cp.ntt_forward_batched(rows)
@@ -214,7 +214,7 @@ def test_lde_gates_and_layergkr_entry_points():
 
 
 def test_lde_full_baseline_shape_properties(cp):
-    """BASELINE config 2 shape (1024 x 2^16 -> 2^18): bit-exact against the oracle on a
+    """The headline LDE shape (1024 x 2^16 -> 2^18): bit-exact against the oracle on a
     row sample, codeword property (inverse transform has no coefficient >= K) on all rows."""
     K, N, m = 1 << 16, 1 << 18, 1024
     g = torch.Generator(device="cuda").manual_seed(2)
