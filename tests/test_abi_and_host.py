@@ -38,12 +38,14 @@ def test_library_exports_every_declared_symbol(L):
 
 
 def test_size_queries_and_argument_validation_without_a_device(L):
-    assert L.vi_ntt_workspace_bytes(4, 1 << 12) == 0
+    assert L.vi_ntt_workspace_bytes(4, 1 << 9) == 0
+    assert L.vi_ntt_workspace_bytes(4, 1 << 12) == 4 * (1 << 12) * 8
     assert L.vi_ntt_workspace_bytes(4, 1 << 16) == 4 * (1 << 16) * 8
     assert L.vi_ntt_workspace_bytes(4, 12) == 0
     one = L.vi_coset_lde_min_workspace_bytes(1 << 16, 1 << 18)
     assert one == (1 << 16) * 8 * 5
-    assert L.vi_coset_lde_min_workspace_bytes(1 << 10, 1 << 12) == (1 << 10) * 8
+    assert L.vi_coset_lde_min_workspace_bytes(1 << 10, 1 << 12) == (1 << 10) * 8 * 5
+    assert L.vi_coset_lde_min_workspace_bytes(1 << 8, 1 << 10) == (1 << 8) * 8
     assert L.vi_coset_lde_workspace_bytes(1024, 1 << 16, 1 << 18) % one == 0
     assert L.vi_coset_lde_min_workspace_bytes(24, 96) == 0
     assert L.vi_sumcheck_workspace_bytes() > 0

@@ -74,7 +74,7 @@ def test_device_inverse_chain(emu):
     assert emu.emu_inv(P + 5) == pow(5, P - 2, P)
 
 
-@pytest.mark.parametrize("logn,m", [(1, 3), (2, 5), (4, 300), (5, 9), (6, 7), (7, 70), (8, 33), (10, 5), (12, 3),
+@pytest.mark.parametrize("logn,m", [(1, 3), (2, 5), (4, 300), (5, 9), (6, 7), (7, 70), (8, 33), (9, 6), (10, 5), (11, 4), (12, 3),
                                     (13, 2), (14, 3), (15, 2), (16, 2), (17, 1), (18, 1), (19, 1)])
 def test_ntt_passes_match_oracle(emu, logn, m):
     a = _rand((m, 1 << logn), 100 + logn)
@@ -100,7 +100,8 @@ def test_ntt_25_bit_split_is_well_formed(emu):
 
 @pytest.mark.parametrize("logK,logN,m,w", [(5, 6, 4, 16), (7, 8, 9, 64), (9, 10, 3, 256), (3, 5, 700, 8),
                                            (12, 14, 2, 4096), (13, 15, 2, 5000), (14, 16, 1, 8192),
-                                           (16, 18, 1, 65536), (10, 10, 3, 1000), (4, 7, 5, 11)])
+                                           (16, 18, 1, 65536), (10, 10, 3, 1000), (4, 7, 5, 11),
+                                           (10, 12, 5, 1024), (11, 13, 3, 2000), (11, 12, 2, 2048)])
 def test_lde_passes_match_oracle(emu, logK, logN, m, w):
     msgs = _rand((m, w), 200 + logK)
     want = O.coset_lde_rows(msgs, 1 << logK, 1 << logN, 7)

@@ -40,7 +40,7 @@ def test_ntt_small_sizes_match_definition(cp, n):
     assert to_np(x).tolist() == want
 
 
-@pytest.mark.parametrize("logn,m", [(1, 5), (3, 1000), (5, 77), (8, 33), (9, 9), (11, 5), (12, 16), (13, 3),
+@pytest.mark.parametrize("logn,m", [(1, 5), (3, 1000), (5, 77), (8, 33), (9, 9), (10, 6), (11, 5), (12, 16), (13, 3),
                                     (14, 8), (15, 8), (16, 8), (17, 2), (18, 3), (20, 2)])
 def test_batched_ntt_matches_oracle(cp, logn, m):
     a = rand_field((m, 1 << logn), 100 + logn)
@@ -133,7 +133,7 @@ def test_lde_golden(cp, golden_dir):
 
 
 @pytest.mark.parametrize("logK,logN,m,w", [(1, 1, 3, 2), (1, 3, 3, 1), (3, 5, 700, 8), (5, 6, 4, 16), (7, 8, 9, 64),
-                                           (9, 10, 3, 256), (10, 10, 3, 1000), (4, 7, 5, 11), (12, 14, 16, 4096),
+                                           (9, 10, 3, 256), (10, 10, 3, 1000), (10, 12, 7, 1024), (11, 13, 3, 2000), (4, 7, 5, 11), (12, 14, 16, 4096),
                                            (13, 15, 5, 5000), (14, 16, 9, 8192), (16, 18, 5, 65536),
                                            (16, 17, 3, 40000), (17, 19, 2, 1 << 17), (18, 20, 2, 200000), (20, 22, 1, 1 << 20),
                                            (8, 14, 3, 256), (12, 18, 2, 4000)])

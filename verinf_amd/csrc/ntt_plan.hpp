@@ -19,11 +19,12 @@ struct Split {
     int a[4];
 };
 
-// n <= 2^12 is a single in-LDS pass; above that the digits are as even as possible
-// and at most 2^MAX_A, largest first.
+// n < 2^10 is a single in-LDS pass; from 2^10 on the digits are as even as possible and at most
+// 2^MAX_A, largest first, so that every pass is a register-blocked one (2^10 .. 2^12 would fit a
+// single in-LDS pass, but two register-blocked passes are 1.5 x faster: 0.65 vs 1.0 ms for 2^26 points).
 inline Split split_digits(int logn) {
     Split s{};
-    if (logn <= TILE_LOG) { s.p = 1; s.a[0] = logn; return s; }
+    if (logn < 10) { s.p = 1; s.a[0] = logn; return s; }
     s.p = (logn + MAX_A - 1) / MAX_A;
     int base = logn / s.p, extra = logn % s.p;
     for (int q = 0; q < s.p; ++q) s.a[q] = base + (q < extra ? 1 : 0);
