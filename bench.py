@@ -373,8 +373,8 @@ def copy_probe(torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-rows", type=int, default=1024, help="rows of the CPU baseline sample")
     ap.add_argument("--cpu-reps", type=int, default=5, help="passes of the CPU baseline over its sample")
     ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
