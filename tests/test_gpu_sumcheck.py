@@ -77,6 +77,31 @@ def test_sum_of_products_shared_tables_and_coefficients(mods):
     _check(gpu, [eq, a, b, c], [(11, [0, 1, 2]), (P - 11, [0, 3]), (13, [0, 2, 2]), (P - 13, [0, 2])], 9, True)
 
 
+@pytest.mark.parametrize("name,nt,terms", [
+    # every term holds table 0: it is taken out as the common factor
+    ("common+products", 5, [(3, [0, 1, 2]), (P - 5, [0, 3, 4]), (7, [1, 0, 4])]),
+    # ... and what is left of a term may be one factor (linear part) or nothing (constant part)
+    ("common+linear+constant", 4, [(3, [0, 1, 2]), (P - 5, [0, 3]), (9, [0]), (P - 1, [2, 0]), (4, [0])]),
+    # the common table twice in one term: only one occurrence leaves the term
+    ("common squared", 3, [(6, [0, 0]), (P - 6, [0]), (2, [0, 0, 1]), (5, [2, 0])]),
+    # no table in every term: linear and product terms without a common factor
+    ("no common", 6, [(3, [0, 1]), (P - 5, [2]), (7, [3]), (11, [4, 5, 0]), (13, [1])]),
+    # affine / rescale relations only: every term linear after eq is taken out (layergkr/relations.py:68-82)
+    ("all linear", 7, [(3, [0, 1]), (P - 5, [0, 2]), (7, [0, 3]), (P - 1, [0, 4]), (2, [0, 5]), (P - 9, [0, 6])]),
+    # only linear terms and no common table: the round polynomial has degree 1
+    ("degree one", 3, [(3, [0]), (P - 5, [1]), (7, [2])]),
+    # two candidates for the common table
+    ("two common", 3, [(3, [0, 1, 2]), (5, [1, 0])]),
+])
+@pytest.mark.parametrize("v", [1, 5, 12])
+def test_factored_term_forms_match_oracle(mods, name, nt, terms, v):
+    """Sums of several terms are evaluated as common * (constant + linear part + products);
+    every such form against the oracle, which evaluates the terms as they are written."""
+    gpu, _ = mods
+    tabs = [rand_field(1 << v, 300 + 7 * v + j) for j in range(nt)]
+    _check(gpu, tabs, terms, 21 + v, as_tensor=True)
+
+
 def test_more_tables_than_fit_in_registers(mods):
     gpu, _ = mods
     r = random.Random(12)

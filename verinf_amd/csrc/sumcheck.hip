@@ -35,6 +35,16 @@ struct Desc {
     u64 coeff[VI_SC_MAX_TERMS];
     unsigned char term_off[VI_SC_MAX_TERMS + 1];
     unsigned char fidx[VI_SC_MAX_FACTORS];
+    // Several terms over tables a thread keeps in registers are stored factored:
+    //   S(x) = common(x) * ( c0 + sum_k lin_coeff[k] f_lin[k](x) + sum_k coeff[k] prod_j f_kj(x) )
+    // where `common` is a table every term contains (eq(z, .) in a batched gate check, layergkr/relations.py:117-121;
+    // -1 = none, the bracket alone), a term left without factors adds its coefficient to c0, a term left with one
+    // factor is linear in x (its coefficient is applied once per pair to the value and the step of that factor,
+    // not once per evaluation point), and coeff / term_off / fidx keep only the terms with two or more factors left.
+    u64 lin_coeff[VI_SC_MAX_TERMS];
+    unsigned char lin_idx[VI_SC_MAX_TERMS];
+    u64 c0;
+    int n_lin, common;
     int n_tables, n_terms, deg;
     int coeff_at_end;                       // single term: apply its coefficient in the final reduction
     int product;                            // one term whose factors are exactly the n_tables tables, once each
@@ -58,8 +68,9 @@ __device__ __forceinline__ u64 wave_sum(u64 v) {
 // need no second launch).
 // PROD: the sum is a single product of all NT tables (a matmul contraction, eq * a * b, the
 // three-factor benchmark instance): the term interpreter below -- scalar loads of the term
-// description and a select chain per factor -- gives way to a fully unrolled product.
-template <int NT, int MODE, int U, bool PROD>
+// description and a register picked by index per factor -- gives way to a fully unrolled product.
+// NS: evaluation points the general path keeps per pair (4 when the degree is at most 3, else NSAMP)
+template <int NT, int MODE, int U, bool PROD, int NS>
 __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial, u64 *out,
                                                  u64 scale, int direct) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
@@ -122,31 +133,71 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
             }
             continue;
         }
-        for (int x = 0; x <= D.deg; ++x) {
-            if (!(D.skip1 && x == 1)) {
-                u64 sx = 0;
-                for (int k = 0; k < D.n_terms; ++k) {
-                    // factors are canonical; partial products may stay non-canonical words,
-                    // only the last multiplication of a term reduces fully
-                    u64 prod = D.coeff_at_end ? 1 : D.coeff[k];
-                    bool first = D.coeff_at_end;
-                    const int j1 = D.term_off[k + 1];
-                    for (int j = D.term_off[k]; j < j1; ++j) {
-                        int t = D.fidx[j];
-                        u64 v = cur[t];
-                        prod = first ? v : (j + 1 < j1 ? gl::mul_lazy(prod, v) : gl::mul(prod, v));
-                        first = false;
-                    }
-                    sx = gl::addc(sx, prod);
-                }
-#pragma unroll
-                for (int y = 0; y < NSAMP; ++y)
-                    if (y == x) acc[y] = gl::addc(acc[y], sx);
+        // General sums: the term description is walked once per pair, and each factor it names (a register
+        // picked by a wave-uniform index) is applied to all evaluation points before the next one is
+        // fetched, so the cost of interpreting is paid per factor and not per factor and point.
+        u64 sx[NS];
+        {
+            // the terms that are linear in x, as value and step
+            u64 lc = D.c0, ld = 0;
+            for (int k = 0; k < D.n_lin; ++k) {
+                const int t = D.lin_idx[k];
+                const u64 c = D.lin_coeff[k];
+                lc = gl::addc(lc, gl::mul(c, cur[t]));
+                ld = gl::addc(ld, gl::mul(c, dif[t]));
             }
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-                if (t < D.n_tables) cur[t] = gl::addc(cur[t], dif[t]);
+            for (int x = 0; x < NS; ++x) {
+                sx[x] = lc;
+                if (D.n_lin && x < D.deg) lc = gl::addc(lc, ld);
+            }
         }
+        for (int k = 0; k < D.n_terms; ++k) {
+            // factors are canonical; the running products stay non-canonical words and are
+            // reduced fully once, when the term is added
+            u64 prod[NS];
+            int j = D.term_off[k];
+            const int j1 = D.term_off[k + 1];
+            if (D.coeff_at_end) {
+                const int t = D.fidx[j++];
+                u64 v = cur[t];
+                const u64 d = dif[t];
+#pragma unroll
+                for (int x = 0; x < NS; ++x) {
+                    prod[x] = v;
+                    if (x < D.deg) v = gl::addc(v, d);
+                }
+            } else {
+                const u64 c = D.coeff[k];
+#pragma unroll
+                for (int x = 0; x < NS; ++x) prod[x] = c;
+            }
+            for (; j < j1; ++j) {
+                const int t = D.fidx[j];
+                u64 v = cur[t];
+                const u64 d = dif[t];
+#pragma unroll
+                for (int x = 0; x < NS; ++x) {
+                    if (x <= D.deg && !(D.skip1 && x == 1)) prod[x] = gl::mul_lazy(prod[x], v);
+                    if (x < D.deg) v = gl::addc(v, d);
+                }
+            }
+#pragma unroll
+            for (int x = 0; x < NS; ++x)
+                if (x <= D.deg) sx[x] = gl::addc(sx[x], gl::canon(prod[x]));
+        }
+        if (D.common >= 0) {
+            u64 v = cur[D.common];
+            const u64 d = dif[D.common];
+#pragma unroll
+            for (int x = 0; x < NS; ++x) {
+                if (x <= D.deg && !(D.skip1 && x == 1)) sx[x] = gl::mul(sx[x], v);
+                if (x < D.deg) v = gl::addc(v, d);
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < NS; ++x)
+            if (x <= D.deg) acc[x] = gl::addc(acc[x], sx[x]);
       }
     }
     if (MODE == 1) return;
@@ -242,6 +293,43 @@ __global__ __launch_bounds__(BLOCK) void k_final(const u64 *partial, int nb, int
     }
 }
 
+// Rewrites the terms of D (already validated and copied) into the factored form described at Desc.
+void factor_terms(Desc &D, const int *term_off, const int *factor_idx, int n_terms) {
+    // a table that occurs in every term
+    for (int j = term_off[0]; j < term_off[1] && D.common < 0; ++j) {
+        bool everywhere = true;
+        for (int k = 1; k < n_terms && everywhere; ++k) {
+            bool found = false;
+            for (int i = term_off[k]; i < term_off[k + 1]; ++i) found = found || factor_idx[i] == factor_idx[j];
+            everywhere = found;
+        }
+        if (everywhere) D.common = factor_idx[j];
+    }
+    int n_prod = 0, n_fac = 0;
+    for (int k = 0; k < n_terms; ++k) {
+        const u64 c = D.coeff[k];           // reads entry k before entry n_prod <= k is overwritten
+        int rest[MAX_DEG], nr = 0;
+        bool dropped = false;
+        for (int i = term_off[k]; i < term_off[k + 1]; ++i) {
+            if (!dropped && factor_idx[i] == D.common) { dropped = true; continue; }
+            rest[nr++] = factor_idx[i];
+        }
+        if (nr == 0) {
+            D.c0 = gl::add(D.c0, c);
+        } else if (nr == 1) {
+            D.lin_idx[D.n_lin] = (unsigned char)rest[0];
+            D.lin_coeff[D.n_lin++] = c;
+        } else {
+            D.coeff[n_prod] = c;
+            D.term_off[n_prod] = (unsigned char)n_fac;
+            for (int i = 0; i < nr; ++i) D.fidx[n_fac++] = (unsigned char)rest[i];
+            ++n_prod;
+        }
+    }
+    D.term_off[n_prod] = (unsigned char)n_fac;
+    D.n_terms = n_prod;
+}
+
 int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_tables, const int *term_off,
               const int *factor_idx, const uint64_t *coeffs, int n_terms, bool need_terms, const char *who) {
     if (n_tables < 1 || n_tables > VI_SC_MAX_TABLES) return vi::fail(VI_EINVAL, "%s: n_tables = %d (1..%d)", who, n_tables, VI_SC_MAX_TABLES);
@@ -252,6 +340,9 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         D.dst[t] = dst ? dst[t] : nullptr;
     }
     D.n_terms = 0;
+    D.n_lin = 0;
+    D.common = -1;
+    D.c0 = 0;
     D.deg = 0;
     D.coeff_at_end = 0;
     D.product = 0;
@@ -280,6 +371,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         for (int j = 0; j < n_tables; ++j) seen |= 1u << factor_idx[j];
         D.product = (seen == (1u << n_tables) - 1);
     }
+    if (n_terms >= 2 && n_tables <= REG_TABLES) factor_terms(D, term_off, factor_idx, n_terms);
     return VI_OK;
 }
 
@@ -306,19 +398,20 @@ int resident_blocks(K kernel) {
     return nb > MAX_BLOCKS ? MAX_BLOCKS : nb;
 }
 
-template <int NT, int MODE, int U, bool PROD>
+template <int NT, int MODE, int U, bool PROD, int NS>
 int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
-    static const int cap = resident_blocks(k_round<NT, MODE, U, PROD>);     // per instantiation, first use
+    static const int cap = resident_blocks(k_round<NT, MODE, U, PROD, NS>);     // per instantiation, first use
     if (nb > cap) nb = cap;
-    hipLaunchKernelGGL((k_round<NT, MODE, U, PROD>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    hipLaunchKernelGGL((k_round<NT, MODE, U, PROD, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
     return nb;
 }
 
 template <int NT, int MODE, int U>
 int launch_k(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
     if (MODE != 1 && NT <= 4 && D.product && D.n_tables == NT)
-        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4)>(D, half, r, partial, nb, out, scale, direct, s);
-    return launch_kp<NT, MODE, U, false>(D, half, r, partial, nb, out, scale, direct, s);
+        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4), NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
+    if (MODE != 1 && D.deg <= 3) return launch_kp<NT, MODE, U, false, (MODE != 1 ? 4 : NSAMP)>(D, half, r, partial, nb, out, scale, direct, s);
+    return launch_kp<NT, MODE, U, false, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
 }
 
 template <int MODE, int U>
