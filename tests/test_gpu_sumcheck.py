@@ -92,6 +92,10 @@ def test_sum_of_products_shared_tables_and_coefficients(mods):
     ("degree one", 3, [(3, [0]), (P - 5, [1]), (7, [2])]),
     # two candidates for the common table
     ("two common", 3, [(3, [0, 1, 2]), (5, [1, 0])]),
+    # more tables than a thread keeps in registers: the same forms with the factors read from memory
+    ("many tables", 11, [(3, [0, 1, 2]), (P - 5, [0, 3]), (7, [0, 4, 5]), (11, [0, 6]), (13, [0, 7, 8]), (17, [0, 9]),
+                         (19, [0, 10, 10]), (23, [0])]),
+    ("many tables, no common", 10, [(3, [0, 1, 2]), (P - 5, [3]), (7, [4, 5]), (11, [6]), (13, [7, 8, 9, 0])]),
 ])
 @pytest.mark.parametrize("v", [1, 5, 12])
 def test_factored_term_forms_match_oracle(mods, name, nt, terms, v):

@@ -35,7 +35,7 @@ struct Desc {
     u64 coeff[VI_SC_MAX_TERMS];
     unsigned char term_off[VI_SC_MAX_TERMS + 1];
     unsigned char fidx[VI_SC_MAX_FACTORS];
-    // Several terms over tables a thread keeps in registers are stored factored:
+    // Several terms are stored factored:
     //   S(x) = common(x) * ( c0 + sum_k lin_coeff[k] f_lin[k](x) + sum_k coeff[k] prod_j f_kj(x) )
     // where `common` is a table every term contains (eq(z, .) in a batched gate check, layergkr/relations.py:117-121;
     // -1 = none, the bracket alone), a term left without factors adds its coefficient to c0, a term left with one
@@ -234,6 +234,22 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
 #pragma unroll
     for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride) {
+        // the factored form described at Desc, every factor fetched from its table
+        u64 sx[NSAMP];
+        {
+            u64 lc = D.c0, ld = 0;
+            for (int k = 0; k < D.n_lin; ++k) {
+                const u64 *f = D.src[D.lin_idx[k]];
+                const u64 c = D.lin_coeff[k], cur = f[i], dif = gl::sub(f[half + i], cur);
+                lc = gl::add(lc, gl::mul(c, cur));
+                ld = gl::add(ld, gl::mul(c, dif));
+            }
+#pragma unroll
+            for (int x = 0; x < NSAMP; ++x) {
+                sx[x] = lc;
+                if (D.n_lin) lc = gl::add(lc, ld);
+            }
+        }
         for (int k = 0; k < D.n_terms; ++k) {
             u64 prod[NSAMP];
 #pragma unroll
@@ -249,8 +265,20 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
             }
 #pragma unroll
             for (int x = 0; x < NSAMP; ++x)
-                if (x <= D.deg) acc[x] = gl::add(acc[x], prod[x]);
+                if (x <= D.deg) sx[x] = gl::add(sx[x], prod[x]);
         }
+        if (D.common >= 0) {
+            const u64 *f = D.src[D.common];
+            u64 cur = f[i], dif = gl::sub(f[half + i], cur);
+#pragma unroll
+            for (int x = 0; x < NSAMP; ++x) {
+                if (x <= D.deg) sx[x] = gl::mul(sx[x], cur);
+                cur = gl::add(cur, dif);
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < NSAMP; ++x)
+            if (x <= D.deg) acc[x] = gl::add(acc[x], sx[x]);
     }
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
@@ -371,7 +399,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         for (int j = 0; j < n_tables; ++j) seen |= 1u << factor_idx[j];
         D.product = (seen == (1u << n_tables) - 1);
     }
-    if (n_terms >= 2 && n_tables <= REG_TABLES) factor_terms(D, term_off, factor_idx, n_terms);
+    if (n_terms >= 2) factor_terms(D, term_off, factor_idx, n_terms);
     return VI_OK;
 }
 
