@@ -188,6 +188,20 @@ def bench_kquant(torch, steps=20, cpu=True):
         t = s.elapsed_time(e) / steps
         res[qt.lower() + "_ms"] = t
         res[qt.lower() + "_gbs_algorithmic"] = nb * (bb + 2048) / (t * 1e-3) / 1e9
+    # the loader's call site (prover/loader.py:427-436) wants the (k_in, n_out) transpose: one fused pass
+    # against decode followed by torch's .T.contiguous()
+    def two_step():
+        return kq.kquant_to_field(raw, "Q4_K", 4096).view(4096, 11008).view(torch.int64).T.contiguous()
+    for name, fn in (("transposed_fused_ms", lambda: kq.kquant_to_field_transposed(raw, "Q4_K", 4096, 4096)),
+                     ("transposed_two_step_ms", two_step)):
+        fn()
+        torch.cuda.synchronize()
+        s.record()
+        for _ in range(steps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        res[name] = s.elapsed_time(e) / steps
     if cpu:
         # C oracle (scalar byte map, OpenMP over blocks) on the whole matrix, compared bit for bit
         import numpy as np

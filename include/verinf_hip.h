@@ -128,6 +128,12 @@ int vi_coset_extend(const uint64_t *coeffs, int64_t m, int64_t width, int64_t co
  * elements, round-half-even(double(fp32 dequant) * S), negatives as p - |x|. */
 int vi_kquant_to_field(int qtype, const uint8_t *raw, int64_t n_blocks, double S, uint64_t *out,
                        void *stream);
+/* The same decode of a (d_out, d_in) matrix stored row by row (d_in a multiple of 256), written
+ * transposed: out[c * d_out + r] = weight (r, c).  Replaces the decode followed by the
+ * `.view(d_out, d_in).T.contiguous()` pass with which the loader brings an expert matrix into
+ * (k_in, n_out) order (prover/loader.py:427-436). */
+int vi_kquant_to_field_transposed(int qtype, const uint8_t *raw, int64_t d_out, int64_t d_in, double S,
+                                  uint64_t *out, void *stream);
 
 /* ---- multilinear sumcheck --------------------------------------------------------
  * Replace the per-round torch composition of layergkr/gpu.py:341-410 (fold_t,

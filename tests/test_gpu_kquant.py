@@ -91,3 +91,37 @@ def test_kquant_baseline_shape(kq):
     # the caller's reshape/transposition of prover/loader.py:433-436 works on the result
     w = got.view(4096, 11008).view(torch.int64).T.contiguous().view(torch.uint64)
     assert tuple(w.shape) == (11008, 4096)
+
+
+@pytest.mark.parametrize("qtype", ["Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("d_out,bpr", [(1, 1), (16, 1), (37, 3), (64, 2), (130, 5), (1000, 4)])
+def test_kquant_transposed_matches_oracle(kq, qtype, d_out, bpr):
+    """Decode + transpose in one pass against the oracle's decode transposed on the host:
+    row counts below, at and across the 16-row tile, one and several super-blocks per row."""
+    raw = synth_blocks(qtype, d_out * bpr, 7 + d_out)
+    want = O.kquant_to_field(raw, qtype, 1 << 12).reshape(d_out, bpr * 256).T.reshape(-1)
+    d = torch.from_numpy(raw).cuda()
+    got = kq.kquant_to_field_transposed(d, qtype, 1 << 12, d_out)
+    assert got.shape == (d_out * bpr * 256,)
+    assert np.array_equal(to_np(got), want)
+    # the two-step form of prover/loader.py:427-436 gives the same tensor
+    two = kq.kquant_to_field(d, qtype, 1 << 12).view(d_out, bpr * 256).view(torch.int64).T.contiguous().view(torch.uint64)
+    assert torch.equal(got.view(torch.int64), two.reshape(-1).view(torch.int64))
+    # a buffer at an odd address takes the one-thread-per-weight kernel
+    buf = torch.empty(raw.size + 1, dtype=torch.uint8, device="cuda")
+    buf[1:] = d.reshape(-1)
+    assert np.array_equal(to_np(kq.kquant_to_field_transposed(buf[1:], qtype, 1 << 12, d_out)), want)
+
+
+def test_kquant_transposed_errors_and_baseline_shape(kq):
+    z = torch.zeros(144 * 6, dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError):
+        kq.kquant_to_field_transposed(z, "Q4_K", 4096, 4)            # 6 blocks are not 4 rows
+    with pytest.raises(RuntimeError):
+        kq.kquant_to_field_transposed(z, "Q4_K", 4096, 0)
+    assert kq.kquant_to_field_transposed(z[:0], "Q4_K", 4096, 3).numel() == 0
+    nb = 4096 * 11008 // 256
+    raw = synth_blocks("Q4_K", nb, 3)
+    got = kq.kquant_to_field_transposed(torch.from_numpy(raw).cuda(), "Q4_K", 1 << 12, 4096)
+    want = O.kquant_to_field(raw, "Q4_K", 1 << 12).reshape(4096, 11008).T
+    assert np.array_equal(to_np(got).reshape(11008, 4096), want)
