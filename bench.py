@@ -33,6 +33,10 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 # each scaled by what the same counter reads for a 1 GiB device copy.  roofline.traffic is this figure divided
 # by the launches of a step, like roofline.achieved.
 LDE_TRAFFIC_BYTES_PER_STEP = 9.57e9
+# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU: 4 forward launches of 375.2 M and
+# 4 inverse launches of 85.3 M) and the rate at which 1024 SIMDs issue them at 2.4 GHz, one per four cycles
+LDE_VALU_INSTS_PER_STEP = 4 * 375_205_376 + 4 * 85_323_264
+VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / 4
 
 
 def _events(torch):
@@ -456,7 +460,13 @@ def main():
                                        "(x2.000 / x1.000); not re-measured in this run",
                      "kernel": "k_ntt_fast", "launches_per_step": lde["launches_per_step"],
                      "avg_launch_us": lde["kernel_avg_us"],
-                     "algorithmic_bytes_per_launch": lde["alg_bytes_per_launch"]},
+                     "algorithmic_bytes_per_launch": lde["alg_bytes_per_launch"],
+                     # the same launches against the integer-VALU issue rate, which is what bounds this kernel
+                     "valu_issue": {"wave_instructions_per_step": LDE_VALU_INSTS_PER_STEP,
+                                    "achieved_per_s": LDE_VALU_INSTS_PER_STEP / (lde["ms_per_step"] * 1e-3),
+                                    "peak_per_s": VALU_ISSUE_PEAK_PER_S,
+                                    "frac": LDE_VALU_INSTS_PER_STEP / (lde["ms_per_step"] * 1e-3) / VALU_ISSUE_PEAK_PER_S,
+                                    "source": "rocprofv3 --pmc SQ_INSTS_VALU of this command; not re-measured in this run"}},
         "cpu_baseline": cpu,
         "extra": extra,
     }
