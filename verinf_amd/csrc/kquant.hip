@@ -157,7 +157,7 @@ __global__ __launch_bounds__(BLOCK) void k_kq(const unsigned char *__restrict__ 
 // an LDS tile [row][column] (16-byte writes, row pitch 258 words), then every thread collects two
 // consecutive rows of one column and stores them, so that a wavefront store covers eight runs of
 // T_ROWS * 8 = 128 consecutive bytes.
-constexpr int T_ROWS = 16;       // 8 rows: 0.233 ms, 16: 0.106 ms, 32: 0.110 ms on a 4096 x 11008 Q4_K matrix
+constexpr int T_ROWS = 16;       // 8-row tiles were twice as slow, 32-row tiles no faster (4096 x 11008 Q4_K)
 constexpr int T_PITCH = 258;
 
 template <int QT>
@@ -184,9 +184,20 @@ __global__ __launch_bounds__(BLOCK) void k_kq_t(const unsigned char *__restrict_
         const int c = (threadIdx.x / RP) + i * (BLOCK / RP);
         const u64 v0 = tile[(2 * rp) * T_PITCH + c], v1 = tile[(2 * rp + 1) * T_PITCH + c];
         u64 *o = dst + (i64)c * d_out;
-        // streaming stores: 0.106 ms against 0.142 ms with ordinary ones
-        if (r0 + 2 * rp < d_out) __builtin_nontemporal_store(v0, o);
-        if (r0 + 2 * rp + 1 < d_out) __builtin_nontemporal_store(v1, o + 1);
+        // streaming stores (ordinary ones were a third slower).  With an even row count a pair of rows is
+        // there or not as a whole and sits at a 16-byte boundary: one 16-byte store, so that the eight lanes of a
+        // run write whole 32-byte sectors (two 8-byte stores per lane wrote 1.66 x the bytes)
+        if ((d_out & 1) == 0 && ((uintptr_t)out & 15) == 0) {
+            if (r0 + 2 * rp < d_out) {
+                ulonglong2 v;
+                v.x = v0;
+                v.y = v1;
+                stream_store((ulonglong2 *)o, v);
+            }
+        } else {
+            if (r0 + 2 * rp < d_out) __builtin_nontemporal_store(v0, o);
+            if (r0 + 2 * rp + 1 < d_out) __builtin_nontemporal_store(v1, o + 1);
+        }
     }
 }
 
@@ -249,7 +260,10 @@ extern "C" int vi_kquant_to_field(int qtype, const uint8_t *raw, int64_t n_block
     hipStream_t s = (hipStream_t)stream;
     const i64 n = n_blocks * 256;
     const bool out16 = ((uintptr_t)out & 15) == 0;
-    const unsigned gw = grid_cap((n_blocks + 3) / 4, 256 * 32);        // one wavefront per super-block
+    // one wavefront per super-block and a workgroup per four of them: 0.062 ms on 4096 x 11008 Q4_K against 0.067 ms
+    // for a grid capped at 32 workgroups per CU that strides over the blocks (the loop in the kernel covers the
+    // sizes beyond the grid limit)
+    const unsigned gw = grid_cap((n_blocks + 3) / 4, 0x7FFFFFFF);
     if (qtype == 4 && ((uintptr_t)raw & 3) == 0 && out16) {
         hipLaunchKernelGGL(k_kq<4>, dim3(gw), dim3(BLOCK), 0, s, raw, out, (i64)n_blocks, S);
     } else if (qtype == 5 && ((uintptr_t)raw & 3) == 0 && out16) {
