@@ -92,6 +92,10 @@ def test_sum_of_products_shared_tables_and_coefficients(mods):
     ("degree one", 3, [(3, [0]), (P - 5, [1]), (7, [2])]),
     # two candidates for the common table
     ("two common", 3, [(3, [0, 1, 2]), (5, [1, 0])]),
+    # the first product term's coefficient is divided out of the sum: zero, one and p - 1 as that coefficient
+    ("first coefficient zero", 5, [(0, [0, 1, 2]), (5, [0, 3, 4]), (7, [0, 2])]),
+    ("first coefficient one", 5, [(1, [0, 1, 2]), (5, [0, 3, 4]), (7, [0, 2]), (9, [0])]),
+    ("first coefficient minus one", 5, [(P - 1, [0, 1, 2]), (5, [0, 3, 4]), (7, [0, 2]), (9, [0])]),
     # more tables than a thread keeps in registers: the same forms with the factors read from memory
     ("many tables", 11, [(3, [0, 1, 2]), (P - 5, [0, 3]), (7, [0, 4, 5]), (11, [0, 6]), (13, [0, 7, 8]), (17, [0, 9]),
                          (19, [0, 10, 10]), (23, [0])]),

@@ -47,6 +47,9 @@ struct Desc {
     int n_lin, common;
     int n_tables, n_terms, deg;
     int coeff_at_end;                       // single term: apply its coefficient in the final reduction
+    u64 out_scale;                          // factor the finished samples are multiplied by (1 = none): the single
+                                            // term's coefficient, or the first product term's coefficient of a
+                                            // factored sum, whose other coefficients are divided by it
     int product;                            // one term whose factors are exactly the n_tables tables, once each
     int skip1;                              // S(1) is not summed: it is claim - S(0) (the round's known total)
     u64 claim;                              // S(0) + S(1) when skip1
@@ -158,7 +161,8 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
             u64 prod[NS];
             int j = D.term_off[k];
             const int j1 = D.term_off[k + 1];
-            if (D.coeff_at_end) {
+            const u64 c = D.coeff[k];
+            if (D.coeff_at_end || c == 1) {
                 const int t = D.fidx[j++];
                 u64 v = cur[t];
                 const u64 d = dif[t];
@@ -168,7 +172,6 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
                     if (x < D.deg) v = gl::addc(v, d);
                 }
             } else {
-                const u64 c = D.coeff[k];
 #pragma unroll
                 for (int x = 0; x < NS; ++x) prod[x] = c;
             }
@@ -356,6 +359,15 @@ void factor_terms(Desc &D, const int *term_off, const int *factor_idx, int n_ter
     }
     D.term_off[n_prod] = (unsigned char)n_fac;
     D.n_terms = n_prod;
+    // the first product term's coefficient leaves the sum: one multiplication per evaluation point less
+    if (n_prod >= 1 && D.coeff[0] > 1) {
+        const u64 s = D.coeff[0], s_inv = gl::inv(s);
+        D.out_scale = s;
+        D.coeff[0] = 1;
+        for (int k = 1; k < n_prod; ++k) D.coeff[k] = gl::mul(D.coeff[k], s_inv);
+        for (int k = 0; k < D.n_lin; ++k) D.lin_coeff[k] = gl::mul(D.lin_coeff[k], s_inv);
+        D.c0 = gl::mul(D.c0, s_inv);
+    }
 }
 
 int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_tables, const int *term_off,
@@ -373,6 +385,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
     D.c0 = 0;
     D.deg = 0;
     D.coeff_at_end = 0;
+    D.out_scale = 1;
     D.product = 0;
     D.skip1 = 0;
     D.claim = 0;
@@ -394,6 +407,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         D.fidx[j] = (unsigned char)factor_idx[j];
     }
     D.coeff_at_end = (n_terms == 1);
+    if (n_terms == 1 && n_tables <= REG_TABLES) D.out_scale = D.coeff[0];     // k_eval_mem applies it per term instead
     if (n_terms == 1 && term_off[1] == n_tables && n_tables <= 4) {
         unsigned seen = 0;
         for (int j = 0; j < n_tables; ++j) seen |= 1u << factor_idx[j];
@@ -479,7 +493,7 @@ int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, 
     if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
     hipStream_t s = (hipStream_t)stream;
     int nb = blocks_for(half);
-    u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
+    const u64 scale = D.out_scale;
     if (n_tables <= REG_TABLES && half <= DIRECT_MAX) {
         launch_round<0>(D, half, 0, (u64 *)ws, 1, out_samples, scale, 1, s);
         VI_LAUNCH_CHECK("sumcheck eval");
@@ -523,7 +537,7 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
         return VI_OK;
     }
     int nb;
-    const u64 scale = (D.coeff_at_end && n_tables <= REG_TABLES) ? D.coeff[0] : 1;
+    const u64 scale = D.out_scale;
     if (n_tables <= REG_TABLES) {
         if ((half >> 1) <= DIRECT_MAX) {
             launch_round<2>(D, half, r, (u64 *)ws, 1, out_samples, scale, 1, s);
