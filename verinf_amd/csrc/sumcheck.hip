@@ -429,10 +429,14 @@ constexpr i64 DIRECT_MAX = 256;     // one loop trip per thread
 // would run its surplus workgroups as a second, mostly empty wave (measured: 8 waves
 // per SIMD requested, 7 resident -> almost 2x the time).  So the grid is capped at the
 // kernel's own occupancy times the CU count.
+// max_per_cu: the fused fold + evaluate round streams four runs per table and is faster with at most five
+// workgroups per CU than with the seven or eight its registers would allow (rounds 1-3 of the 3 x 2^26 proof:
+// 5,140 / 4,870 / 4,520 GB/s against 4,850 / 4,560 / 4,200); the evaluation-only round wants all it can get.
 template <typename K>
-int resident_blocks(K kernel) {
+int resident_blocks(K kernel, int max_per_cu) {
     int per_cu = 0, dev = 0, cus = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, BLOCK, 0) != hipSuccess || per_cu < 1) per_cu = 4;
+    if (per_cu > max_per_cu) per_cu = max_per_cu;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
         cus = 256;
@@ -442,7 +446,7 @@ int resident_blocks(K kernel) {
 
 template <int NT, int MODE, int U, bool PROD, int NS>
 int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
-    static const int cap = resident_blocks(k_round<NT, MODE, U, PROD, NS>);     // per instantiation, first use
+    static const int cap = resident_blocks(k_round<NT, MODE, U, PROD, NS>, MODE == 2 ? 5 : 64);     // per instantiation, first use
     if (nb > cap) nb = cap;
     hipLaunchKernelGGL((k_round<NT, MODE, U, PROD, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
     return nb;
