@@ -24,7 +24,8 @@ def _matmul_ref(A, B):
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 1, 1), (1, 7, 300), (3, 64, 64), (5, 200, 513), (1, 4096, 8192),
-                                   (2, 1000, 70000), (16, 16, 1000), (40, 33, 257)])
+                                   (2, 1000, 70000), (16, 16, 1000), (40, 33, 257),
+                                   (4, 129, 300), (7, 50, 600), (6, 4100, 256), (3, 9, 5)])
 def test_matmul_matches_bigint(cp, m, k, n):
     A, B = rand_field((m, k), 1 + m), rand_field((k, n), 2 + n)
     got = cp.gl_matmul(to_dev(A), to_dev(B))
@@ -42,6 +43,14 @@ def test_matmul_extreme_values_many_wraps(cp):
     B[::2] = 1
     got = to_np(cp.gl_matmul(to_dev(A), to_dev(B)))
     assert (got == np.uint64((k // 2 + (k // 2) * (P - 1)) % P)).all()
+
+
+@pytest.mark.parametrize("m,n", [(1, 1), (37, 1001), (3, 4096), (5, 5000), (9000, 70), (300, 255), (2, 20011)])
+def test_matvec_matches_bigint(cp, m, n):
+    """Short and long rows (a wavefront or a whole workgroup per row), lengths around the unrolled stride."""
+    M, v = rand_field((m, n), 3 + m), rand_field(n, 4 + n)
+    got = to_np(cp.gl_matvec(to_dev(M), to_dev(v)))
+    assert np.array_equal(got, _matmul_ref(M, v.reshape(-1, 1)).reshape(-1))
 
 
 def test_matvec_and_poly_eval(cp):

@@ -120,7 +120,15 @@ __global__ __launch_bounds__(BLOCK) void k_sum_partial(const u64 *a, i64 n, u64 
     __shared__ u64 lds4[BLOCK / 64];
     i64 stride = (i64)gridDim.x * BLOCK;
     u64 acc = 0;
-    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) {
+    i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    for (; i + 3 * stride < n; i += 4 * stride) {     // four loads in flight
+        u64 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = a[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc = gl::add(acc, v[u] >= gl::P ? v[u] - gl::P : v[u]);
+    }
+    for (; i < n; i += stride) {
         u64 v = a[i];
         acc = gl::add(acc, v >= gl::P ? v - gl::P : v);
     }

