@@ -123,9 +123,13 @@ VI_HD ColRef col_ref(const PassArgs &A, i64 tile, int c) {
 // stage-1 thread -> (column, n2)
 template <int A2>
 VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
-    const int lt = logT(A);
-    if (!A.is_final) { c = tid & ((1 << lt) - 1); n2 = tid >> lt; }
-    else { n2 = tid & ((1 << A2) - 1); c = tid >> A2; }
+    // low bits / high bits of the thread id, then one select each: written as two branches that assign c and n2
+    // crosswise the compiler routed the values through scratch memory (a store and a load in front of the
+    // first address computation of every workgroup)
+    const int sh = A.is_final ? A2 : logT(A);
+    const int lo = tid & ((1 << sh) - 1), hi = tid >> sh;
+    c = A.is_final ? hi : lo;
+    n2 = A.is_final ? lo : hi;
 }
 
 // phase 1: this thread's 16 stage-1 inputs x[n1*E2 + n2], zero beyond src_width
