@@ -39,13 +39,14 @@ void run_fast(const PassArgs &A) {
     i64 tiles = pass_tiles(A);
     std::vector<u64> lds(fast_lds_words(A.a));
     std::vector<u64> regs((size_t)NTHREADS * 16);
+    std::vector<u32> oks(NTHREADS);
     int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
     for (i64 tile = 0; tile < tiles; ++tile) {
         for (int tid = 0; tid < NTHREADS; ++tid)
-            fast_load<A2>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]));
+            fast_load<A2>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
         for (int t = 0; t < n_loop; ++t) {
             for (int tid = 0; tid < NTHREADS; ++tid)
-                fast_stage1<A2, INV>(A, tile, tid, t, *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
+                fast_stage1<A2, INV>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
                                      A.twi, lds.data());
             for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV>(A, tile, tid, t, lds.data());
         }

@@ -70,8 +70,23 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
         t = (int)(slot & ((1u << A.log_rho) - 1));
         tile = (i64)(slot >> A.log_rho) * 8 + xcd;
     }
+    // the inner twiddle rows this thread copies into LDS are requested first, the tile after them
+    const int lt = TILE_LOG - A.a;
+    const int lane = tid & 63, first = ((tid & ~63) >> lt) * 16, count = lt >= 6 ? 16 : (16 << (6 - lt));
+    u64 tw_mine[(16 << A2) / NTHREADS > 0 ? (16 << A2) / NTHREADS : 1];
+    u64 tw_wave = 0;
+    if (!A.is_final) {
+        // strided pass: a wavefront uses only the table rows of its own n2 values (at most 64 words), so each
+        // wavefront fills just those and no workgroup barrier is needed before stage 1
+        if (lane < count) tw_wave = A.twi[first + lane];
+    } else {
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(tw_mine) / sizeof(u64)); ++i)
+            tw_mine[i] = (tid + i * NTHREADS < (16 << A2)) ? A.twi[tid + i * NTHREADS] : 0;
+    }
     u64 reg[16];
-    fast_load<A2>(A, tile, tid, reg);
+    u32 ok;
+    fast_load<A2>(A, tile, tid, reg, ok);
     // Warm the L2 for a workgroup that will run on this XCD a little later: after its own loads (loads return in
     // order, so the touch must be the youngest) every thread reads one word of tile + TOUCH_AHEAD.  The slot that
     // later loads that tile finds it in the L2 instead of waiting on HBM.  Measured on 1024 x 2^16 -> 2^18 with
@@ -79,17 +94,15 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     // 3.58 / 3.79 / 3.87 ms (about 1024 workgroups are resident; further ahead and the lines are evicted before use).
     const u64 touched = fast_touch<A2>(A, tile + (expand ? (TOUCH_AHEAD >> A.log_rho) : TOUCH_AHEAD), n_tiles, tid);
     if (!A.is_final) {
-        // strided pass: a wavefront uses only the table rows of its own n2 values (at most 64 words), so each
-        // wavefront fills just those and no workgroup barrier is needed before stage 1
-        const int lt = TILE_LOG - A.a;
-        const int lane = tid & 63, first = ((tid & ~63) >> lt) * 16, count = lt >= 6 ? 16 : (16 << (6 - lt));
-        if (lane < count) twi[first + lane] = A.twi[first + lane];
+        if (lane < count) twi[first + lane] = tw_wave;
         __builtin_amdgcn_wave_barrier();
     } else {
-        for (int i = tid; i < (16 << A2); i += NTHREADS) twi[i] = A.twi[i];
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(tw_mine) / sizeof(u64)); ++i)
+            if (tid + i * NTHREADS < (16 << A2)) twi[tid + i * NTHREADS] = tw_mine[i];
         __syncthreads();
     }
-    fast_stage1<A2, INV>(A, tile, tid, t, reg, twi, lds);
+    fast_stage1<A2, INV>(A, tile, tid, t, ok, reg, twi, lds);
     __syncthreads();
     fast_stage2<A2, INV>(A, tile, tid, t, lds);
     asm volatile("" ::"v"(touched));      // the touch load must not be optimised away; its value is unused

@@ -132,17 +132,32 @@ VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
     n2 = A.is_final ? lo : hi;
 }
 
-// phase 1: this thread's 16 stage-1 inputs x[n1*E2 + n2], zero beyond src_width
+// phase 1: this thread's 16 stage-1 inputs x[n1*E2 + n2] as loaded, and in `ok` which of them exist.
+// All sixteen loads are issued before the first value is looked at: an element that does not exist (a row past
+// the batch, a point past the source width) reads word 0 of the source instead and is zeroed in fast_fix.  With
+// the load inside the test, and the reduction mod p right behind it, every second load waited for the one
+// before -- eight memory round trips per tile instead of one.
 template <int A2>
-VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16]) {
+VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &ok) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
     const ColRef R = col_ref(A, tile, c);
     const int sh = A.is_final ? 0 : A.logR;
+    ok = 0;
 #pragma unroll
     for (int n1 = 0; n1 < 16; ++n1) {
         const i64 l = (i64)((n1 << A2) + n2) << sh;
-        u64 v = (R.valid && R.idx_base + l < A.src_width) ? A.src[R.src_base + l] : 0;
+        const bool there = R.valid && R.idx_base + l < A.src_width;
+        ok |= there ? (1u << n1) : 0u;
+        reg[n1] = A.src[there ? R.src_base + l : 0];
+    }
+}
+
+// zero for the elements that do not exist, caller data reduced mod p
+VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
+#pragma unroll
+    for (int n1 = 0; n1 < 16; ++n1) {
+        const u64 v = ((ok >> n1) & 1) ? reg[n1] : 0;
         reg[n1] = A.canon_src ? gl::canon(v) : v;
     }
 }
@@ -165,7 +180,7 @@ VI_HD u64 fast_touch(const PassArgs &A, i64 tile_ahead, i64 n_tiles, int tid) {
 // phase 2: optional coset pre-multiplier, 16-point transform, w_L^(n2 k1), into LDS
 // twi: w_L^(n2 k1) at [n2 * 16 + k1]
 template <int A2, bool INV>
-VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, const u64 (&reg)[16],
+VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok, const u64 (&reg)[16],
                        const u64 *twi, u64 *lds) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
@@ -174,21 +189,23 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, const u
     for (int i = 0; i < 16; ++i) x[i] = reg[i];
     if (A.pre) {
         const ColRef R = col_ref(A, tile, c);
-        if (R.valid) {
-            const int sh = A.is_final ? 0 : A.logR;
-            const int t = A.is_final ? R.t : t_loop;
-            const u64 *pre = A.pre + ((i64)t << A.logn) + R.idx_base;
-            // all sixteen multipliers are requested at once (they arrive while the data loads are still in flight)
-            u64 pw[16];
+        const int sh = A.is_final ? 0 : A.logR;
+        const int t = A.is_final ? R.t : t_loop;
+        // all sixteen multipliers are requested before the data loads are waited for (a column that does not
+        // exist takes those of point 0 of coset 0; its data are zero)
+        const u64 *pre = A.pre + (R.valid ? ((i64)t << A.logn) + R.idx_base : 0);
+        u64 pw[16];
 #pragma unroll
-            for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[(i64)((n1 << A2) + n2) << sh];
+        for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[R.valid ? (i64)((n1 << A2) + n2) << sh : 0];
+        fast_fix(A, ok, x);
 #pragma unroll
-            for (int g = 0; g < 16; g += 4) {
+        for (int g = 0; g < 16; g += 4) {
 #pragma unroll
-                for (int n1 = g; n1 < g + 4; ++n1) x[n1] = gl::mul(x[n1], pw[n1]);
-                VI_SCHED_FENCE();
-            }
+            for (int n1 = g; n1 < g + 4; ++n1) x[n1] = gl::mul(x[n1], pw[n1]);
+            VI_SCHED_FENCE();
         }
+    } else {
+        fast_fix(A, ok, x);
     }
     VI_SCHED_FENCE();
     dft_reg<4, INV>(x);
