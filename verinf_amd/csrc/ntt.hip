@@ -21,10 +21,6 @@
 
 using namespace ntt;
 
-// tiles between a workgroup and the one whose source it touches ahead; a multiple of 8 so that both run on the
-// same XCD (workgroups are dealt to the 8 XCDs in turn)
-constexpr int TOUCH_AHEAD = 448;
-
 __global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
     __shared__ u64 lds[LDS_WORDS];
     const int tid = threadIdx.x;
@@ -87,12 +83,6 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     u64 reg[16];
     u32 ok;
     fast_load<A2>(A, tile, tid, reg, ok);
-    // Warm the L2 for a workgroup that will run on this XCD a little later: after its own loads (loads return in
-    // order, so the touch must be the youngest) every thread reads one word of tile + TOUCH_AHEAD.  The slot that
-    // later loads that tile finds it in the L2 instead of waiting on HBM.  Measured on 1024 x 2^16 -> 2^18 with
-    // streaming stores: no touch 3.96 ms, distance 256 / 384 / 448 / 512 / 768 / 1024 tiles -> 3.75 / 3.63 / 3.56 /
-    // 3.58 / 3.79 / 3.87 ms (about 1024 workgroups are resident; further ahead and the lines are evicted before use).
-    const u64 touched = fast_touch<A2>(A, tile + (expand ? (TOUCH_AHEAD >> A.log_rho) : TOUCH_AHEAD), n_tiles, tid);
     if (!A.is_final) {
         if (lane < count) twi[first + lane] = tw_wave;
         __builtin_amdgcn_wave_barrier();
@@ -105,7 +95,6 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     fast_stage1<A2, INV>(A, tile, tid, t, ok, reg, twi, lds);
     __syncthreads();
     fast_stage2<A2, INV>(A, tile, tid, t, lds);
-    asm volatile("" ::"v"(touched));      // the touch load must not be optimised away; its value is unused
 }
 
 namespace {

@@ -21,8 +21,8 @@
 #include "ntt_pass.hpp"
 
 // Outputs of a pass are not read again by the launch that writes them: a non-temporal store keeps them
-// from displacing the lines the workgroups of the same launch have touched ahead for each other.
-#if defined(__HIP_DEVICE_COMPILE__)
+// from displacing the source lines that the coset workgroups of a tile share in the L2.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(VI_PLAIN_STORES)
 #define VI_STREAM_STORE(p, v) __builtin_nontemporal_store((v), (p))
 #else
 #define VI_STREAM_STORE(p, v) (*(p) = (v))
@@ -160,21 +160,6 @@ VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
         const u64 v = ((ok >> n1) & 1) ? reg[n1] : 0;
         reg[n1] = A.canon_src ? gl::canon(v) : v;
     }
-}
-
-// One word of one 128-byte line of tile `tile_ahead`'s source, chosen so that the 256 threads of a workgroup
-// touch every line of that tile once (strided pass: a line is a run of 16 columns of one point; final pass: a
-// line is 16 consecutive points of one column).
-// Returns the loaded word, or 0 when the tile does not exist; the caller keeps it alive, nothing uses it.
-template <int A2>
-VI_HD u64 fast_touch(const PassArgs &A, i64 tile_ahead, i64 n_tiles, int tid) {
-    if (tile_ahead >= n_tiles) return 0;
-    int c, n2;
-    s1_coords<A2>(A, tid, c, n2);
-    const ColRef R = col_ref(A, tile_ahead, c);
-    // strided pass: point (c mod 16) * E2 + n2 of column c; final pass: the first point of line n2 of column c
-    const i64 l = A.is_final ? (i64)16 * n2 : ((i64)(((c & 15) << A2) + n2) << A.logR);
-    return (R.valid && R.idx_base + l < A.src_width) ? A.src[R.src_base + l] : 0;
 }
 
 // phase 2: optional coset pre-multiplier, 16-point transform, w_L^(n2 k1), into LDS
