@@ -169,9 +169,18 @@ VI_HD Elem scatter_elem(const PassArgs &A, i64 tile, int e, int t_loop) {
 
 // phase 1: gather this thread's EPT source elements (zero beyond src_width)
 VI_HD void ph_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[EPT]) {
+    // every load is issued before the first value is used: an element that does not exist reads word 0
+    // of the source and is zeroed afterwards
+    bool ok[EPT];
+#pragma unroll
     for (int i = 0; i < EPT; ++i) {
         Elem E = gather_elem(A, tile, tid + i * NTHREADS);
-        u64 v = (E.valid && E.idx < A.src_width) ? A.src[E.addr] : 0;
+        ok[i] = E.valid && E.idx < A.src_width;
+        reg[i] = A.src[ok[i] ? E.addr : 0];
+    }
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+        const u64 v = ok[i] ? reg[i] : 0;
         reg[i] = A.canon_src ? gl::canon(v) : v;
     }
 }
