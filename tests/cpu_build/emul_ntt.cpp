@@ -46,8 +46,12 @@ void run_fast(const PassArgs &A) {
             fast_load<A2>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
         for (int t = 0; t < n_loop; ++t) {
             for (int tid = 0; tid < NTHREADS; ++tid)
+            {
+                u64 pw[16] = {};
+                if (A.pre) fast_pre_load<A2>(A, tile, tid, t, pw);
                 fast_stage1<A2, INV>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
-                                     A.twi, lds.data());
+                                     pw, A.twi, lds.data());
+            }
             for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV>(A, tile, tid, t, lds.data());
         }
     }

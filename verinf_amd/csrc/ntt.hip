@@ -80,8 +80,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
         for (int i = 0; i < (int)(sizeof(tw_mine) / sizeof(u64)); ++i)
             tw_mine[i] = (tid + i * NTHREADS < (16 << A2)) ? A.twi[tid + i * NTHREADS] : 0;
     }
-    u64 reg[16];
+    u64 reg[16], pw[16];
     u32 ok;
+    if (A.pre) fast_pre_load<A2>(A, tile, tid, t, pw);
     fast_load<A2>(A, tile, tid, reg, ok);
     if (!A.is_final) {
         if (lane < count) twi[first + lane] = tw_wave;
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
             if (tid + i * NTHREADS < (16 << A2)) twi[tid + i * NTHREADS] = tw_mine[i];
         __syncthreads();
     }
-    fast_stage1<A2, INV>(A, tile, tid, t, ok, reg, twi, lds);
+    fast_stage1<A2, INV>(A, tile, tid, t, ok, reg, pw, twi, lds);
     __syncthreads();
     fast_stage2<A2, INV>(A, tile, tid, t, lds);
 }

@@ -164,33 +164,36 @@ VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
 
 // phase 2: optional coset pre-multiplier, 16-point transform, w_L^(n2 k1), into LDS
 // twi: w_L^(n2 k1) at [n2 * 16 + k1]
+// the coset pre-multipliers of this thread's sixteen inputs (a column that does not exist takes those of
+// point 0 of coset 0; its data are zero); requested before the tile so that they are there when it arrives
+template <int A2>
+VI_HD void fast_pre_load(const PassArgs &A, i64 tile, int tid, int t_loop, u64 (&pw)[16]) {
+    int c, n2;
+    s1_coords<A2>(A, tid, c, n2);
+    const ColRef R = col_ref(A, tile, c);
+    const int sh = A.is_final ? 0 : A.logR;
+    const int t = A.is_final ? R.t : t_loop;
+    const u64 *pre = A.pre + (R.valid ? ((i64)t << A.logn) + R.idx_base : 0);
+#pragma unroll
+    for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[R.valid ? (i64)((n1 << A2) + n2) << sh : 0];
+}
+
 template <int A2, bool INV>
 VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok, const u64 (&reg)[16],
-                       const u64 *twi, u64 *lds) {
+                       const u64 (&pw)[16], const u64 *twi, u64 *lds) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
     u64 x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = reg[i];
+    fast_fix(A, ok, x);
     if (A.pre) {
-        const ColRef R = col_ref(A, tile, c);
-        const int sh = A.is_final ? 0 : A.logR;
-        const int t = A.is_final ? R.t : t_loop;
-        // all sixteen multipliers are requested before the data loads are waited for (a column that does not
-        // exist takes those of point 0 of coset 0; its data are zero)
-        const u64 *pre = A.pre + (R.valid ? ((i64)t << A.logn) + R.idx_base : 0);
-        u64 pw[16];
-#pragma unroll
-        for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[R.valid ? (i64)((n1 << A2) + n2) << sh : 0];
-        fast_fix(A, ok, x);
 #pragma unroll
         for (int g = 0; g < 16; g += 4) {
 #pragma unroll
             for (int n1 = g; n1 < g + 4; ++n1) x[n1] = gl::mul(x[n1], pw[n1]);
             VI_SCHED_FENCE();
         }
-    } else {
-        fast_fix(A, ok, x);
     }
     VI_SCHED_FENCE();
     dft_reg<4, INV>(x);
