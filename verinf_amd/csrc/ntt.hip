@@ -49,11 +49,8 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
     const int tid = threadIdx.x;
     // A pass that expands one source tile into rho cosets runs rho workgroups per tile, the coset being the low
     // bits of the workgroup id, so that the workgroups that read the same coefficients run at about the same time
-    // (3.394 vs 3.420 ms against the coset as grid.y); each of them re-reads the tile.  Measured alternatives, all slower:
-    //  * a loop over the cosets inside one workgroup: every address becomes loop-invariant,
-    //    ~50 more live registers, spills;
-    //  * persistent workgroups prefetching the next tile into a second register buffer: -3 %;
-    //  * two tiles per workgroup with both tiles' loads issued up front: -6 % (128 registers, spills);
+    // (3.394 vs 3.420 ms against the coset as grid.y); each of them re-reads the tile.  A loop over the cosets
+    // inside one workgroup was slower: every address becomes loop-invariant, ~50 more live registers, spills.
     const bool expand = !A.is_final && A.loop_cosets;
     const i64 n_tiles = expand ? (i64)(gridDim.x >> A.log_rho) : (i64)gridDim.x;
     i64 tile = expand ? (i64)(blockIdx.x >> A.log_rho) : (i64)blockIdx.x;
