@@ -32,10 +32,10 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 # WRITE_SIZE read by rocprofv3 in two counter runs of this script (3.80 GB read + 5.77 GB written per step),
 # each scaled by what the same counter reads for a 1 GiB device copy.  roofline.traffic is this figure divided
 # by the launches of a step, like roofline.achieved.
-LDE_TRAFFIC_BYTES_PER_STEP = 9.57e9
-# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU: 4 forward launches of 375.2 M and
-# 4 inverse launches of 85.3 M) and the rate at which 1024 SIMDs issue them at 2.4 GHz, one per four cycles
-LDE_VALU_INSTS_PER_STEP = 4 * 375_205_376 + 4 * 85_323_264
+LDE_TRAFFIC_BYTES_PER_STEP = 9.14e9
+# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU: 4 forward launches of 386.5 M and
+# 4 inverse launches of 87.7 M) and the rate at which 1024 SIMDs issue them at 2.4 GHz, one per four cycles
+LDE_VALU_INSTS_PER_STEP = 4 * 386_531_328 + 4 * 87_719_936
 VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / 4
 
 
