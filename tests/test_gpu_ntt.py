@@ -177,6 +177,25 @@ def test_lde_small_workspace_chunks_are_bit_identical(cp):
     assert rc == -3 and b"workspace" in L.vi_last_error()
 
 
+def test_lde_of_the_empty_message_through_the_c_abi():
+    """width = 0 (no source word exists, the pointer may be null): codewords and coefficients are zero,
+    written with the caller's row pitches; the slack beyond a row is left alone."""
+    from verinf_amd import _lib
+    L = _lib.lib()
+    K, N, m = 1 << 10, 1 << 12, 3
+    out = torch.full((m, N + 5), 7, dtype=torch.int64, device="cuda").view(torch.uint64)
+    coeffs = torch.full((m, K + 2), 9, dtype=torch.int64, device="cuda").view(torch.uint64)
+    ws = torch.empty(L.vi_coset_lde_min_workspace_bytes(K, N) * m, dtype=torch.uint8, device="cuda")
+    _lib.check(L.vi_coset_lde_coeffs(None, m, 0, 0, K, N, 7, coeffs.data_ptr(), K + 2, out.data_ptr(), N + 5,
+                                     ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    o, c = to_np(out), to_np(coeffs)
+    assert (o[:, :N] == 0).all() and (o[:, N:] == 7).all()
+    assert (c[:, :K] == 0).all() and (c[:, K:] == 9).all()
+    out2 = torch.full((m, N), 5, dtype=torch.int64, device="cuda").view(torch.uint64)
+    _lib.check(L.vi_coset_lde(None, m, 0, 0, K, N, 7, out2.data_ptr(), N, ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    assert int(out2.view(torch.int64).abs().sum().item()) == 0
+
+
 def test_lde_gates_and_layergkr_entry_points():
     from verinf_amd.layergkr import gpu, rs
     for cfg in (rs.Config(ELL=16, K_DEG=32, N_LIG=64, T_QUERIES=4),

@@ -283,6 +283,21 @@ int64_t vi_coset_lde_launches(int64_t m, int64_t K, int64_t N, size_t ws_bytes) 
 
 namespace {
 
+// m rows of `cols` zeros (row pitch `stride`)
+__global__ __launch_bounds__(NTHREADS) void k_zero_rows(u64 *dst, i64 m, i64 cols, i64 stride) {
+    const i64 total = m * cols;
+    for (i64 e = (i64)blockIdx.x * NTHREADS + threadIdx.x; e < total; e += (i64)gridDim.x * NTHREADS)
+        dst[(e / cols) * stride + (e % cols)] = 0;
+}
+
+int zero_rows(u64 *dst, i64 m, i64 cols, i64 stride, hipStream_t s) {
+    i64 blocks = (m * cols + NTHREADS - 1) / NTHREADS;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(k_zero_rows, dim3((unsigned)blocks), dim3(NTHREADS), 0, s, dst, m, cols, stride);
+    VI_LAUNCH_CHECK("k_zero_rows");
+    return VI_OK;
+}
+
 // values (or coefficients) -> optional coefficients -> optional codewords, chunked over rows
 int coset_lde_impl(const char *who, const uint64_t *in, int64_t m, int64_t width, int64_t in_stride, int64_t K,
                    int64_t N, uint64_t shift, uint64_t *out, int64_t out_stride, uint64_t *coeffs,
@@ -295,7 +310,15 @@ int coset_lde_impl(const char *who, const uint64_t *in, int64_t m, int64_t width
                         (long long)m, (long long)width, (long long)in_stride, (long long)out_stride, (long long)coeffs_stride);
     if (shift == 0 || shift >= gl::P) return vi::fail(VI_EINVAL, "%s: shift must be in [1, p)", who);
     if (m == 0) return VI_OK;
-    if (!in || (!out && !coeffs)) return vi::fail(VI_EINVAL, "%s: null pointer", who);
+    if ((!in && width > 0) || (!out && !coeffs)) return vi::fail(VI_EINVAL, "%s: null pointer", who);
+    if (width == 0) {
+        // the empty message is the zero polynomial; the kernels are not run on it (they read word 0 of the
+        // source in place of every element that does not exist, and here there is no word 0)
+        int rc = VI_OK;
+        if (coeffs && !in_is_coeffs) rc = zero_rows(coeffs, m, K, coeffs_stride, (hipStream_t)stream);
+        if (!rc && out) rc = zero_rows(out, m, N, out_stride, (hipStream_t)stream);
+        return rc;
+    }
     const int logK = vi::ilog2(K), logN = vi::ilog2(N);
     size_t one = (size_t)lde_ws_elems(logK, logN, 1) * sizeof(u64);
     i64 chunk = (i64)(ws_bytes / one);
