@@ -92,6 +92,7 @@ int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, 
  * w_K^c (slots [width, K) read as zero);  row r of `out` receives its N values at
  * shift * w_N^j.  K, N powers of two, 2 <= K <= N.  `in` rows are in_stride
  * elements apart, `out` rows out_stride >= N.  in and out must not overlap.
+ * width = 0 is the zero polynomial: zero rows are written and `in` is not read.
  * The workspace may be smaller than vi_coset_lde_workspace_bytes(m, K, N): rows
  * are then processed in chunks; vi_coset_lde_min_workspace_bytes(K, N) is the
  * least that is accepted (one row). */
