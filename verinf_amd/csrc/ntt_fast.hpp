@@ -155,10 +155,15 @@ VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &
 
 // zero for the elements that do not exist, caller data reduced mod p
 VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
+    // both as blocks behind one test each, so that the passes that need neither (all elements there, source
+    // written by an earlier pass) skip them: as per-element selects they ran in every pass
+    if (ok != 0xFFFFu) {
 #pragma unroll
-    for (int n1 = 0; n1 < 16; ++n1) {
-        const u64 v = ((ok >> n1) & 1) ? reg[n1] : 0;
-        reg[n1] = A.canon_src ? gl::canon(v) : v;
+        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = ((ok >> n1) & 1) ? reg[n1] : 0;
+    }
+    if (A.canon_src) {
+#pragma unroll
+        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = gl::canon(reg[n1]);
     }
 }
 
