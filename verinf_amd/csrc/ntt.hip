@@ -42,8 +42,13 @@ __global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
 
 // Register-blocked pass for digits of 2^5 .. 2^8 points (ntt_fast.hpp): one LDS
 // crossing, shift-only butterflies, 16 elements per thread held in registers.
-template <int A2, bool INV>
-__global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A) {
+// FIN: compiled for the final (transposing) pass only, without the strided passes' addressing (110 instead of
+// 120 registers).  The strided passes keep the run-time flag: compiled with it fixed to 0 they took 128
+// registers and spilled.
+template <int A2, bool INV, bool FIN>
+__global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
+    PassArgs A = A_in;
+    if (FIN) A.is_final = 1;
     __shared__ u64 lds[TILE + (16 << A2)];
     __shared__ u64 twi[16 << A2];
     const int tid = threadIdx.x;
@@ -186,6 +191,25 @@ int get_pre(int logK, int logN, u64 shift, const u64 **out) {
     return VI_OK;
 }
 
+template <int A2>
+void launch_fast_a(const PassArgs &A, dim3 grid, dim3 block, hipStream_t s) {
+    switch ((A.inverse ? 2 : 0) + (A.is_final ? 1 : 0)) {
+        case 0: hipLaunchKernelGGL((k_ntt_fast<A2, false, false>), grid, block, 0, s, A); break;
+        case 1: hipLaunchKernelGGL((k_ntt_fast<A2, false, true>), grid, block, 0, s, A); break;
+        case 2: hipLaunchKernelGGL((k_ntt_fast<A2, true, false>), grid, block, 0, s, A); break;
+        default: hipLaunchKernelGGL((k_ntt_fast<A2, true, true>), grid, block, 0, s, A); break;
+    }
+}
+
+void launch_fast(const PassArgs &A, dim3 grid, dim3 block, hipStream_t s) {
+    switch (A.a - FAST_A1) {
+        case 1: launch_fast_a<1>(A, grid, block, s); break;
+        case 2: launch_fast_a<2>(A, grid, block, s); break;
+        case 3: launch_fast_a<3>(A, grid, block, s); break;
+        default: launch_fast_a<4>(A, grid, block, s); break;
+    }
+}
+
 int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
     for (const PassArgs &A : passes) {
         i64 tiles = pass_tiles(A);
@@ -194,16 +218,7 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
         dim3 grid((unsigned)tiles), block(NTHREADS);
         if (fast_ok(A.a) && A.twi) {
             if (!A.is_final && A.loop_cosets) grid.x <<= A.log_rho;       // tiles * rho <= 2^31 by max_rows_per_launch
-            switch ((A.a - FAST_A1) * 2 + (A.inverse ? 1 : 0)) {
-                case 2: hipLaunchKernelGGL((k_ntt_fast<1, false>), grid, block, 0, s, A); break;
-                case 3: hipLaunchKernelGGL((k_ntt_fast<1, true>), grid, block, 0, s, A); break;
-                case 4: hipLaunchKernelGGL((k_ntt_fast<2, false>), grid, block, 0, s, A); break;
-                case 5: hipLaunchKernelGGL((k_ntt_fast<2, true>), grid, block, 0, s, A); break;
-                case 6: hipLaunchKernelGGL((k_ntt_fast<3, false>), grid, block, 0, s, A); break;
-                case 7: hipLaunchKernelGGL((k_ntt_fast<3, true>), grid, block, 0, s, A); break;
-                case 8: hipLaunchKernelGGL((k_ntt_fast<4, false>), grid, block, 0, s, A); break;
-                default: hipLaunchKernelGGL((k_ntt_fast<4, true>), grid, block, 0, s, A); break;
-            }
+            launch_fast(A, grid, block, s);
         } else {
             hipLaunchKernelGGL(k_ntt_pass, grid, block, 0, s, A);
         }
