@@ -33,9 +33,9 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 # each scaled by what the same counter reads for a 1 GiB device copy.  roofline.traffic is this figure divided
 # by the launches of a step, like roofline.achieved.
 LDE_TRAFFIC_BYTES_PER_STEP = 9.14e9
-# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU: 4 forward launches of 386.5 M and
-# 4 inverse launches of 87.7 M) and the rate at which 1024 SIMDs issue them at 2.4 GHz, one per four cycles
-LDE_VALU_INSTS_PER_STEP = 4 * 386_531_328 + 4 * 87_719_936
+# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU: per 512-row chunk 433.7 M + 285.7 M in the
+# two forward launches and 92.8 M + 71.3 M in the two inverse ones) and the rate at which 1024 SIMDs issue them at 2.4 GHz, one per four cycles
+LDE_VALU_INSTS_PER_STEP = 2 * (433_717_248 + 285_736_960 + 92_766_208 + 71_335_936)
 VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / 4
 
 
