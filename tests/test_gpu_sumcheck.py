@@ -250,6 +250,29 @@ def test_verifier_accepts_and_rejects_device_table_proofs(mods):
     assert not ok and "terminal" in why
 
 
+def test_baseline_shape_three_tables_of_2p26(mods):
+    """The benchmark instance at full size (three tables of 2^26, degree 3, 26 rounds), through the
+    properties that do not need a CPU run: the claim is the sum of the elementwise product, every
+    round satisfies S(0) + S(1) = previous claim, and the last claim equals the product of the three
+    multilinear extensions at the challenge point (all checked by the verifier, the terminal values
+    on the device); a tampered table is rejected."""
+    gpu, sc = mods
+    v = 26
+    g = torch.Generator(device="cuda").manual_seed(26)
+    tabs = [torch.randint(0, 1 << 62, (1 << v,), generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
+            for _ in range(3)]
+    coins = [random.Random(5).randrange(P) for _ in range(v)]
+    terms = [(1, tabs)]
+    proof = sc.prove_terms(terms, lambda i: coins[i])
+    assert len(proof.round_polys) == v and all(len(s) == 4 for s in proof.round_polys)
+    assert proof.claim == int(gpu.gl_sum(cp_mul(cp_mul(tabs[0], tabs[1]), tabs[2])).cpu().item())
+    ok, why = sc.verify_terms(proof, terms, lambda i: coins[i])
+    assert ok, why
+    tabs[1].view(torch.int64)[(1 << v) - 3] += 1
+    ok, why = sc.verify_terms(proof, terms, lambda i: coins[i])
+    assert not ok and "terminal" in why
+
+
 def cp_mul(x, y):
     from verinf_amd.prover import cuda_primitives as cp
     return cp.gl_mul(x, y)
