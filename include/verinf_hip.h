@@ -209,7 +209,11 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
  * vi_merkle_level replaces merkle_one_level + the odd-node duplication around it
  * (prover/cuda_primitives.py:1388-1402, layergkr/rs.py:135-144): out[i] = BLAKE3(nodes[2i] ||
  * nodes[2i+1]) over 32-byte nodes, the odd last node paired with itself; out holds
- * ceil(count / 2) nodes.  nodes and out must not overlap. */
+ * ceil(count / 2) nodes.  nodes and out must not overlap.
+ *
+ * vi_merkle_tree builds every level above `count` leaves with up to nine levels per launch (the loop of
+ * merkle_build_blake3, prover/cuda_primitives.py:1388-1402): levels_out receives level 1 (ceil(count/2)
+ * nodes), then level 2, ... up to the root, vi_merkle_tree_nodes(count) nodes of 32 bytes in all. */
 size_t vi_hash_columns_workspace_bytes(int64_t m, int64_t n);
 int vi_hash_columns(const uint64_t *mat, int64_t m, int64_t n, int64_t row_stride, uint8_t *digests, void *ws,
                     size_t ws_bytes, void *stream);
@@ -218,6 +222,8 @@ int vi_hash_columns_update(const uint64_t *rows, int64_t slab_rows, int64_t n, i
 int vi_hash_columns_finalize(int64_t n, int64_t n_chunks_total, void *ws, size_t ws_bytes, uint8_t *digests,
                              void *stream);
 int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *stream);
+int64_t vi_merkle_tree_nodes(int64_t count);
+int vi_merkle_tree(const uint8_t *leaves, int64_t count, uint8_t *levels_out, void *stream);
 
 /* Zero-knowledge pad generator; replaces row_prg / row_prg_indexed (prover/cuda_primitives.py:1262-1294,
  * kernels :877-930): out[r * out_stride + k] = (BLAKE3(seed[32] || row_le8 || k_le8)[0:8] as a little-endian

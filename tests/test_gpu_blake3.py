@@ -97,7 +97,9 @@ def test_accumulator_requires_all_rows(cp):
         cp.MerkleColumnAccumulator(4, 128)
 
 
-@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 31, 32, 33, 1000, 4097, 65536])
+# counts around the 512-leaf blocks of the fused tree kernel and around its nine levels per launch
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 31, 32, 33, 511, 512, 513, 1000, 1023, 1025, 4097, 65536, 65537,
+                               262143, 262144, 262147, 524289])
 def test_merkle_build_matches_oracle(cp, k):
     rng = np.random.default_rng(k)
     leaves = rng.integers(0, 256, (k, 32), dtype=np.uint8)
@@ -107,6 +109,11 @@ def test_merkle_build_matches_oracle(cp, k):
     for g, w in zip(levels, want):
         assert np.array_equal(to_np(g), w)
     assert to_np(root).tobytes() == want[-1][0].tobytes()
+    # the level-by-level entry point gives the same nodes
+    cur = to_dev(leaves)
+    for w in want[1:]:
+        cur = cp.merkle_one_level(cur)
+        assert np.array_equal(to_np(cur), w)
 
 
 def test_commit_root_and_openings(cp):

@@ -28,7 +28,7 @@ EXPORTS = [
     "vi_kquant_to_field_transposed",
     "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval", "vi_sumcheck_prove",
     "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
-    "vi_merkle_level", "vi_row_prg",
+    "vi_merkle_level", "vi_merkle_tree_nodes", "vi_merkle_tree", "vi_row_prg",
     "vi_eq_vector", "vi_mle_eval_workspace_bytes", "vi_mle_eval",
     "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities",
 ]
@@ -96,6 +96,9 @@ def lib():
     L.vi_hash_columns_update.argtypes = [vp, i64, i64, i64, i64, i64, vp, sz, vp]
     L.vi_hash_columns_finalize.argtypes = [i64, i64, vp, sz, vp, vp]
     L.vi_merkle_level.argtypes = [vp, i64, vp, vp]
+    L.vi_merkle_tree_nodes.restype = i64
+    L.vi_merkle_tree_nodes.argtypes = [i64]
+    L.vi_merkle_tree.argtypes = [vp, i64, vp, vp]
     L.vi_row_prg.argtypes = [vp, vp, i64, i64, i64, vp, i64, vp]
     L.vi_challenge.argtypes = [vp, vp, c_int, vp, i64, vp, vp]
     L.vi_gl_spmv.argtypes = [vp, vp, vp, i64, i64, vp, vp, vp, c_int, vp, vp]
@@ -110,7 +113,7 @@ def lib():
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
                  "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_kquant_to_field_transposed", "vi_sumcheck_eval",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
-                 "vi_merkle_level", "vi_row_prg", "vi_eq_vector", "vi_mle_eval",
+                 "vi_merkle_level", "vi_merkle_tree_nodes", "vi_merkle_tree", "vi_row_prg", "vi_eq_vector", "vi_mle_eval",
                  "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities"):
         getattr(L, name).restype = c_int
     _lib = L

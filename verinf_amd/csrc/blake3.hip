@@ -151,6 +151,50 @@ __global__ __launch_bounds__(BLOCK) void k_merkle_level(const u32 *__restrict__ 
     for (int k = 0; k < 8; ++k) out[i * 8 + k] = cv[k];
 }
 
+// Up to SUB_LEVELS Merkle levels in one launch.  A workgroup owns 2^SUB_LEVELS consecutive nodes of the input
+// level, builds the parents of every level above them that lies inside its block (children of a block-aligned
+// node are in the block too), keeps the newest level in LDS for the next one and writes every level to `out`:
+// level j (1-based) of this launch starts at out + 8 * (c_1 + ... + c_{j-1}) words, c_j = ceil(c_{j-1} / 2),
+// c_0 = count.  The odd last node of a level is paired with itself, as in k_merkle_level.
+constexpr int SUB_LEVELS = 9;
+
+__global__ __launch_bounds__(BLOCK) void k_merkle_subtree(const u32 *__restrict__ nodes, i64 count, int levels, u32 *__restrict__ out) {
+    __shared__ u32 buf[2][BLOCK * 8];
+    const i64 base = (i64)blockIdx.x << SUB_LEVELS;            // first input node of the block
+    i64 c_prev = count, off = 0;                               // nodes of the level below, word offset of this level in out
+    for (int j = 1; j <= levels; ++j) {
+        const i64 c = (c_prev + 1) >> 1;
+        const i64 first = base >> j;                           // first node of level j in the block
+        const int in_block = 1 << (SUB_LEVELS - j);
+        const i64 i = first + threadIdx.x;
+        if ((int)threadIdx.x < in_block && i < c) {
+            u32 m[16], cv[8];
+            const bool has_right = 2 * i + 1 < c_prev;
+            if (j == 1) {
+                const u32 *l = nodes + (2 * i) * 8;
+                const u32 *r = nodes + (has_right ? 2 * i + 1 : 2 * i) * 8;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) { m[k] = l[k]; m[8 + k] = r[k]; }
+            } else {
+                const u32 *l = buf[j & 1] + (2 * threadIdx.x) * 8;
+                const u32 *r = buf[j & 1] + (has_right ? 2 * threadIdx.x + 1 : 2 * threadIdx.x) * 8;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) { m[k] = l[k]; m[8 + k] = r[k]; }
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) cv[k] = IV[k];
+            compress(cv, m, 0, 64, CHUNK_START | CHUNK_END | ROOT);
+            u32 *o = out + off + i * 8;
+            u32 *keep = buf[(j + 1) & 1] + threadIdx.x * 8;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { o[k] = cv[k]; keep[k] = cv[k]; }
+        }
+        __syncthreads();
+        off += c * 8;
+        c_prev = c;
+    }
+}
+
 // Zero-knowledge pad generator (prover/cuda_primitives.py:870-930, k_row_prg / k_row_prg_indexed):
 //   out[r][k] = (first 8 bytes of BLAKE3(seed[32] || row_le8 || k_le8), little-endian) mod p.
 // The 48-byte message is a single block, so a value costs one compression, of which only the
@@ -347,6 +391,35 @@ int vi_merkle_level(const uint8_t *nodes, int64_t count, uint8_t *out, void *str
     hipLaunchKernelGGL(k_merkle_level, dim3((unsigned)((parents + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, (hipStream_t)stream,
                        (const u32 *)nodes, (i64)count, (u32 *)out);
     VI_LAUNCH_CHECK("k_merkle_level");
+    return VI_OK;
+}
+
+int64_t vi_merkle_tree_nodes(int64_t count) {
+    int64_t total = 0;
+    for (int64_t c = count; c > 1;) { c = (c + 1) / 2; total += c; }
+    return count < 1 ? 0 : total;
+}
+
+int vi_merkle_tree(const uint8_t *leaves, int64_t count, uint8_t *levels_out, void *stream) {
+    if (count < 1 || !leaves) return vi::fail(VI_EINVAL, "vi_merkle_tree: bad arguments");
+    if (count == 1) return VI_OK;
+    if (!levels_out) return vi::fail(VI_EINVAL, "vi_merkle_tree: null output");
+    if (((uintptr_t)leaves | (uintptr_t)levels_out) & 3) return vi::fail(VI_EINVAL, "vi_merkle_tree: nodes must be 4-byte aligned");
+    const u32 *cur = (const u32 *)leaves;
+    u32 *out = (u32 *)levels_out;
+    i64 c = count;
+    while (c > 1) {
+        int levels = 0;
+        i64 written = 0, cl = c;
+        while (cl > 1 && levels < SUB_LEVELS) { cl = (cl + 1) / 2; written += cl; ++levels; }
+        const i64 blocks = (c + ((i64)1 << SUB_LEVELS) - 1) >> SUB_LEVELS;
+        if (blocks > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "vi_merkle_tree: too many leaves");
+        hipLaunchKernelGGL(k_merkle_subtree, dim3((unsigned)blocks), dim3(BLOCK), 0, (hipStream_t)stream, cur, c, levels, out);
+        VI_LAUNCH_CHECK("k_merkle_subtree");
+        cur = out + (written - cl) * 8;                       // the last level written is the next input
+        out += written * 8;
+        c = cl;
+    }
     return VI_OK;
 }
 

@@ -572,14 +572,23 @@ def merkle_one_level(nodes):
 def merkle_build_blake3(leaves):
     """(N, 32) uint8 leaves -> (root: (32,) uint8, levels: list of (k_i, 32) uint8);
     levels[0] = leaves, levels[-1] = (1, 32) holding the root
-    (prover/cuda_primitives.py:1388-1402)."""
+    (prover/cuda_primitives.py:1388-1402).  All levels above the leaves are built by one library
+    call (up to nine levels per launch) into one buffer; the list holds views of it."""
     assert leaves.dim() == 2 and leaves.size(1) == 32
     assert leaves.dtype == torch.uint8 and leaves.is_cuda
-    levels = [leaves]
     cur = leaves.contiguous()
-    while cur.size(0) > 1:
-        cur = merkle_one_level(cur)
-        levels.append(cur)
+    levels = [leaves]
+    k = int(cur.size(0))
+    if k > 1:
+        L = _lib.lib()
+        buf = torch.empty((int(L.vi_merkle_tree_nodes(k)), 32), dtype=torch.uint8, device=cur.device)
+        with torch.cuda.device(cur.device):
+            _lib.check(L.vi_merkle_tree(cur.data_ptr(), k, buf.data_ptr(), _lib.stream_ptr()))
+        off = 0
+        while k > 1:
+            k = (k + 1) // 2
+            levels.append(buf[off:off + k])
+            off += k
     root = levels[-1].view(-1)[:32].clone()
     return root, levels
 
