@@ -13,6 +13,8 @@
 #pragma once
 #include <stdint.h>
 
+#include <type_traits>
+
 #if defined(__HIPCC__)
 #include <hip/hip_runtime.h>
 #define VI_HD __host__ __device__ __forceinline__
@@ -38,6 +40,172 @@ namespace gl {
 constexpr u64 P = 0xFFFFFFFF00000001ull;
 constexpr u64 EPS = 0xFFFFFFFFull;   // 2^32 - 1 = 2^64 mod p
 
+#if defined(__HIP_DEVICE_COMPILE__)
+// Hand-scheduled gfx950 sequences.  Written from 64-bit C++ the compiler spends a 64-bit compare (two issue
+// slots) and two selects on every carry test and builds register pairs with moves: 29 VALU instructions (42
+// issue slots) for a product, 7 (11) for a modular sum.  On 32-bit halves with explicit carries the same
+// functions are 19 (24), 6 and 5.  On this chip a VALU instruction that reads a carry or mask needs two
+// wait states after the VALU instruction that wrote it; inside an asm block the assembler does not add
+// them, so every such pair below is separated by two instructions or an s_nop.  s_or_b64 also writes SCC, which the
+// compiler may be holding a loop condition in: the blocks that use it say so in their clobber lists.  A carry that leaves a
+// block in an SGPR pair is only read by a scalar instruction, or by a vector instruction at least two
+// instructions into the next block.
+namespace dev {
+
+__device__ __forceinline__ u64 pack(u32 lo, u32 hi) { return ((u64)hi << 32) | lo; }
+
+// w, plus 2^64 when the carry `cin` is set, lies in [0, 2p): subtract p when it is >= p.
+// r = w + (2^32 - 1) mod 2^64 is that difference, and it is the answer exactly when one of the two additions wrapped.
+__device__ __forceinline__ u64 canon_tail(u32 w0, u32 w1, u64 cin) {
+    u32 r0, r1;
+    asm("v_add_co_u32 %[r0], vcc, -1, %[w0]\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[r1], vcc, 0, %[w1], vcc\n\t"
+        "s_or_b64 vcc, vcc, %[cin]\n\t"
+        "v_cndmask_b32 %[r0], %[w0], %[r0], vcc\n\t"
+        "v_cndmask_b32 %[r1], %[w1], %[r1], vcc"
+        : [r0] "=&v"(r0), [r1] "=&v"(r1)
+        : [w0] "v"(w0), [w1] "v"(w1), [cin] "s"(cin)
+        : "vcc", "scc");
+    return pack(r0, r1);
+}
+
+__device__ __forceinline__ u64 addc(u64 a, u64 b) {
+    u32 a0 = (u32)a, a1 = (u32)(a >> 32), b0 = (u32)b, b1 = (u32)(b >> 32);
+    u32 s0, s1, r0, r1;
+    u64 st;
+    asm("v_add_co_u32 %[s0], vcc, %[a0], %[b0]\n\t"
+        "v_add_co_u32 %[r0], %[st], -1, %[s0]\n\t"
+        "s_nop 0\n\t"
+        "v_addc_co_u32 %[s1], vcc, %[a1], %[b1], vcc\n\t"
+        "v_addc_co_u32 %[r1], %[st], 0, %[s1], %[st]\n\t"
+        "s_or_b64 vcc, vcc, %[st]\n\t"
+        "v_cndmask_b32 %[r0], %[s0], %[r0], vcc\n\t"
+        "v_cndmask_b32 %[r1], %[s1], %[r1], vcc"
+        : [s0] "=&v"(s0), [s1] "=&v"(s1), [r0] "=&v"(r0), [r1] "=&v"(r1), [st] "=&s"(st)
+        : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1)
+        : "vcc", "scc");
+    return pack(r0, r1);
+}
+
+// a - b, minus 2^32 - 1 more when it borrowed (the mask -borrow is that constant)
+__device__ __forceinline__ u64 sub(u64 a, u64 b) {
+    u32 a0 = (u32)a, a1 = (u32)(a >> 32), b0 = (u32)b, b1 = (u32)(b >> 32);
+    u32 d0, d1, m;
+    asm("v_sub_co_u32 %[d0], vcc, %[a0], %[b0]\n\t"
+        "s_nop 1\n\t"
+        "v_subb_co_u32 %[d1], vcc, %[a1], %[b1], vcc\n\t"
+        "s_nop 1\n\t"
+        "v_subb_co_u32 %[m], vcc, %[d0], %[d0], vcc\n\t"
+        "v_sub_co_u32 %[d0], vcc, %[d0], %[m]\n\t"
+        "s_nop 1\n\t"
+        "v_subbrev_co_u32 %[d1], vcc, 0, %[d1], vcc"
+        : [d0] "=&v"(d0), [d1] "=&v"(d1), [m] "=&v"(m)
+        : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1)
+        : "vcc");
+    return pack(d0, d1);
+}
+
+__device__ __forceinline__ u64 canon(u64 x) {
+    u32 x0 = (u32)x, x1 = (u32)(x >> 32), r0, r1;
+    asm("v_add_co_u32 %[r0], vcc, -1, %[x0]\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[r1], vcc, 0, %[x1], vcc\n\t"
+        "s_nop 1\n\t"
+        "v_cndmask_b32 %[r0], %[x0], %[r0], vcc\n\t"
+        "v_cndmask_b32 %[r1], %[x1], %[r1], vcc"
+        : [r0] "=&v"(r0), [r1] "=&v"(r1)
+        : [x0] "v"(x0), [x1] "v"(x1)
+        : "vcc");
+    return pack(r0, r1);
+}
+
+// (hi:lo) given as four words l0 l1 hl hh -> [0, p):  lo - hh + hl (2^32 - 1)
+__device__ __forceinline__ u64 reduce_words(u32 l0, u32 l1, u32 hl, u32 hh) {
+    u32 x0, x1, m;
+    asm("v_sub_co_u32 %[x0], vcc, %[l0], %[hh]\n\t"
+        "s_nop 1\n\t"
+        "v_subbrev_co_u32 %[x1], vcc, 0, %[l1], vcc\n\t"
+        "s_nop 1\n\t"
+        "v_subb_co_u32 %[m], vcc, %[x0], %[x0], vcc\n\t"
+        "v_sub_co_u32 %[x0], vcc, %[x0], %[m]\n\t"
+        "s_nop 1\n\t"
+        "v_subbrev_co_u32 %[x1], vcc, 0, %[x1], vcc"
+        : [x0] "=&v"(x0), [x1] "=&v"(x1), [m] "=&v"(m)
+        : [l0] "v"(l0), [l1] "v"(l1), [hh] "v"(hh)
+        : "vcc");
+    u64 w, st;
+    asm("v_mad_u64_u32 %[w], %[st], %[hl], -1, %[x]"
+        : [w] "=&v"(w), [st] "=&s"(st)
+        : [hl] "v"(hl), [x] "v"(pack(x0, x1)));
+    return canon_tail((u32)w, (u32)(w >> 32), st);
+}
+
+__device__ __forceinline__ u64 mul(u64 a, u64 b) {
+    u32 a0 = (u32)a, a1 = (u32)(a >> 32), b0 = (u32)b, b1 = (u32)(b >> 32);
+    u64 p00, mm, p11, st;
+    asm("v_mad_u64_u32 %[p00], vcc, %[a0], %[b0], 0\n\t"
+        "v_mad_u64_u32 %[mm], vcc, %[a1], %[b0], 0\n\t"
+        "v_mad_u64_u32 %[p11], vcc, %[a1], %[b1], 0\n\t"
+        "v_mad_u64_u32 %[mm], %[st], %[a0], %[b1], %[mm]"
+        : [p00] "=&v"(p00), [mm] "=&v"(mm), [p11] "=&v"(p11), [st] "=&s"(st)
+        : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1)
+        : "vcc");
+    // words of the 128-bit product: p00.lo, p00.hi + mm.lo, p11.lo + mm.hi + carry, p11.hi + carry + (carry of the cross sum)
+    u32 w1 = (u32)(p00 >> 32), hl, hh;
+    asm("v_add_co_u32 %[w1], vcc, %[w1], %[m0]\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[hl], vcc, %[q0], %[m1], vcc\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[hh], vcc, 0, %[q1], vcc\n\t"
+        "v_addc_co_u32 %[hh], vcc, 0, %[hh], %[st]"
+        : [w1] "+v"(w1), [hl] "=&v"(hl), [hh] "=&v"(hh)
+        : [m0] "v"((u32)mm), [m1] "v"((u32)(mm >> 32)), [q0] "v"((u32)p11), [q1] "v"((u32)(p11 >> 32)), [st] "s"(st)
+        : "vcc");
+    return reduce_words((u32)p00, w1, hl, hh);
+}
+
+// canonical v times 2^E, 0 <= E < 96, canonical result; s = 32 q + r moves v into limbs m0 m1 m2 at phi^q
+template <int E>
+__device__ __forceinline__ u64 mul_pow2(u64 v) {
+    static_assert(E >= 0 && E < 96, "shift out of range");
+    if (E == 0) return v;
+    constexpr int q = E >> 5, r = E & 31;
+    const u32 v0 = (u32)v, v1 = (u32)(v >> 32);
+    const u32 m0 = v0 << r;
+    const u32 m1 = r ? __builtin_amdgcn_alignbit(v1, v0, (32 - r) & 31) : v1;
+    const u32 m2 = r ? (v1 >> ((32 - r) & 31)) : 0u;
+    if (q == 0) {
+        // m0 + m1 phi + m2 phi^2 = (m1:m0) + m2 (2^32 - 1)
+        u64 w, st;
+        asm("v_mad_u64_u32 %[w], %[st], %[m2], -1, %[x]"
+            : [w] "=&v"(w), [st] "=&s"(st)
+            : [m2] "v"(m2), [x] "v"(pack(m0, m1)));
+        return canon_tail((u32)w, (u32)(w >> 32), st);
+    } else if (q == 1) {
+        // m0 phi + m1 phi^2 + m2 phi^3 = (m0:0) + m1 (2^32 - 1) - m2
+        u64 w, st;
+        asm("v_mad_u64_u32 %[w], %[st], %[m1], -1, %[x]"
+            : [w] "=&v"(w), [st] "=&s"(st)
+            : [m1] "v"(m1), [x] "v"(pack(0u, m0)));
+        const u64 x = canon_tail((u32)w, (u32)(w >> 32), st);
+        return r ? sub(x, (u64)m2) : x;
+    } else {
+        // m0 phi^2 + m1 phi^3 + m2 phi^4 = m0 (2^32 - 1) - (m2:m1); both operands are below p
+        u32 e0, e1;
+        asm("v_sub_co_u32 %[e0], vcc, 0, %[m0]\n\t"
+            "s_nop 1\n\t"
+            "v_subbrev_co_u32 %[e1], vcc, 0, %[m0], vcc"
+            : [e0] "=&v"(e0), [e1] "=&v"(e1)
+            : [m0] "v"(m0)
+            : "vcc");
+        return sub(pack(e0, e1), pack(m1, m2));
+    }
+}
+
+}  // namespace dev
+#endif
+
 VI_HD u64 add(u64 a, u64 b) {
     u64 s = a + b;
     if (s < a) s += EPS;             // wrapped past 2^64: add 2^64 mod p
@@ -46,6 +214,9 @@ VI_HD u64 add(u64 a, u64 b) {
 }
 
 VI_HD u64 sub(u64 a, u64 b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::sub(a, b);
+#endif
     u64 d = a - b;
     if (a < b) d -= EPS;             // borrowed 2^64: take 2^64 mod p back out
     return d;
@@ -57,6 +228,9 @@ VI_HD u64 neg(u64 a) { return a == 0 ? 0 : P - a; }
 // overshoot past p take the same correction, + (2^32 - 1) mod 2^64, so one select
 // serves both).  Not for arbitrary words: with both operands >= p it can be wrong.
 VI_HD u64 addc(u64 a, u64 b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::addc(a, b);
+#endif
     u64 s = a + b;
     u64 r = s + EPS;
     return ((s < a) | (r < s)) ? r : s;
@@ -64,12 +238,18 @@ VI_HD u64 addc(u64 a, u64 b) {
 
 // x mod p for an arbitrary 64-bit word
 VI_HD u64 canon(u64 x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::canon(x);
+#endif
     u64 r = x + EPS;
     return (r < x) ? r : x;
 }
 
 // (hi:lo) -> [0, p).  hi = hh*2^32 + hl  =>  value = lo - hh + hl*(2^32 - 1).
 VI_HD u64 reduce128(u64 lo, u64 hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::reduce_words((u32)lo, (u32)(lo >> 32), (u32)hi, (u32)(hi >> 32));
+#endif
     u32 hh = (u32)(hi >> 32), hl = (u32)hi;
     u64 t0 = lo - hh;
     if (lo < hh) t0 -= EPS;
@@ -105,6 +285,9 @@ VI_HD void mul_wide(u64 a, u64 b, u64 &lo, u64 &hi) {
 }
 
 VI_HD u64 mul(u64 a, u64 b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::mul(a, b);
+#endif
     u64 lo, hi;
     mul_wide(a, b, lo, hi);
     return reduce128(lo, hi);
@@ -112,6 +295,9 @@ VI_HD u64 mul(u64 a, u64 b) {
 
 // product as a non-canonical word (see reduce128_lazy): for chains of multiplications
 VI_HD u64 mul_lazy(u64 a, u64 b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::mul(a, b);           // the scheduled canonical product is shorter than a lazy one written in C++
+#endif
     u64 lo, hi;
     mul_wide(a, b, lo, hi);
     return reduce128_lazy(lo, hi);
@@ -167,4 +353,23 @@ VI_HD u64 mul_pow2(u64 x, u32 s) {
     return sub(sub(pos, negv), small);
 }
 
+// the same with the exponent fixed at compile time
+template <int E>
+VI_HD u64 mul_pow2c(u64 x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::mul_pow2<E>(x);
+#else
+    return mul_pow2(x, (u32)E);
+#endif
+}
+
 }  // namespace gl
+
+// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N)
+template <int I0, int N, class F>
+VI_HD void static_for(F &&f) {
+    if constexpr (I0 < N) {
+        f(std::integral_constant<int, I0>{});
+        static_for<I0 + 1, N>(f);
+    }
+}

@@ -45,35 +45,33 @@ VI_HD constexpr int brev(int i) {
 }
 
 // in-register transform of 2^A points, natural order in and out; inputs must be
-// canonical, outputs are canonical
+// canonical, outputs are canonical.  Every exponent is a compile-time constant, so a
+// twiddle is two or three fixed shifts and one fold (gl::mul_pow2c).
 template <int A, bool INV>
 VI_HD void dft_reg(u64 (&x)[1 << A]) {
     constexpr int N = 1 << A;
     u64 y[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) y[i] = x[brev<A>(i)];
-#pragma unroll
-    for (int s = 0; s < A; ++s) {
-#pragma unroll
-        for (int b = 0; b < N / 2; ++b) {
-            const int half = 1 << s;
-            const int j = b & (half - 1), i0 = ((b >> s) << (s + 1)) + j, i1 = i0 + half;
-            const int e = level_exp<A, INV>(s, j);
-            u64 u = y[i0], v = y[i1];
-            if (e == 0) {
-                y[i0] = gl::addc(u, v);
-                y[i1] = gl::sub(u, v);
-            } else if (e < 96) {
-                v = gl::mul_pow2(v, (u32)e);
+    static_for<0, A>([&](auto s_) {
+        constexpr int s = decltype(s_)::value;
+        static_for<0, N / 2>([&](auto b_) {
+            constexpr int b = decltype(b_)::value;
+            constexpr int half = 1 << s;
+            constexpr int j = b & (half - 1), i0 = ((b >> s) << (s + 1)) + j, i1 = i0 + half;
+            constexpr int e = level_exp<A, INV>(s, j);
+            const u64 u = y[i0];
+            if constexpr (e < 96) {
+                const u64 v = gl::mul_pow2c<e>(y[i1]);
                 y[i0] = gl::addc(u, v);
                 y[i1] = gl::sub(u, v);
             } else {                                   // 2^e = -2^(e-96)
-                v = gl::mul_pow2(v, (u32)(e - 96));
+                const u64 v = gl::mul_pow2c<e - 96>(y[i1]);
                 y[i0] = gl::sub(u, v);
                 y[i1] = gl::addc(u, v);
             }
-        }
-    }
+        });
+    });
 #pragma unroll
     for (int i = 0; i < N; ++i) x[i] = y[i];
 }
