@@ -160,6 +160,18 @@ int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, 
                      const int *factor_idx, const uint64_t *coeffs, int n_terms,
                      uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream);
 
+/* vi_sumcheck_eval without a workspace argument and without any allocation: for callers that cannot call
+ * hipMalloc (code under HIP graph capture, tight serving loops, harnesses that forbid it).  It has no
+ * counterpart in the reference.  The per-workgroup partial sums live in a file-scope device array of the
+ * library, vi_sumcheck_workspace_bytes() = 128 KiB per GPU, held until the process ends; its device address is
+ * looked up once per device on the first call there.  half above VI_SC_STATIC_MAX_HALF is rejected (VI_EINVAL).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race;
+ * calls queued on one stream do not.  Same results as vi_sumcheck_eval. */
+#define VI_SC_STATIC_MAX_HALF ((int64_t)1 << 32)
+int vi_sumcheck_eval_static(const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
+                            const int *factor_idx, const uint64_t *coeffs, int n_terms, uint64_t *out_samples,
+                            void *stream);
+
 /* fold every table by r (sumcheck.py:51-54 / gpu.py:341-347): dst[t][i] = src[t][i] +
  * r (src[t][half+i] - src[t][i]), i < half; and, when half >= 2, also return the
  * NEXT round's samples computed from the folded tables in the same pass.

@@ -26,7 +26,8 @@ EXPORTS = [
     "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend",
     "vi_kquant_to_field",
     "vi_kquant_to_field_transposed",
-    "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_fold_eval", "vi_sumcheck_prove",
+    "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_eval_static", "vi_sumcheck_fold_eval",
+    "vi_sumcheck_prove",
     "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
     "vi_merkle_level", "vi_merkle_tree_nodes", "vi_merkle_tree", "vi_row_prg",
     "vi_eq_vector", "vi_mle_eval_workspace_bytes", "vi_mle_eval",
@@ -85,6 +86,7 @@ def lib():
     L.vi_sumcheck_workspace_bytes.restype = sz
     L.vi_sumcheck_workspace_bytes.argtypes = []
     L.vi_sumcheck_eval.argtypes = [POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int, vp, vp, sz, vp]
+    L.vi_sumcheck_eval_static.argtypes = [POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int, vp, vp]
     L.vi_sumcheck_fold_eval.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, u64, ip, ip,
                                         POINTER(u64), c_int, POINTER(u64), vp, vp, sz, vp]
     L.vi_sumcheck_prove.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int,
@@ -111,7 +113,7 @@ def lib():
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
-                 "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_kquant_to_field_transposed", "vi_sumcheck_eval",
+                 "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_kquant_to_field_transposed", "vi_sumcheck_eval", "vi_sumcheck_eval_static",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
                  "vi_merkle_level", "vi_merkle_tree_nodes", "vi_merkle_tree", "vi_row_prg", "vi_eq_vector", "vi_mle_eval",
                  "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities"):

@@ -18,6 +18,8 @@
 //
 // Variable order is most-significant first, pairs are (i, half + i)
 // (layergkr/sumcheck.py:51-54).
+#include <mutex>
+
 #include "common.hpp"
 #include "gl_field.hpp"
 
@@ -486,29 +488,80 @@ extern "C" {
 
 size_t vi_sumcheck_workspace_bytes(void) { return (size_t)MAX_BLOCKS * NSAMP * sizeof(u64); }
 
-int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
-                     const int *factor_idx, const uint64_t *coeffs, int n_terms,
-                     uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream) {
+namespace {
+
+int sumcheck_eval_on(const char *who, const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
+                     const int *factor_idx, const uint64_t *coeffs, int n_terms, uint64_t *out_samples, u64 *partial,
+                     void *stream) {
     Desc D;
-    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, "vi_sumcheck_eval");
+    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, who);
     if (rc) return rc;
-    if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_eval: half = %lld", (long long)half);
-    if (!out_samples) return vi::fail(VI_EINVAL, "vi_sumcheck_eval: null out_samples");
-    if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
+    if (half < 1) return vi::fail(VI_EINVAL, "%s: half = %lld", who, (long long)half);
+    if (!out_samples) return vi::fail(VI_EINVAL, "%s: null out_samples", who);
     hipStream_t s = (hipStream_t)stream;
     int nb = blocks_for(half);
     const u64 scale = D.out_scale;
     if (n_tables <= REG_TABLES && half <= DIRECT_MAX) {
-        launch_round<0>(D, half, 0, (u64 *)ws, 1, out_samples, scale, 1, s);
+        launch_round<0>(D, half, 0, partial, 1, out_samples, scale, 1, s);
         VI_LAUNCH_CHECK("sumcheck eval");
         return VI_OK;
     }
-    if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, (u64 *)ws, nb, nullptr, 1, 0, s);
-    else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, (u64 *)ws);
+    if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, partial, nb, nullptr, 1, 0, s);
+    else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, partial);
     VI_LAUNCH_CHECK("sumcheck eval");
-    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, 0, (u64)0, out_samples);
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, D.deg, scale, 0, (u64)0, out_samples);
     VI_LAUNCH_CHECK("sumcheck final");
     return VI_OK;
+}
+
+}  // namespace
+
+int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
+                     const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                     uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream) {
+    if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
+    return sumcheck_eval_on("vi_sumcheck_eval", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, out_samples,
+                            (u64 *)ws, stream);
+}
+
+// The per-workgroup partial sums of vi_sumcheck_eval_static: MAX_BLOCKS x NSAMP words (128 KiB) per GPU for the
+// life of the process.  In host code this name is only a handle for hipGetSymbolAddress; kernels get the address.
+static __device__ __align__(256) u64 scratch[MAX_BLOCKS * NSAMP];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+u64 *g_scratch_ptr[MAX_DEVICES] = {nullptr};
+
+// device address of `scratch` on the current device, looked up once per device
+int scratch_on_current_device(u64 **out) {
+    int dev = 0;
+    VI_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return vi::fail(VI_EINVAL, "vi_sumcheck_eval_static: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        VI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = (u64 *)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return VI_OK;
+}
+}  // namespace
+
+int vi_sumcheck_eval_static(const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
+                            const int *factor_idx, const uint64_t *coeffs, int n_terms, uint64_t *out_samples,
+                            void *stream) {
+    if (half > VI_SC_STATIC_MAX_HALF)
+        return vi::fail(VI_EINVAL, "vi_sumcheck_eval_static: half = %lld exceeds the limit of %lld pairs; use vi_sumcheck_eval",
+                        (long long)half, (long long)VI_SC_STATIC_MAX_HALF);
+    u64 *partial = nullptr;
+    int rc = scratch_on_current_device(&partial);
+    if (rc) return rc;
+    // every workgroup of the launch overwrites its own NSAMP words and the final kernel reads exactly those, so
+    // nothing of an earlier call has to be cleared
+    return sumcheck_eval_on("vi_sumcheck_eval_static", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms,
+                            out_samples, partial, stream);
 }
 
 int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
