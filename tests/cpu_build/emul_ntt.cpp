@@ -34,8 +34,8 @@ Owned *make_owned(int logn, int inv) {
 
 int g_use_fast = 1;
 
-template <int A2, bool INV>
-void run_fast(const PassArgs &A) {
+template <int A2, bool INV, bool UNI>
+void run_fast_u(const PassArgs &A) {
     i64 tiles = pass_tiles(A);
     std::vector<u64> lds(fast_lds_words(A.a));
     std::vector<u64> regs((size_t)NTHREADS * 16);
@@ -43,18 +43,29 @@ void run_fast(const PassArgs &A) {
     int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
     for (i64 tile = 0; tile < tiles; ++tile) {
         for (int tid = 0; tid < NTHREADS; ++tid)
-            fast_load<A2>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
+            fast_load<A2, UNI>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
         for (int t = 0; t < n_loop; ++t) {
             for (int tid = 0; tid < NTHREADS; ++tid)
             {
                 u64 pw[16] = {};
-                if (A.pre) fast_pre_load<A2>(A, tile, tid, t, pw);
+                if (A.pre) fast_pre_load<A2, UNI>(A, tile, tid, t, pw);
                 fast_stage1<A2, INV>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
                                      pw, A.twi, lds.data());
             }
-            for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV>(A, tile, tid, t, lds.data());
+            for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds.data());
         }
     }
+}
+
+int g_allow_uniform = 1;
+
+// the same choice the HIP launcher makes: scalar-base addressing when the pass qualifies
+template <int A2, bool INV>
+void run_fast(const PassArgs &A_in) {
+    PassArgs A = A_in;
+    A.uniform = (g_allow_uniform && pass_uniform(A, &A.n1_valid)) ? 1 : 0;
+    if (A.uniform) run_fast_u<A2, INV, true>(A);
+    else run_fast_u<A2, INV, false>(A);
 }
 
 void run_pass(const PassArgs &A) {
@@ -92,6 +103,7 @@ void run_pass(const PassArgs &A) {
 extern "C" {
 
 void emu_set_fast(int on) { g_use_fast = on; }
+void emu_set_uniform(int on) { g_allow_uniform = on; }
 u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
 u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
 u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }

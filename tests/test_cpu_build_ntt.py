@@ -31,6 +31,7 @@ def emu():
     L.emu_inv.argtypes = [c_uint64]
     L.emu_mul_pow2.argtypes = [c_uint64, c_uint]
     L.emu_set_fast.argtypes = [c_int]
+    L.emu_set_uniform.argtypes = [c_int]
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
     L.emu_coset_lde_ex.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p, c_long, u64p, c_int]
@@ -79,14 +80,17 @@ def test_device_inverse_chain(emu):
 def test_ntt_passes_match_oracle(emu, logn, m):
     a = _rand((m, 1 << logn), 100 + logn)
     want = O.ntt_rows(a)
-    for fast in (1, 0):                      # register-blocked passes, then the generic radix-2 passes
+    # register-blocked passes with scalar-base and with per-element addressing, then the generic radix-2 passes
+    for fast, uni in ((1, 1), (1, 0), (0, 0)):
         emu.emu_set_fast(fast)
+        emu.emu_set_uniform(uni)
         got = a.copy()
         emu.emu_ntt_batched(_p(got), m, logn, 0)
-        assert np.array_equal(got, want), fast
+        assert np.array_equal(got, want), (fast, uni)
         emu.emu_ntt_batched(_p(got), m, logn, 1)
-        assert np.array_equal(got, a), fast
+        assert np.array_equal(got, a), (fast, uni)
     emu.emu_set_fast(1)
+    emu.emu_set_uniform(1)
 
 
 def test_ntt_25_bit_split_is_well_formed(emu):
@@ -105,12 +109,14 @@ def test_ntt_25_bit_split_is_well_formed(emu):
 def test_lde_passes_match_oracle(emu, logK, logN, m, w):
     msgs = _rand((m, w), 200 + logK)
     want = O.coset_lde_rows(msgs, 1 << logK, 1 << logN, 7)
-    for fast in (1, 0):
+    for fast, uni in ((1, 1), (1, 0), (0, 0)):
         emu.emu_set_fast(fast)
+        emu.emu_set_uniform(uni)
         got = np.zeros((m, 1 << logN), dtype=np.uint64)
         emu.emu_coset_lde(_p(msgs), m, w, w, logK, logN, 7, _p(got))
-        assert np.array_equal(got, want), fast
+        assert np.array_equal(got, want), (fast, uni)
     emu.emu_set_fast(1)
+    emu.emu_set_uniform(1)
 
 
 def test_lde_strided_input_and_other_shift(emu):
@@ -132,8 +138,9 @@ def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w
     padded = np.zeros((m, K), dtype=np.uint64)
     padded[:, :w] = msgs
     want_c = O.ntt_rows(padded, inverse=True)
-    for fast in (1, 0):
+    for fast, uni in ((1, 1), (1, 0), (0, 0)):
         emu.emu_set_fast(fast)
+        emu.emu_set_uniform(uni)
         pitch = K + 3
         co = np.zeros((m, pitch), dtype=np.uint64)
         got = np.zeros((m, N), dtype=np.uint64)
@@ -159,3 +166,4 @@ def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w
         emu.emu_coset_lde_ex(_p(full), m, K, K, logK, logN, 7, None, 0, _p(got4), 1)
         assert np.array_equal(got3, got4)
     emu.emu_set_fast(1)
+    emu.emu_set_uniform(1)

@@ -120,10 +120,11 @@ __device__ __forceinline__ u64 canon(u64 x) {
     return pack(r0, r1);
 }
 
-// (hi:lo) given as four words l0 l1 hl hh -> [0, p):  lo - hh + hl (2^32 - 1)
-__device__ __forceinline__ u64 reduce_words(u32 l0, u32 l1, u32 hl, u32 hh) {
+// (hi:lo) given as four words l0 l1 hl hh, minus the borrow-in `bin` -> [0, p):  lo - hh - bin + hl (2^32 - 1).
+// hh + bin must be below 2^32.
+__device__ __forceinline__ u64 reduce_words(u32 l0, u32 l1, u32 hl, u32 hh, u64 bin) {
     u32 x0, x1, m;
-    asm("v_sub_co_u32 %[x0], vcc, %[l0], %[hh]\n\t"
+    asm("v_subb_co_u32 %[x0], vcc, %[l0], %[hh], %[bin]\n\t"
         "s_nop 1\n\t"
         "v_subbrev_co_u32 %[x1], vcc, 0, %[l1], vcc\n\t"
         "s_nop 1\n\t"
@@ -132,7 +133,7 @@ __device__ __forceinline__ u64 reduce_words(u32 l0, u32 l1, u32 hl, u32 hh) {
         "s_nop 1\n\t"
         "v_subbrev_co_u32 %[x1], vcc, 0, %[x1], vcc"
         : [x0] "=&v"(x0), [x1] "=&v"(x1), [m] "=&v"(m)
-        : [l0] "v"(l0), [l1] "v"(l1), [hh] "v"(hh)
+        : [l0] "v"(l0), [l1] "v"(l1), [hh] "v"(hh), [bin] "s"(bin)
         : "vcc");
     u64 w, st;
     asm("v_mad_u64_u32 %[w], %[st], %[hl], -1, %[x]"
@@ -151,18 +152,18 @@ __device__ __forceinline__ u64 mul(u64 a, u64 b) {
         : [p00] "=&v"(p00), [mm] "=&v"(mm), [p11] "=&v"(p11), [st] "=&s"(st)
         : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1)
         : "vcc");
-    // words of the 128-bit product: p00.lo, p00.hi + mm.lo, p11.lo + mm.hi + carry, p11.hi + carry + (carry of the cross sum)
+    // words of the 128-bit product: p00.lo, p00.hi + mm.lo, p11.lo + mm.hi + carry, p11.hi + carry.  The carry of the
+    // cross sum (in st) weighs 2^96 = -1: it goes into the reduction as a borrow.
     u32 w1 = (u32)(p00 >> 32), hl, hh;
     asm("v_add_co_u32 %[w1], vcc, %[w1], %[m0]\n\t"
         "s_nop 1\n\t"
         "v_addc_co_u32 %[hl], vcc, %[q0], %[m1], vcc\n\t"
         "s_nop 1\n\t"
-        "v_addc_co_u32 %[hh], vcc, 0, %[q1], vcc\n\t"
-        "v_addc_co_u32 %[hh], vcc, 0, %[hh], %[st]"
+        "v_addc_co_u32 %[hh], vcc, 0, %[q1], vcc"
         : [w1] "+v"(w1), [hl] "=&v"(hl), [hh] "=&v"(hh)
-        : [m0] "v"((u32)mm), [m1] "v"((u32)(mm >> 32)), [q0] "v"((u32)p11), [q1] "v"((u32)(p11 >> 32)), [st] "s"(st)
+        : [m0] "v"((u32)mm), [m1] "v"((u32)(mm >> 32)), [q0] "v"((u32)p11), [q1] "v"((u32)(p11 >> 32))
         : "vcc");
-    return reduce_words((u32)p00, w1, hl, hh);
+    return reduce_words((u32)p00, w1, hl, hh, st);
 }
 
 // canonical v times 2^E, 0 <= E < 96, canonical result; s = 32 q + r moves v into limbs m0 m1 m2 at phi^q
@@ -248,7 +249,7 @@ VI_HD u64 canon(u64 x) {
 // (hi:lo) -> [0, p).  hi = hh*2^32 + hl  =>  value = lo - hh + hl*(2^32 - 1).
 VI_HD u64 reduce128(u64 lo, u64 hi) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    return dev::reduce_words((u32)lo, (u32)(lo >> 32), (u32)hi, (u32)(hi >> 32));
+    return dev::reduce_words((u32)lo, (u32)(lo >> 32), (u32)hi, (u32)(hi >> 32), 0);
 #endif
     u32 hh = (u32)(hi >> 32), hl = (u32)hi;
     u64 t0 = lo - hh;

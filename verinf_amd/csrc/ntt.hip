@@ -45,7 +45,8 @@ __global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
 // FIN: compiled for the final (transposing) pass only, without the strided passes' addressing (110 instead of
 // 120 registers).  The strided passes keep the run-time flag: compiled with it fixed to 0 they took 128
 // registers and spilled.
-template <int A2, bool INV, bool FIN>
+// UNI: compiled for passes whose tiles are all addressed by scalar bases plus 32-bit thread offsets (pass_uniform).
+template <int A2, bool INV, bool FIN, bool UNI>
 __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     PassArgs A = A_in;
     if (FIN) A.is_final = 1;
@@ -84,8 +85,8 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     }
     u64 reg[16], pw[16];
     u32 ok;
-    if (A.pre) fast_pre_load<A2>(A, tile, tid, t, pw);
-    fast_load<A2>(A, tile, tid, reg, ok);
+    if (A.pre) fast_pre_load<A2, UNI>(A, tile, tid, t, pw);
+    fast_load<A2, UNI>(A, tile, tid, reg, ok);
     if (!A.is_final) {
         if (lane < count) twi[first + lane] = tw_wave;
         __builtin_amdgcn_wave_barrier();
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     }
     fast_stage1<A2, INV>(A, tile, tid, t, ok, reg, pw, twi, lds);
     __syncthreads();
-    fast_stage2<A2, INV>(A, tile, tid, t, lds);
+    fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds);
 }
 
 namespace {
@@ -191,14 +192,22 @@ int get_pre(int logK, int logN, u64 shift, const u64 **out) {
     return VI_OK;
 }
 
-template <int A2>
-void launch_fast_a(const PassArgs &A, dim3 grid, dim3 block, hipStream_t s) {
+template <int A2, bool UNI>
+void launch_fast_u(const PassArgs &A, dim3 grid, dim3 block, hipStream_t s) {
     switch ((A.inverse ? 2 : 0) + (A.is_final ? 1 : 0)) {
-        case 0: hipLaunchKernelGGL((k_ntt_fast<A2, false, false>), grid, block, 0, s, A); break;
-        case 1: hipLaunchKernelGGL((k_ntt_fast<A2, false, true>), grid, block, 0, s, A); break;
-        case 2: hipLaunchKernelGGL((k_ntt_fast<A2, true, false>), grid, block, 0, s, A); break;
-        default: hipLaunchKernelGGL((k_ntt_fast<A2, true, true>), grid, block, 0, s, A); break;
+        case 0: hipLaunchKernelGGL((k_ntt_fast<A2, false, false, UNI>), grid, block, 0, s, A); break;
+        case 1: hipLaunchKernelGGL((k_ntt_fast<A2, false, true, UNI>), grid, block, 0, s, A); break;
+        case 2: hipLaunchKernelGGL((k_ntt_fast<A2, true, false, UNI>), grid, block, 0, s, A); break;
+        default: hipLaunchKernelGGL((k_ntt_fast<A2, true, true, UNI>), grid, block, 0, s, A); break;
     }
+}
+
+template <int A2>
+void launch_fast_a(const PassArgs &A_in, dim3 grid, dim3 block, hipStream_t s) {
+    PassArgs A = A_in;
+    A.uniform = pass_uniform(A, &A.n1_valid) ? 1 : 0;
+    if (A.uniform) launch_fast_u<A2, true>(A, grid, block, s);
+    else launch_fast_u<A2, false>(A, grid, block, s);
 }
 
 void launch_fast(const PassArgs &A, dim3 grid, dim3 block, hipStream_t s) {

@@ -118,6 +118,93 @@ VI_HD ColRef col_ref(const PassArgs &A, i64 tile, int c) {
     return R;
 }
 
+// A pass whose every tile the workgroup can address with one set of bases and 32-bit per-thread offsets ("uniform
+// pass"): the columns of a tile lie in one batch row, every row of the launch exists (a row is a whole number of
+// tiles), which of a thread's sixteen inputs exist depends only on their position n1, and the offsets that differ
+// between threads stay below 2^29 elements.  The bases are then the same for all threads of the workgroup and live
+// in scalar registers; a load or store is "scalar base + thread offset" with no 64-bit vector arithmetic and no
+// per-element test.  Passes that do not qualify (short transforms whose rows are narrower than a tile, source rows
+// of a ragged width) take the per-element path; the host decides per launch (pass_uniform) and the kernel is
+// compiled for one or the other.
+struct TileU {
+    i64 src_u;        // element offset into src of (first column, point 0), without the per-thread part
+    i64 dst_u;        // the same into dst (without the coset plane of a strided pass)
+    i64 pre_u;        // index inside the source row of (first column, point 0)
+    i64 tw_u;         // strided pass: r of the first column
+    int sh1;          // log2 of the element stride between a thread's stage-1 inputs n1, n1 + 1
+    int sh2;          // log2 of the element stride between a thread's stage-2 outputs k2, k2 + 1
+    int shk;          // log2 of the element stride between outputs k1, k1 + 1
+    int shc;          // final pass: log2 of the source stride between column groups (c >> log_rho)
+};
+
+// does the pass qualify?  On success *n1_valid = how many of a thread's sixteen stage-1 inputs exist (the first
+// n1_valid; 16 unless the source rows are narrower than the transform).
+inline bool pass_uniform(const PassArgs &A, int *n1_valid) {
+    const int lt = logT(A), a2 = A.a - 4;
+    *n1_valid = 16;
+    if (A.logn > 26 || A.n_rows < 1) return false;
+    const i64 n = (i64)1 << A.logn;
+    if (!A.is_final) {
+        const int lc = A.B + A.logR;
+        if (lc < lt || A.logR < lt) return false;
+        if (A.src_width == n) return true;
+        // a narrower source: only on the first pass (B = 0, so the index of input n1 is below (n1 + 1) << sh1)
+        const int sh1 = a2 + A.logR;
+        if (A.B != 0 || A.src_width < 1 || (A.src_width & (((i64)1 << sh1) - 1)) != 0) return false;
+        *n1_valid = (int)(A.src_width >> sh1);
+        return true;
+    }
+    const int lc = A.B + A.log_rho;
+    if (A.pre || A.ndig < 1 || lc < lt || lt < A.log_rho || lt - A.log_rho > A.dig[0]) return false;
+    if (A.src_width != n) return false;
+    return (((i64)1 << A.log_rho) - 1) * A.src_coset_stride + n < ((i64)1 << 29);
+}
+
+template <int A2>
+VI_HD TileU tile_uniform(const PassArgs &A, i64 tile) {
+    TileU U;
+    U.src_u = U.dst_u = U.pre_u = U.tw_u = 0;
+    U.sh1 = U.sh2 = U.shk = U.shc = 0;
+    const int lt = logT(A);
+    if (!A.is_final) {
+        const int lc = A.B + A.logR;
+        const i64 row = tile >> (lc - lt);
+        const i64 col0 = (tile & (((i64)1 << (lc - lt)) - 1)) << lt;
+        const i64 prefix = col0 >> A.logR, r0 = col0 & (((i64)1 << A.logR) - 1);
+        const i64 idx_u = (prefix << (A.a + A.logR)) + r0;
+        U.src_u = row * A.src_row_stride + idx_u;
+        U.dst_u = row * A.dst_row_stride + idx_u;
+        U.pre_u = idx_u;
+        U.tw_u = r0;
+        U.sh1 = A2 + A.logR;
+        U.sh2 = 4 + A.logR;
+        U.shk = A.logR;
+    } else {
+        const int lc = A.B + A.log_rho;
+        const i64 row = tile >> (lc - lt);
+        const i64 v0 = (tile & (((i64)1 << (lc - lt)) - 1)) << lt;
+        U.src_u = row * A.src_row_stride + (storage_prefix(A, v0 >> A.log_rho) << A.a);
+        U.dst_u = row * A.dst_row_stride + v0;
+        U.sh1 = A2;
+        U.sh2 = 4 + lc;
+        U.shk = lc;
+        U.shc = A.B - A.dig[0] + A.a;
+    }
+    return U;
+}
+
+// element `off` (a per-thread 32-bit element offset) of the run that starts at the uniform address `base`
+VI_HD const u64 *at32(const u64 *base, u32 off) { return (const u64 *)((const char *)base + (size_t)(u32)(off * 8u)); }
+VI_HD u64 *at32(u64 *base, u32 off) { return (u64 *)((char *)base + (size_t)(u32)(off * 8u)); }
+
+// the per-thread part of the stage-1 source offset in a tile described by a TileU
+template <int A2>
+VI_HD u32 lane_src_off(const PassArgs &A, const TileU &U, int c, int n2) {
+    if (!A.is_final) return (u32)c + ((u32)n2 << A.logR);
+    const u32 t = (u32)c & ((1u << A.log_rho) - 1), cu = (u32)c >> A.log_rho;
+    return t * (u32)A.src_coset_stride + (cu << U.shc) + (u32)n2;
+}
+
 // stage-1 thread -> (column, n2)
 template <int A2>
 VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
@@ -135,10 +222,20 @@ VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
 // the batch, a point past the source width) reads word 0 of the source instead and is zeroed in fast_fix.  With
 // the load inside the test, and the reduction mod p right behind it, every second load waited for the one
 // before -- eight memory round trips per tile instead of one.
-template <int A2>
+template <int A2, bool UNI>
 VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &ok) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
+    if constexpr (UNI) {
+        const TileU U = tile_uniform<A2>(A, tile);
+        const u32 off = lane_src_off<A2>(A, U, c, n2);
+        // an input past the source width reads input 0 instead (and is zeroed in fast_fix): the choice is the same
+        // for every thread, so it is made on the scalar base
+#pragma unroll
+        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = *at32(A.src + U.src_u + ((i64)(n1 < A.n1_valid ? n1 : 0) << U.sh1), off);
+        ok = A.n1_valid >= 16 ? 0xFFFFu : ((1u << A.n1_valid) - 1u);
+        return;
+    }
     const ColRef R = col_ref(A, tile, c);
     const int sh = A.is_final ? 0 : A.logR;
     ok = 0;
@@ -169,10 +266,18 @@ VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
 // twi: w_L^(n2 k1) at [n2 * 16 + k1]
 // the coset pre-multipliers of this thread's sixteen inputs (a column that does not exist takes those of
 // point 0 of coset 0; its data are zero); requested before the tile so that they are there when it arrives
-template <int A2>
+template <int A2, bool UNI>
 VI_HD void fast_pre_load(const PassArgs &A, i64 tile, int tid, int t_loop, u64 (&pw)[16]) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
+    if constexpr (UNI) {                                   // a strided pass: a final pass with pre-multipliers is never uniform
+        const TileU U = tile_uniform<A2>(A, tile);
+        const u32 off = lane_src_off<A2>(A, U, c, n2);
+        const u64 *pre = A.pre + ((i64)t_loop << A.logn) + U.pre_u;
+#pragma unroll
+        for (int n1 = 0; n1 < 16; ++n1) pw[n1] = *at32(pre + ((i64)n1 << U.sh1), off);
+        return;
+    }
     const ColRef R = col_ref(A, tile, c);
     const int sh = A.is_final ? 0 : A.logR;
     const int t = A.is_final ? R.t : t_loop;
@@ -215,12 +320,40 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok,
 }
 
 // phase 3: 16/E2 stage-2 transforms, inter-pass twiddle (or final scale), scatter
-template <int A2, bool INV>
+template <int A2, bool INV, bool UNI>
 VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u64 *lds) {
     constexpr int E2 = 1 << A2;
     const int lt = logT(A);
     const int st = (1 << lt) + 1;
     const int c = tid & ((1 << lt) - 1);
+    if constexpr (UNI) {
+        const TileU U = tile_uniform<A2>(A, tile);
+        u64 *dst = A.dst + U.dst_u + (A.is_final ? 0 : (i64)t_loop * A.dst_coset_stride);
+#pragma unroll
+        for (int i = 0; i < 16 / E2; ++i) {
+            const int k1 = (tid + i * NTHREADS) >> lt;
+            const u32 off = (u32)c + ((u32)k1 << U.shk);
+            u64 x[E2], tw[E2];
+            if (!A.is_final) {
+#pragma unroll
+                for (int k2 = 0; k2 < E2; ++k2) tw[k2] = *at32(A.tw + U.tw_u + ((i64)k2 << U.sh2), off);
+            }
+#pragma unroll
+            for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
+            VI_SCHED_FENCE();
+            dft_reg<A2, INV>(x);
+            VI_SCHED_FENCE();
+#pragma unroll
+            for (int k2 = 0; k2 < E2; ++k2) {
+                u64 v = x[k2];
+                if (!A.is_final) v = gl::mul(v, tw[k2]);
+                else if (A.scale != 1) v = gl::mul(v, A.scale);
+                VI_STREAM_STORE(at32(dst + ((i64)k2 << U.sh2), off), v);
+                if ((k2 & 3) == 3) VI_SCHED_FENCE();
+            }
+        }
+        return;
+    }
     const ColRef R = col_ref(A, tile, c);
     const int lc = A.B + A.log_rho;
 #pragma unroll

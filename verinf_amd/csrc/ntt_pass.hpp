@@ -57,6 +57,8 @@ struct PassArgs {
     u64 scale;                                // final pass: scalar multiplier (1 = none)
     int inverse;                              // direction of the transform
     int canon_src;                            // src is caller data: reduce every word mod p on load
+    int uniform;                              // register-blocked kernel: every tile is addressed by scalar bases (ntt_fast.hpp)
+    int n1_valid;                             // uniform pass: how many of a thread's sixteen stage-1 inputs exist
 };
 
 VI_HD int logT(const PassArgs &A) { return TILE_LOG - A.a; }
