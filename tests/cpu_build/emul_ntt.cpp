@@ -68,6 +68,35 @@ void run_fast(const PassArgs &A_in) {
     else run_fast_u<A2, INV, false>(A);
 }
 
+// the fused launch of the last inverse and the first forward pass, phase by phase like the kernel
+template <int A2>
+void run_fused(const PassArgs &Ai_in, const PassArgs &Af_in) {
+    PassArgs Ai = Ai_in, Af = Af_in;
+    Ai.uniform = Af.uniform = 1;
+    Ai.n1_valid = Af.n1_valid = 16;
+    const i64 tiles = pass_tiles(Ai);
+    std::vector<u64> lds(fast_lds_words(Ai.a));
+    std::vector<u64> regs((size_t)NTHREADS * 16), coef((size_t)NTHREADS * 16);
+    std::vector<u32> oks(NTHREADS);
+    auto R = [&](std::vector<u64> &v, int tid) -> u64(&)[16] { return *reinterpret_cast<u64(*)[16]>(&v[(size_t)tid * 16]); };
+    for (i64 tile = 0; tile < tiles; ++tile) {
+        u64 pw[16] = {};
+        for (int tid = 0; tid < NTHREADS; ++tid) fast_load<A2, true>(Ai, tile, tid, R(regs, tid), oks[tid]);
+        for (int tid = 0; tid < NTHREADS; ++tid)
+            fast_stage1<A2, true>(Ai, tile, tid, 0, oks[tid], R(regs, tid), pw, Ai.twi, lds.data());
+        for (int tid = 0; tid < NTHREADS; ++tid) fused_stage2_inv<A2>(Ai, tile, tid, lds.data(), R(coef, tid));
+        for (int t = 0; t < (1 << Af.log_rho); ++t) {
+            for (int tid = 0; tid < NTHREADS; ++tid) fused_stage1_fwd<A2>(Af, tile, tid, t, R(coef, tid), Af.twi, lds.data());
+            for (int tid = 0; tid < NTHREADS; ++tid) fused_stage2_fwd<A2>(Af, tile, tid, t, lds.data());
+        }
+    }
+}
+
+int g_allow_fusion = 1;
+
+// runs passes[q] (and passes[q + 1] with it when the two fuse); returns how many passes it consumed
+int run_passes_at(const std::vector<PassArgs> &passes, size_t q);
+
 void run_pass(const PassArgs &A) {
     if (g_use_fast && fast_ok(A.a)) {
         switch ((A.a - FAST_A1) * 2 + (A.inverse ? 1 : 0)) {
@@ -98,12 +127,33 @@ void run_pass(const PassArgs &A) {
     }
 }
 
+int run_passes_at(const std::vector<PassArgs> &passes, size_t q) {
+    const PassArgs &A = passes[q];
+    if (g_use_fast && g_allow_uniform && g_allow_fusion && A.fuse_next && q + 1 < passes.size() &&
+        passes_fusable(A, passes[q + 1])) {
+        switch (A.a - FAST_A1) {
+            case 1: run_fused<1>(A, passes[q + 1]); break;
+            case 2: run_fused<2>(A, passes[q + 1]); break;
+            case 3: run_fused<3>(A, passes[q + 1]); break;
+            default: run_fused<4>(A, passes[q + 1]); break;
+        }
+        return 2;
+    }
+    run_pass(A);
+    return 1;
+}
+
+void run_all(const std::vector<PassArgs> &passes) {
+    for (size_t q = 0; q < passes.size();) q += run_passes_at(passes, q);
+}
+
 }  // namespace
 
 extern "C" {
 
 void emu_set_fast(int on) { g_use_fast = on; }
 void emu_set_uniform(int on) { g_allow_uniform = on; }
+void emu_set_fusion(int on) { g_allow_fusion = on; }
 u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
 u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
 u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }
@@ -115,7 +165,7 @@ int emu_ntt_batched(u64 *buf, long m, int logn, int inverse) {
     std::vector<u64> ws(o->T.sp.p > 1 ? (size_t)m << logn : 1);
     std::vector<PassArgs> passes;
     build_ntt_passes(o->T, buf, ws.data(), m, passes);
-    for (auto &A : passes) run_pass(A);
+    run_all(passes);
     delete o;
     return (int)passes.size();
 }
@@ -127,8 +177,8 @@ int emu_coset_lde(const u64 *in, long m, long w, long in_stride, int logK, int l
     std::vector<u64> ws((size_t)lde_ws_elems(logK, logN, m));
     std::vector<PassArgs> passes;
     build_lde_passes(oi->T, of->T, pre.data(), logN, in, w, in_stride, out, (i64)1 << logN, ws.data(), m,
-                     passes);
-    for (auto &A : passes) run_pass(A);
+                     passes, nullptr, 0, false, g_use_fast && g_allow_uniform && g_allow_fusion);
+    run_all(passes);
     delete oi;
     delete of;
     return (int)passes.size();
@@ -141,8 +191,8 @@ int emu_coset_lde_ex(const u64 *in, long m, long w, long in_stride, int logK, in
     std::vector<u64> ws((size_t)lde_ws_elems(logK, logN, m));
     std::vector<PassArgs> passes;
     build_lde_passes(oi->T, of->T, pre.data(), logN, in, w, in_stride, out, (i64)1 << logN, ws.data(), m,
-                     passes, coeffs, coeffs_stride, in_is_coeffs != 0);
-    for (auto &A : passes) run_pass(A);
+                     passes, coeffs, coeffs_stride, in_is_coeffs != 0, g_use_fast && g_allow_uniform && g_allow_fusion);
+    run_all(passes);
     delete oi;
     delete of;
     return (int)passes.size();

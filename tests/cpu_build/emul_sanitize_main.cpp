@@ -63,8 +63,10 @@ int main() {
         {14, 16, 2, 8192, 16384}, {14, 16, 1, 16384, 16384}, {16, 18, 1, 65536, 65536}, {16, 17, 1, 40000, 40000},
         {16, 16, 1, 65536, 65536}, {8, 10, 0, 256, 256},
     };
-    for (int uni = 0; uni < 2; ++uni) {                    // per-element addressing, then scalar-base addressing where it applies
-        emu_set_uniform(uni);
+    // per-element addressing, scalar-base addressing where it applies, and the fused middle launch of the LDE
+    for (int mode = 0; mode < 3; ++mode) {
+        emu_set_uniform(mode >= 1);
+        emu_set_fusion(mode >= 2);
         for (auto &s : lde) bad += check_lde((int)s[0], (int)s[1], s[2], s[3], s[4]);
         bad += check_ntt(12, 3);
         bad += check_ntt(18, 1);

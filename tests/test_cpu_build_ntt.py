@@ -32,10 +32,15 @@ def emu():
     L.emu_mul_pow2.argtypes = [c_uint64, c_uint]
     L.emu_set_fast.argtypes = [c_int]
     L.emu_set_uniform.argtypes = [c_int]
+    L.emu_set_fusion.argtypes = [c_int]
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
     L.emu_coset_lde_ex.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p, c_long, u64p, c_int]
     return L
+
+
+# (register-blocked passes, scalar-base addressing, fused middle launch of the LDE): every way a pass can run
+MODES = ((1, 1, 1), (1, 1, 0), (1, 0, 0), (0, 0, 0))
 
 
 def _p(a):
@@ -81,16 +86,18 @@ def test_ntt_passes_match_oracle(emu, logn, m):
     a = _rand((m, 1 << logn), 100 + logn)
     want = O.ntt_rows(a)
     # register-blocked passes with scalar-base and with per-element addressing, then the generic radix-2 passes
-    for fast, uni in ((1, 1), (1, 0), (0, 0)):
+    for fast, uni, fuse in MODES:
         emu.emu_set_fast(fast)
         emu.emu_set_uniform(uni)
+        emu.emu_set_fusion(fuse)
         got = a.copy()
         emu.emu_ntt_batched(_p(got), m, logn, 0)
-        assert np.array_equal(got, want), (fast, uni)
+        assert np.array_equal(got, want), (fast, uni, fuse)
         emu.emu_ntt_batched(_p(got), m, logn, 1)
-        assert np.array_equal(got, a), (fast, uni)
+        assert np.array_equal(got, a), (fast, uni, fuse)
     emu.emu_set_fast(1)
     emu.emu_set_uniform(1)
+    emu.emu_set_fusion(1)
 
 
 def test_ntt_25_bit_split_is_well_formed(emu):
@@ -109,14 +116,16 @@ def test_ntt_25_bit_split_is_well_formed(emu):
 def test_lde_passes_match_oracle(emu, logK, logN, m, w):
     msgs = _rand((m, w), 200 + logK)
     want = O.coset_lde_rows(msgs, 1 << logK, 1 << logN, 7)
-    for fast, uni in ((1, 1), (1, 0), (0, 0)):
+    for fast, uni, fuse in MODES:
         emu.emu_set_fast(fast)
         emu.emu_set_uniform(uni)
+        emu.emu_set_fusion(fuse)
         got = np.zeros((m, 1 << logN), dtype=np.uint64)
         emu.emu_coset_lde(_p(msgs), m, w, w, logK, logN, 7, _p(got))
-        assert np.array_equal(got, want), (fast, uni)
+        assert np.array_equal(got, want), (fast, uni, fuse)
     emu.emu_set_fast(1)
     emu.emu_set_uniform(1)
+    emu.emu_set_fusion(1)
 
 
 def test_lde_strided_input_and_other_shift(emu):
@@ -138,9 +147,10 @@ def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w
     padded = np.zeros((m, K), dtype=np.uint64)
     padded[:, :w] = msgs
     want_c = O.ntt_rows(padded, inverse=True)
-    for fast, uni in ((1, 1), (1, 0), (0, 0)):
+    for fast, uni, fuse in MODES:
         emu.emu_set_fast(fast)
         emu.emu_set_uniform(uni)
+        emu.emu_set_fusion(fuse)
         pitch = K + 3
         co = np.zeros((m, pitch), dtype=np.uint64)
         got = np.zeros((m, N), dtype=np.uint64)
@@ -167,3 +177,4 @@ def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w
         assert np.array_equal(got3, got4)
     emu.emu_set_fast(1)
     emu.emu_set_uniform(1)
+    emu.emu_set_fusion(1)

@@ -106,6 +106,32 @@ __device__ __forceinline__ u64 sub(u64 a, u64 b) {
     return pack(d0, d1);
 }
 
+// (u + v, u - v) of canonical u, v in one block: the two carry chains are interleaved so that each carry is read
+// three instructions after it was written and no wait has to be inserted
+__device__ __forceinline__ void bfly(u64 u, u64 v, u64 &sum, u64 &dif) {
+    u32 u0 = (u32)u, u1 = (u32)(u >> 32), v0 = (u32)v, v1 = (u32)(v >> 32);
+    u32 s0, s1, r0, r1, d0, d1, m;
+    u64 st, sb;
+    asm("v_add_co_u32 %[s0], vcc, %[u0], %[v0]\n\t"
+        "v_sub_co_u32 %[d0], %[sb], %[u0], %[v0]\n\t"
+        "v_add_co_u32 %[r0], %[st], -1, %[s0]\n\t"
+        "v_addc_co_u32 %[s1], vcc, %[u1], %[v1], vcc\n\t"
+        "v_subb_co_u32 %[d1], %[sb], %[u1], %[v1], %[sb]\n\t"
+        "v_addc_co_u32 %[r1], %[st], 0, %[s1], %[st]\n\t"
+        "s_or_b64 vcc, vcc, %[st]\n\t"
+        "v_subb_co_u32 %[m], %[sb], %[d0], %[d0], %[sb]\n\t"
+        "v_sub_co_u32 %[d0], %[sb], %[d0], %[m]\n\t"
+        "v_cndmask_b32 %[r0], %[s0], %[r0], vcc\n\t"
+        "v_cndmask_b32 %[r1], %[s1], %[r1], vcc\n\t"
+        "v_subbrev_co_u32 %[d1], %[sb], 0, %[d1], %[sb]"
+        : [s0] "=&v"(s0), [s1] "=&v"(s1), [r0] "=&v"(r0), [r1] "=&v"(r1), [d0] "=&v"(d0), [d1] "=&v"(d1), [m] "=&v"(m),
+          [st] "=&s"(st), [sb] "=&s"(sb)
+        : [u0] "v"(u0), [u1] "v"(u1), [v0] "v"(v0), [v1] "v"(v1)
+        : "vcc", "scc");
+    sum = pack(r0, r1);
+    dif = pack(d0, d1);
+}
+
 __device__ __forceinline__ u64 canon(u64 x) {
     u32 x0 = (u32)x, x1 = (u32)(x >> 32), r0, r1;
     asm("v_add_co_u32 %[r0], vcc, -1, %[x0]\n\t"
@@ -235,6 +261,16 @@ VI_HD u64 addc(u64 a, u64 b) {
     u64 s = a + b;
     u64 r = s + EPS;
     return ((s < a) | (r < s)) ? r : s;
+}
+
+// (u + v, u - v) for canonical u, v
+VI_HD void bfly(u64 u, u64 v, u64 &sum, u64 &dif) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    dev::bfly(u, v, sum, dif);
+#else
+    sum = addc(u, v);
+    dif = sub(u, v);
+#endif
 }
 
 // x mod p for an arbitrary 64-bit word

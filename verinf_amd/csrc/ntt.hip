@@ -101,6 +101,50 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds);
 }
 
+
+// The last inverse pass and the first forward pass of a coset extension in one launch (fused_stage2_inv): the
+// coefficients stay in registers between the two, so they are neither written to nor read back from HBM (unless the
+// caller wants them), and the rho cosets are expanded by a loop inside the workgroup.
+#ifndef VI_MID_MIN_WG
+#define VI_MID_MIN_WG 3
+#endif
+template <int A2>
+__global__ __launch_bounds__(NTHREADS, VI_MID_MIN_WG) void k_lde_mid(const PassArgs Ai_in, const PassArgs Af_in) {
+    PassArgs Ai = Ai_in, Af = Af_in;
+    Ai.is_final = 1;
+    Af.is_final = 0;
+    __shared__ u64 lds[TILE + (16 << A2)];
+    __shared__ u64 twi_i[16 << A2];
+    __shared__ u64 twi_f[16 << A2];
+    const int tid = threadIdx.x;
+    const i64 tile = blockIdx.x;
+    constexpr int PER = (16 << A2) / NTHREADS > 0 ? (16 << A2) / NTHREADS : 1;
+    u64 ti[PER], tf[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const bool in = tid + i * NTHREADS < (16 << A2);
+        ti[i] = in ? Ai.twi[tid + i * NTHREADS] : 0;
+        tf[i] = in ? Af.twi[tid + i * NTHREADS] : 0;
+    }
+    u64 reg[16], coef[16];
+    u32 ok;
+    fast_load<A2, true>(Ai, tile, tid, reg, ok);
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+        if (tid + i * NTHREADS < (16 << A2)) { twi_i[tid + i * NTHREADS] = ti[i]; twi_f[tid + i * NTHREADS] = tf[i]; }
+    __syncthreads();
+    fast_stage1<A2, true>(Ai, tile, tid, 0, ok, reg, reg, twi_i, lds);         // no pre-multipliers on the inverse side
+    __syncthreads();
+    fused_stage2_inv<A2>(Ai, tile, tid, lds, coef);
+    const int rho = 1 << Af.log_rho;
+    for (int t = 0; t < rho; ++t) {
+        __syncthreads();                                   // every thread is done reading the tile of the step before
+        fused_stage1_fwd<A2>(Af, tile, tid, t, coef, twi_f, lds);
+        __syncthreads();
+        fused_stage2_fwd<A2>(Af, tile, tid, t, lds);
+    }
+}
+
 namespace {
 
 struct DeviceTables {
@@ -219,10 +263,34 @@ void launch_fast(const PassArgs &A, dim3 grid, dim3 block, hipStream_t s) {
     }
 }
 
+int launch_fused(const PassArgs &Ai_in, const PassArgs &Af_in, hipStream_t s) {
+    PassArgs Ai = Ai_in, Af = Af_in;
+    Ai.uniform = Af.uniform = 1;
+    Ai.n1_valid = Af.n1_valid = 16;
+    const i64 tiles = pass_tiles(Ai);
+    if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
+    dim3 grid((unsigned)tiles), block(NTHREADS);
+    switch (Ai.a - FAST_A1) {
+        case 1: hipLaunchKernelGGL(k_lde_mid<1>, grid, block, 0, s, Ai, Af); break;
+        case 2: hipLaunchKernelGGL(k_lde_mid<2>, grid, block, 0, s, Ai, Af); break;
+        case 3: hipLaunchKernelGGL(k_lde_mid<3>, grid, block, 0, s, Ai, Af); break;
+        default: hipLaunchKernelGGL(k_lde_mid<4>, grid, block, 0, s, Ai, Af); break;
+    }
+    VI_LAUNCH_CHECK("k_lde_mid");
+    return VI_OK;
+}
+
 int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
-    for (const PassArgs &A : passes) {
+    for (size_t q = 0; q < passes.size(); ++q) {
+        const PassArgs &A = passes[q];
         i64 tiles = pass_tiles(A);
         if (tiles <= 0) continue;
+        if (A.fuse_next && q + 1 < passes.size() && passes_fusable(A, passes[q + 1])) {
+            int rc = launch_fused(A, passes[q + 1], s);
+            if (rc) return rc;
+            ++q;
+            continue;
+        }
         if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
         dim3 grid((unsigned)tiles), block(NTHREADS);
         if (fast_ok(A.a) && A.twi) {
@@ -302,7 +370,24 @@ int64_t vi_coset_lde_launches(int64_t m, int64_t K, int64_t N, size_t ws_bytes) 
     i64 chunk = (i64)(ws_bytes / one);
     if (chunk > m) chunk = m;
     if (chunk > max_rows_per_launch(vi::ilog2(N))) chunk = max_rows_per_launch(vi::ilog2(N));
-    return ((m + chunk - 1) / chunk) * 2 * split_digits(vi::ilog2(K)).p;   // balancing keeps the chunk count
+    const i64 n_chunks = (m + chunk - 1) / chunk;         // balancing keeps the chunk count
+    chunk = (m + n_chunks - 1) / n_chunks;
+    // the pass list of one chunk, planned with placeholder addresses (only their being null or not matters)
+    const int logK = vi::ilog2(K), logN = vi::ilog2(N);
+    Tables Ti{}, Tf{};
+    Ti.sp = Tf.sp = split_digits(logK);
+    Ti.logn = Tf.logn = logK;
+    Ti.inverse = 1;
+    Ti.scale = Tf.scale = 1;
+    u64 *dummy = (u64 *)(uintptr_t)4096;
+    std::vector<PassArgs> passes;
+    build_lde_passes(Ti, Tf, dummy, logN, dummy, K, K, dummy, N, dummy, chunk, passes);
+    i64 per_chunk = 0;
+    for (size_t q = 0; q < passes.size(); ++q) {
+        if (passes[q].fuse_next && q + 1 < passes.size() && passes_fusable(passes[q], passes[q + 1])) ++q;
+        ++per_chunk;
+    }
+    return n_chunks * per_chunk;
 }
 
 namespace {

@@ -63,12 +63,10 @@ VI_HD void dft_reg(u64 (&x)[1 << A]) {
             const u64 u = y[i0];
             if constexpr (e < 96) {
                 const u64 v = gl::mul_pow2c<e>(y[i1]);
-                y[i0] = gl::addc(u, v);
-                y[i1] = gl::sub(u, v);
+                gl::bfly(u, v, y[i0], y[i1]);
             } else {                                   // 2^e = -2^(e-96)
                 const u64 v = gl::mul_pow2c<e - 96>(y[i1]);
-                y[i0] = gl::sub(u, v);
-                y[i1] = gl::addc(u, v);
+                gl::bfly(u, v, y[i1], y[i0]);
             }
         });
     });
@@ -386,6 +384,128 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
             if ((k2 & 3) == 3) VI_SCHED_FENCE();
         }
     }
+}
+
+
+// The last inverse pass and the first forward pass of a coset extension share their tiles when K = L * L: the last
+// inverse pass leaves, in the thread that ran the stage-2 transforms (column c, outputs k1 = q + E2 i, i < 16 / E2),
+// the coefficients of points k = k1 + 16 k2 of that column, and the first forward pass wants thread (c, n2) to hold
+// points n1 E2 + n2 -- the same thread with n2 = q and n1 = i + (16 / E2) k2.  So a workgroup can go on to the rho
+// coset transforms without the coefficients leaving its registers (they are still written out when the caller
+// wants them: A.dst non-null).  Uniform passes only.
+template <int A2>
+VI_HD void fused_stage2_inv(const PassArgs &A, i64 tile, int tid, const u64 *lds, u64 (&coef)[16]) {
+    constexpr int E2 = 1 << A2;
+    const int lt = logT(A);
+    const int st = (1 << lt) + 1;
+    const int c = tid & ((1 << lt) - 1);
+    const TileU U = tile_uniform<A2>(A, tile);
+#pragma unroll
+    for (int i = 0; i < 16 / E2; ++i) {
+        const int k1 = (tid + i * NTHREADS) >> lt;
+        u64 x[E2];
+#pragma unroll
+        for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
+        VI_SCHED_FENCE();
+        dft_reg<A2, true>(x);
+        VI_SCHED_FENCE();
+#pragma unroll
+        for (int k2 = 0; k2 < E2; ++k2) {
+            u64 v = x[k2];
+            if (A.scale != 1) v = gl::mul(v, A.scale);
+            coef[i + (16 / E2) * k2] = v;
+        }
+    }
+    if (A.dst) {
+        u64 *dst = A.dst + U.dst_u;
+#pragma unroll
+        for (int i = 0; i < 16 / E2; ++i) {
+            const int k1 = (tid + i * NTHREADS) >> lt;
+            const u32 off = (u32)c + ((u32)k1 << U.shk);
+#pragma unroll
+            for (int k2 = 0; k2 < E2; ++k2) *at32(dst + ((i64)k2 << U.sh2), off) = coef[i + (16 / E2) * k2];
+        }
+    }
+}
+
+
+// Stage 1 and stage 2 of the first forward pass inside the fused launch.  The sixteen coefficients stay live in
+// registers over all cosets there, so the multipliers and twiddles are fetched four at a time, right before use,
+// instead of all sixteen ahead of the tile: other wavefronts cover the latency, and the kernel fits 128 registers.
+template <int A2>
+VI_HD void fused_stage1_fwd(const PassArgs &A, i64 tile, int tid, int t, const u64 (&coef)[16], const u64 *twi, u64 *lds) {
+    int c, n2;
+    s1_coords<A2>(A, tid, c, n2);
+    const TileU U = tile_uniform<A2>(A, tile);
+    const u32 off = lane_src_off<A2>(A, U, c, n2);
+    const u64 *pre = A.pre + ((i64)t << A.logn) + U.pre_u;
+    u64 x[16];
+#pragma unroll
+    for (int g = 0; g < 16; g += 4) {
+        u64 pw[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pw[j] = *at32(pre + ((i64)(g + j) << U.sh1), off);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[g + j] = gl::mul(coef[g + j], pw[j]);
+        VI_SCHED_FENCE();
+    }
+    dft_reg<4, false>(x);
+    VI_SCHED_FENCE();
+    const int st = (1 << logT(A)) + 1;
+#pragma unroll
+    for (int g = 0; g < 16; g += 4) {
+#pragma unroll
+        for (int k1 = g; k1 < g + 4; ++k1) {
+            u64 v = x[k1];
+            if (k1 > 0) v = gl::mul(v, twi[n2 * 16 + k1]);
+            lds[((k1 << A2) + n2) * st + c] = v;
+        }
+        VI_SCHED_FENCE();
+    }
+}
+
+template <int A2>
+VI_HD void fused_stage2_fwd(const PassArgs &A, i64 tile, int tid, int t, const u64 *lds) {
+    constexpr int E2 = 1 << A2;
+    constexpr int G = E2 < 4 ? E2 : 4;
+    const int lt = logT(A);
+    const int st = (1 << lt) + 1;
+    const int c = tid & ((1 << lt) - 1);
+    const TileU U = tile_uniform<A2>(A, tile);
+    u64 *dst = A.dst + U.dst_u + (i64)t * A.dst_coset_stride;
+#pragma unroll
+    for (int i = 0; i < 16 / E2; ++i) {
+        const int k1 = (tid + i * NTHREADS) >> lt;
+        const u32 off = (u32)c + ((u32)k1 << U.shk);
+        u64 x[E2];
+#pragma unroll
+        for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
+        VI_SCHED_FENCE();
+        dft_reg<A2, false>(x);
+        VI_SCHED_FENCE();
+#pragma unroll
+        for (int g = 0; g < E2; g += G) {
+            u64 tw[G];
+#pragma unroll
+            for (int j = 0; j < G; ++j) tw[j] = *at32(A.tw + U.tw_u + ((i64)(g + j) << U.sh2), off);
+#pragma unroll
+            for (int j = 0; j < G; ++j) VI_STREAM_STORE(at32(dst + ((i64)(g + j) << U.sh2), off), gl::mul(x[g + j], tw[j]));
+            VI_SCHED_FENCE();
+        }
+    }
+}
+
+// can passes Ai (last inverse) and Af (first forward, expanding into cosets) run as one fused launch?
+inline bool passes_fusable(const PassArgs &Ai_in, const PassArgs &Af_in) {
+    PassArgs Ai = Ai_in, Af = Af_in;
+    int nv = 16;
+    if (!Ai.is_final || Af.is_final || !Af.loop_cosets || !Ai.inverse || Af.inverse) return false;
+    if (Ai.a != Af.a || Ai.logn != Af.logn || Ai.logn != 2 * Ai.a || !fast_ok(Ai.a)) return false;
+    if (Ai.log_rho != 0 || Ai.pre || !Af.pre || Af.canon_src || Ai.n_rows != Af.n_rows) return false;
+    if (Af.src_width != ((i64)1 << Af.logn)) return false;
+    if (!pass_uniform(Ai, &nv) || nv != 16) return false;
+    if (!pass_uniform(Af, &nv) || nv != 16) return false;
+    return pass_tiles(Ai) == pass_tiles(Af);
 }
 
 }  // namespace ntt

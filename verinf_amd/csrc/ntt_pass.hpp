@@ -59,6 +59,7 @@ struct PassArgs {
     int canon_src;                            // src is caller data: reduce every word mod p on load
     int uniform;                              // register-blocked kernel: every tile is addressed by scalar bases (ntt_fast.hpp)
     int n1_valid;                             // uniform pass: how many of a thread's sixteen stage-1 inputs exist
+    int fuse_next;                            // last inverse pass of a coset extension: runs fused with the pass after it (dst may be null)
 };
 
 VI_HD int logT(const PassArgs &A) { return TILE_LOG - A.a; }

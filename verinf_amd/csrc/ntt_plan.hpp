@@ -175,7 +175,8 @@ inline i64 lde_ws_elems(int logK, int logN, i64 m) {
 inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre, int logN,
                              const u64 *in, i64 w, i64 in_stride, u64 *out, i64 out_stride,
                              u64 *ws, i64 m, std::vector<PassArgs> &passes,
-                             u64 *coeffs = nullptr, i64 coeffs_stride = 0, bool in_is_coeffs = false) {
+                             u64 *coeffs = nullptr, i64 coeffs_stride = 0, bool in_is_coeffs = false,
+                             bool allow_fuse = true) {
     const int logK = Ti.logn, log_rho = logN - logK, p = Ti.sp.p;
     const i64 K = (i64)1 << logK;
     u64 *C = coeffs ? coeffs : ws, *S = ws + m * K;
@@ -208,6 +209,24 @@ inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre,
         A.dst_coset_stride = m * K;
         if (last && !first) A.log_rho = log_rho;
         passes.push_back(A);
+    }
+    // K = L * L: the last inverse pass and the first forward pass run as one launch and the coefficients stay in
+    // registers.  The inverse intermediate then lives in the workspace's coefficient region (the forward planes
+    // are written while other workgroups still read it), and the coefficients go to memory only for the caller.
+    if (allow_fuse && !in_is_coeffs && p == 2) {
+        PassArgs &I0 = passes[passes.size() - 4], &I1 = passes[passes.size() - 3], &F0 = passes[passes.size() - 2];
+        PassArgs T0 = I0, T1 = I1;
+        T0.dst = ws;
+        T0.dst_row_stride = K;
+        T1.src = ws;
+        T1.src_row_stride = K;
+        T1.dst = coeffs;                                   // null when the caller does not want them
+        T1.dst_row_stride = coeffs ? coeffs_stride : K;
+        if (passes_fusable(T1, F0)) {
+            T1.fuse_next = 1;
+            I0 = T0;
+            I1 = T1;
+        }
     }
 }
 
