@@ -44,9 +44,13 @@ def _events(torch):
 
 
 def rand_field(torch, shape, seed):
-    """Seeded canonical field elements on the device (uniform below 2^63 < p)."""
+    """Seeded field elements on the device, uniform in [0, p): 64 random bits, and the 2^32 - 1 words at or
+    above p taken down by p (as tests/gpu_util.py does with `% p`)."""
     g = torch.Generator(device="cuda").manual_seed(seed)
-    return torch.randint(0, (1 << 63) - 1, shape, generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
+    v = torch.randint(-(1 << 63), (1 << 63) - 1, shape, generator=g, dtype=torch.int64, device="cuda")
+    # as unsigned words, [p, 2^64) is the signed range [-(2^32 - 1), -1]; x - p = x + 2^32 - 1 mod 2^64
+    v = torch.where((v < 0) & (v >= -((1 << 32) - 1)), v + ((1 << 32) - 1), v)
+    return v.view(torch.uint64)
 
 
 def bench_lde(torch, steps, warmup, ws_mb=0):
@@ -264,15 +268,21 @@ def bench_hash(torch, steps=10, cpu=True):
     return res
 
 
-def bench_layer(torch):
+def bench_layer(torch, check=True):
     """Config 5: one Llama-2-7B-shape layer proof core.  Commit = coset LDE of every weight
     and activation row at the production geometry ELL = 8192, K = 2^14, N = 2^16 (a row of
     n_in > 8192 values spans two rows); then the GKR sumchecks: one degree-2 contraction
     per matmul (width next_pow2(n_in), layergkr/full_layer.py:216-224) and one degree-3
     eq*a*b gate batch over S*d_ff -> 2^24 (layergkr/relations.py:104-124).  Every committed
-    matrix is hashed by column and gets its Merkle root (layergkr/rs.py:176-187).  Random field
-    tables stand in for the projected vectors of the sumchecks."""
+    matrix is hashed by column and gets its Merkle root (layergkr/rs.py:176-187); the digests
+    and tree of a matrix run on a second stream while the next matrix is encoded.  Random field
+    tables stand in for the projected vectors of the sumchecks.
+
+    check: after the timed regions, verify the full-shape run by samples and by properties (rows, column
+    digests and roots against the CPU oracle, the codeword property on every row, every sumcheck through
+    the verifier, the projection against big-integer sums); the verdicts come back under "checks"."""
     from verinf_amd.layergkr import gpu
+    from verinf_amd.layergkr import sumcheck as sc
     from verinf_amd.prover import cuda_primitives as cp
     d, dff, S = 4096, 11008, 1000
     ELL, K, N = 8192, 1 << 14, 1 << 16
@@ -305,14 +315,26 @@ def bench_layer(torch):
     z = [r.randrange(P) for _ in range(24)]
     # gate batch eq(z, .) * a * b: the eq table is built on the device, the two witness tables are random
     gate_tabs = [gpu.eq_vector_t(z)] + [rand_field(torch, (1 << 24,), 200 + j) for j in range(2)]
+    hash_stream = torch.cuda.Stream()                     # default priority, like the stream the encoder runs on
 
-    def commit(hash_too=True):
-        roots = []
+    def commit(hash_too=True, overlap=True):
+        """-> [(digests, root)] per committed matrix"""
+        done = []
+        main = torch.cuda.current_stream()
         for m, code in zip(msgs, codes):
             cp.coset_lde(m, K, N, 7, out=code)
-            if hash_too:
-                roots.append(cp.merkle_build_blake3(cp.hash_columns_streamed(code))[0])
-        return roots
+            if not hash_too:
+                continue
+            if overlap:
+                hash_stream.wait_stream(main)
+                with torch.cuda.stream(hash_stream):
+                    dig = cp.hash_columns_streamed(code)
+                    done.append((dig, cp.merkle_build_blake3(dig)[0]))
+            else:
+                dig = cp.hash_columns_streamed(code)
+                done.append((dig, cp.merkle_build_blake3(dig)[0]))
+        main.wait_stream(hash_stream)
+        return done
 
     def sumchecks():
         for tabs in mm_tabs:
@@ -325,20 +347,23 @@ def bench_layer(torch):
     def projections():
         """chi^T C per committed weight block: the (1 x rows) @ (rows x N) combination of
         layergkr/gpu.py:301-308 / projection.py:150-167; streams every weight codeword once."""
-        for chi, code in zip(chis, codes[:n_w]):
-            cp.gl_matmul(chi, code)
+        return [cp.gl_matmul(chi, code) for chi, code in zip(chis, codes[:n_w])]
 
-    commit(); projections(); sumchecks()         # warm-up (twiddle tables, workspaces)
+    commit(); commit(overlap=False); projections(); sumchecks()         # warm-up (twiddle tables, workspaces)
     torch.cuda.synchronize()
     tl0 = time.perf_counter()
     commit(hash_too=False)
     torch.cuda.synchronize()
     lde_only_s = time.perf_counter() - tl0
+    ts0 = time.perf_counter()
+    commit(overlap=False)
+    torch.cuda.synchronize()
+    seq_commit_s = time.perf_counter() - ts0
     t0 = time.perf_counter()
-    commit()
+    committed = commit()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    projections()
+    projected = projections()
     torch.cuda.synchronize()
     tp = time.perf_counter()
     proj_ms = (tp - t1) * 1e3
@@ -363,18 +388,90 @@ def bench_layer(torch):
     t7 = time.perf_counter()
     gpu.mle_eval_t(stacked, coins)                       # the terminal evaluations the verifier's last check needs
     t8 = time.perf_counter()
+    del stacked
     lde_bytes = 8 * (K + N) * total_rows
-    return {"rows_committed": total_rows, "geometry": "ELL=8192 K=2^14 N=2^16",
-            "end_to_end_ms": (t2 - t0) * 1e3,
-            "projection_matvec_ms": proj_ms, "projection_matvec_gbs": proj_bytes / proj_ms / 1e6,
-            "commit_ms": (t1 - t0) * 1e3, "commit_hash_and_tree_ms": (t1 - t0 - lde_only_s) * 1e3,
-            "commit_lde_ms": lde_only_s * 1e3, "commit_lde_gbs_algorithmic": lde_bytes / lde_only_s / 1e9,
-            "commit_lde_gelems_per_s": total_rows * N / lde_only_s / 1e9,
-            "sumchecks_ms": (t2 - t1b) * 1e3,
-            "gate_sumcheck_2^24_deg3_ms": (t4 - t3) * 1e3,
-            "gate_sumcheck_gbs_algorithmic": 96 * (1 << 24) / (t4 - t3) / 1e9,
-            "eq_vector_2^24_ms": (t6 - t5) * 1e3, "mle_eval_3x2^24_ms": (t8 - t7) * 1e3,
-            "matmul_sumchecks": "6 x width 2^12 + 1 x width 2^14, degree 2 (launch-latency bound)"}
+    res = {"rows_committed": total_rows, "geometry": "ELL=8192 K=2^14 N=2^16",
+           "end_to_end_ms": (t2 - t0) * 1e3,
+           "projection_matvec_ms": proj_ms, "projection_matvec_gbs": proj_bytes / proj_ms / 1e6,
+           "commit_ms": (t1 - t0) * 1e3, "commit_sequential_ms": seq_commit_s * 1e3,
+           "commit_hash_and_tree_ms": (seq_commit_s - lde_only_s) * 1e3,
+           "commit_hash_and_tree_exposed_ms": (t1 - t0 - lde_only_s) * 1e3,
+           "commit_lde_ms": lde_only_s * 1e3, "commit_lde_gbs_algorithmic": lde_bytes / lde_only_s / 1e9,
+           "commit_lde_gelems_per_s": total_rows * N / lde_only_s / 1e9,
+           "sumchecks_ms": (t2 - t1b) * 1e3,
+           "gate_sumcheck_2^24_deg3_ms": (t4 - t3) * 1e3,
+           "gate_sumcheck_gbs_algorithmic": 96 * (1 << 24) / (t4 - t3) / 1e9,
+           "eq_vector_2^24_ms": (t6 - t5) * 1e3, "mle_eval_3x2^24_ms": (t8 - t7) * 1e3,
+           "matmul_sumchecks": "6 x width 2^12 + 1 x width 2^14, degree 2 (launch-latency bound)",
+           "note": "commit_ms: digests and tree of matrix i on a second stream while matrix i+1 is encoded; "
+                   "commit_sequential_ms: one stream"}
+    if check:
+        res["checks"] = _check_layer(torch, msgs, codes, committed, chis, projected, mm_tabs, gate_tabs, coins, K, N, n_w)
+    return res
+
+
+def _check_layer(torch, msgs, codes, committed, chis, projected, mm_tabs, gate_tabs, coins, K, N, n_w):
+    """The full-shape layer run against the CPU oracle by samples, and by properties over everything."""
+    import numpy as np
+    from oracle import oracle as O
+    from verinf_amd.layergkr import sumcheck as sc
+    from verinf_amd.prover import cuda_primitives as cp
+    out = {}
+    # sampled rows of four matrices (a square weight, the narrow second block of Wdown, two activations)
+    which = [0, 7, n_w, len(msgs) - 1]
+    ok = True
+    for i in which:
+        m = int(msgs[i].shape[0])
+        rows = sorted({0, m // 2, m - 1})
+        sample = msgs[i].view(torch.int64)[rows].contiguous().view(torch.uint64).cpu().numpy()
+        got = codes[i].view(torch.int64)[rows].contiguous().view(torch.uint64).cpu().numpy()
+        ok = ok and bool(np.array_equal(got, O.coset_lde_rows(sample, K, N, 7)))
+    out["sampled_rows_match_oracle"] = ok
+    # every row of every committed matrix is a codeword: its interpolant on the coset has no coefficient >= K
+    ok = True
+    for code in codes:
+        for lo in range(0, int(code.shape[0]), 4096):
+            blk = code[lo:lo + 4096].clone()
+            cp.ntt_inverse_batched(blk)
+            ok = ok and not bool(blk.view(torch.int64)[:, K:].any())
+            del blk
+    out["every_row_is_a_codeword"] = ok
+    # sampled column digests against the oracle's BLAKE3, and each root against the oracle's tree over the digests
+    ok_d = ok_r = True
+    for i in which:
+        dig, root = committed[i]
+        cols = [0, 777, N - 1]
+        sub = codes[i].view(torch.int64)[:, cols].contiguous().view(torch.uint64).cpu().numpy()
+        want = O.hash_columns(sub)
+        ok_d = ok_d and bool(np.array_equal(dig.cpu().numpy()[cols], want))
+        levels = O.merkle_levels(dig.cpu().numpy())
+        ok_r = ok_r and levels[-1][0].tobytes() == bytes(root.cpu().tolist())
+    out["sampled_column_digests_match_oracle"] = ok_d
+    out["roots_match_oracle_tree"] = ok_r
+    # the projection chi^T C on sampled columns against big-integer sums
+    ok = True
+    for i in (0, n_w - 1):
+        chi = [int(v) for v in chis[i].cpu().numpy().reshape(-1)]
+        for col in (0, 12345, N - 1):
+            column = [int(v) for v in codes[i].view(torch.int64)[:, col].contiguous().view(torch.uint64).cpu().numpy()]
+            ok = ok and sum(a * b for a, b in zip(chi, column)) % P == int(projected[i].view(torch.int64)[0, col].item()) % (1 << 64)
+    out["projection_matches_bigint_sums"] = ok
+    # every sumcheck of the layer through the verifier (round consistency + terminal evaluations on the device)
+    ok = True
+    for tabs in mm_tabs + [gate_tabs]:
+        terms = [(1, tabs)]
+        proof = sc.prove_terms(terms, lambda i: coins[i])
+        good, _ = sc.verify_terms(proof, terms, lambda i: coins[i])
+        ok = ok and good
+    out["sumchecks_verify"] = ok
+    # ... and a tampered table is rejected
+    terms = [(1, gate_tabs)]
+    proof = sc.prove_terms(terms, lambda i: coins[i])
+    gate_tabs[2].view(torch.int64)[54321] += 1
+    bad, _ = sc.verify_terms(proof, terms, lambda i: coins[i])
+    gate_tabs[2].view(torch.int64)[54321] -= 1
+    out["tampered_table_rejected"] = not bad
+    return out
 
 
 def copy_probe(torch):

@@ -13,6 +13,15 @@ def rand_field(shape, seed):
     return a % np.uint64(P)
 
 
+def rand_field_dev(shape, seed):
+    """The same distribution drawn on the device (for shapes too large to draw on the host): 64 random bits,
+    the 2^32 - 1 words at or above p taken down by p."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    v = torch.randint(-(1 << 63), (1 << 63) - 1, shape, generator=g, dtype=torch.int64, device="cuda")
+    v = torch.where((v < 0) & (v >= -((1 << 32) - 1)), v + ((1 << 32) - 1), v)     # [p, 2^64) as signed words
+    return v.view(torch.uint64)
+
+
 def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 

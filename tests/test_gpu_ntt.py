@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 torch = pytest.importorskip("torch")
 from oracle import oracle as O  # noqa: E402
-from tests.gpu_util import P, rand_field, to_dev, to_np, unhex  # noqa: E402
+from tests.gpu_util import P, rand_field, rand_field_dev, to_dev, to_np, unhex  # noqa: E402
 
 
 @pytest.fixture(scope="module")
@@ -236,8 +236,8 @@ def test_lde_full_baseline_shape_properties(cp):
     """The headline LDE shape (1024 x 2^16 -> 2^18): bit-exact against the oracle on a
     row sample, codeword property (inverse transform has no coefficient >= K) on all rows."""
     K, N, m = 1 << 16, 1 << 18, 1024
-    g = torch.Generator(device="cuda").manual_seed(2)
-    msgs = torch.randint(0, (1 << 63) - 1, (m, K), generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
+    msgs = rand_field_dev((m, K), 2)                     # uniform in [0, p), words above 2^63 included
+    assert int((msgs.view(torch.int64) < 0).sum()) > m * K // 4
     out = cp.coset_lde(msgs, K, N, 7)
     rows = [0, 1, 511, 1023]
     sample = to_np(msgs.view(torch.int64)[rows].contiguous().view(torch.uint64))

@@ -138,11 +138,23 @@ _ws_cache = {}
 
 
 def workspace(nbytes: int, device=None, tag: str = "ws"):
-    """A cached uint8 device buffer of at least nbytes (grown, never shrunk)."""
+    """A cached uint8 device buffer of at least nbytes for the CURRENT stream of `device`.
+
+    One buffer per (purpose, device, stream): the wrappers launch on torch's current stream, so two streams
+    (or two host threads on their own streams) never share scratch, and a buffer is only ever used on the
+    stream it was allocated on -- when it is outgrown and dropped, the caching allocator may reuse its memory
+    in stream order without further bookkeeping.  Buffers grow and are kept; release_workspaces() drops them."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
-    key = (tag, device.index)
+    key = (tag, device.index, torch.cuda.current_stream(device).cuda_stream)
     buf = _ws_cache.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        with torch.cuda.device(device):
+            buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
         _ws_cache[key] = buf
     return buf
+
+
+def release_workspaces() -> None:
+    """Drop every cached scratch buffer (they come back on demand).  Call it with the device idle: a buffer
+    still in use by queued kernels must not be handed back to the allocator from another stream."""
+    _ws_cache.clear()

@@ -22,6 +22,7 @@ mle_eval work on Python lists).  The dense Lagrange-matrix encoders
 the one encoder here.
 """
 import ctypes
+import threading
 from typing import Optional, Sequence
 
 import torch
@@ -387,14 +388,20 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
     return claim, round_polys, challenges, mu
 
 
-_PINNED = {}
+_PINNED = threading.local()
 
 
 def _pinned_samples():
-    """8 pinned host words the round kernels write their samples into (one per process)."""
-    if "buf" not in _PINNED:
-        _PINNED["buf"] = torch.zeros(8, dtype=torch.uint64).pin_memory()
-    return _PINNED["buf"]
+    """8 pinned host words the round kernels write their samples into.  One buffer per host thread and stream:
+    a proof waits for each round's samples before it goes on, so a thread needs one per stream it drives, and
+    two threads (or two streams) never see each other's samples."""
+    bufs = getattr(_PINNED, "bufs", None)
+    if bufs is None:
+        bufs = _PINNED.bufs = {}
+    key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
+    if key not in bufs:
+        bufs[key] = torch.zeros(8, dtype=torch.uint64).pin_memory()
+    return bufs[key]
 
 
 def _poly_eval(coeffs: Sequence[int], x: int, p: int) -> int:

@@ -130,10 +130,15 @@ def _is_pow2(n):
     return n > 0 and (n & (n - 1)) == 0
 
 
+_NTT_WS_CAP = 1 << 30
+
+
 def _ntt(rows, m, n, inverse):
     L = _lib.lib()
     with torch.cuda.device(rows.device):
-        need = L.vi_ntt_workspace_bytes(m, n)
+        # the library transforms the rows in chunks that fit the workspace it is given: one row is the minimum,
+        # 1 GiB is enough to fill the GPU, and a large batch does not double its footprint for the process's life
+        need = min(L.vi_ntt_workspace_bytes(m, n), max(_NTT_WS_CAP, n * 8))
         ws = _lib.workspace(need, rows.device, "ntt") if need else None
         _lib.check(L.vi_ntt_batched(rows.data_ptr(), m, n, int(inverse),
                                     ws.data_ptr() if ws is not None else None,
