@@ -8,7 +8,10 @@
  * an entry point allocates no device memory: scratch is passed in as a workspace
  * whose size the matching *_workspace_bytes() query returns.  Twiddle tables are
  * the exception: they are built once per (length, direction, device) on first use
- * and cached for the life of the process, like the reference's NTT contexts.
+ * and cached for the life of the process, like the reference's NTT contexts.  That
+ * first use of a length (and of a coset shift) allocates and copies synchronously;
+ * only later calls with it are asynchronous.  Coset multiplier tables (N words per
+ * (K, N, shift, device)) are kept for the sixteen most recently used combinations.
  *
  * All field elements are uint64 words, canonical in [0, p), p = 2^64 - 2^32 + 1.
  * "reference" below = JamesPetrie/VerInf; each entry point names the interface it

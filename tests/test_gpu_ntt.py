@@ -232,6 +232,25 @@ def test_lde_gates_and_layergkr_entry_points():
     assert c.n_rows == 4 and c.col_values(5) == [int(v) for v in got[:, 5]]
 
 
+def test_dense_lagrange_encoder_and_its_gate():
+    """The reference's dense encoder surface (layergkr/gpu.py:80-122, 256-271, 413-434; rs.py:66-77): the matrix
+    against the closed form in Python integers, the matmul encoder against the NTT encoder, the gate green."""
+    from verinf_amd.layergkr import gpu, rs
+    from verinf_amd.prover.protocol import lagrange
+    r = random.Random(8)
+    for cfg in (rs.Config(ELL=16, K_DEG=32, N_LIG=64, T_QUERIES=4), rs.Config(ELL=64, K_DEG=128, N_LIG=256, T_QUERIES=8)):
+        assert gpu.selftest(cfg, n_rows=2) is None
+        L = rs.lagrange_matrix(cfg)
+        assert len(L) == cfg.N_LIG and len(L[0]) == cfg.ELL
+        for _ in range(40):
+            j, c = r.randrange(cfg.N_LIG), r.randrange(cfg.ELL)
+            assert L[j][c] == lagrange(cfg, c, cfg.eta(j))
+        rows = [[r.randrange(P) for _ in range(k)] for k in (cfg.ELL, 5, 0)]
+        dense = gpu.encode_batch_t(cfg, rows)
+        assert torch.equal(dense, gpu.encode_batch_ntt(cfg, rows))
+        assert gpu.encode_batch(cfg, rows) == [[int(v) for v in row] for row in to_np(dense)]
+
+
 def test_lde_full_baseline_shape_properties(cp):
     """The headline LDE shape (1024 x 2^16 -> 2^18): bit-exact against the oracle on a
     row sample, codeword property (inverse transform has no coefficient >= K) on all rows."""

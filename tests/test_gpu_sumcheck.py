@@ -127,6 +127,27 @@ def test_degree_above_three_and_limits(mods):
         gpu.prove_terms_gpu([(1, [obj[0]] * 8)], lambda i: 1, P)          # degree 8 is above the kernel limit
 
 
+@pytest.mark.parametrize("v,nt,terms", [(3, 2, [(1, [0, 1])]), (11, 3, [(1, [0, 1, 2])]),
+                                        (12, 4, [(3, [0, 1, 2]), (P - 5, [0, 3])]),
+                                        (9, 10, [(3, [0, 1, 2]), (P - 5, [3]), (7, [4, 5]), (11, [6]), (13, [7, 8, 9, 0])])])
+def test_tables_with_words_at_or_above_p_are_taken_as_residues(mods, v, nt, terms):
+    """A caller's tensor may hold any 64-bit word (the reference's add / sub / mul chain stays congruent on them):
+    p, p + 1 and 2^64 - 1 in the tables give the proof of their residues."""
+    gpu, _ = mods
+    tabs = [rand_field(1 << v, 500 + v + j) for j in range(nt)]
+    raw = [t.copy() for t in tabs]
+    for j, t in enumerate(raw):
+        for pos, word in ((0, P), (1, P + 1), (t.size - 1, (1 << 64) - 1), (t.size // 2, P + 12345), (t.size // 2 + 1, P)):
+            t[(pos + j) % t.size] = np.uint64(word)
+    residues = [np.array([int(x) % P for x in t], dtype=np.uint64) for t in raw]
+    coins, coin = _coins(v, 77)
+    objs = [to_dev(t) for t in raw]
+    claim, polys, chals, _ = gpu.prove_terms_gpu([(c, [objs[i] for i in fs]) for c, fs in terms], coin, P)
+    want_claim, want_samples, _ = O.sumcheck_prove(residues, terms, coins)
+    assert claim == want_claim
+    assert [[y for _, y in s] for s in polys] == want_samples
+
+
 def test_large_instance_matches_oracle(mods):
     """2^22 x 3 factors, degree 3, 22 rounds: every round's samples against the C oracle."""
     gpu, _ = mods

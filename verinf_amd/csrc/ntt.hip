@@ -160,7 +160,11 @@ std::map<std::tuple<int, int, int, u64>, u64 *> g_pre;               // (device,
 int upload(const std::vector<u64> &h, u64 **out) {
     void *d = nullptr;
     VI_HIP(hipMalloc(&d, h.size() * sizeof(u64)));
-    VI_HIP(hipMemcpy(d, h.data(), h.size() * sizeof(u64), hipMemcpyHostToDevice));
+    hipError_t e = hipMemcpy(d, h.data(), h.size() * sizeof(u64), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(d);
+        return vi::fail(VI_EHIP, "upload of a twiddle table: %s", hipGetErrorString(e));
+    }
     *out = (u64 *)d;
     return VI_OK;
 }
@@ -178,7 +182,8 @@ int get_twl(int dev, int inv, const u64 **out) {
     return VI_OK;
 }
 
-// tables of one (logn, direction) on the current device; built on first use
+// tables of one (logn, direction) on the current device; built on first use (which allocates and copies
+// synchronously; later calls with the same length only look the tables up)
 int get_tables(int logn, int inv, const Tables **out) {
     int dev = 0;
     VI_HIP(hipGetDevice(&dev));
@@ -192,33 +197,39 @@ int get_tables(int logn, int inv, const Tables **out) {
         D->T.logn = logn;
         D->T.scale = H.scale;
         D->T.inverse = inv;
-        for (int q = 0; q < 4; ++q) {
-            D->T.twi[q] = nullptr;
-            if (!H.twi[q].empty()) {
-                u64 *d = nullptr;
-                int rc = upload(H.twi[q], &d);
-                if (rc) return rc;
-                D->T.twi[q] = d;
-                D->owned.push_back(d);
-            }
+        int rc = VI_OK;
+        for (int q = 0; q < 4; ++q) D->T.twi[q] = nullptr;
+        for (int q = 0; q < 3; ++q) D->T.tw[q] = nullptr;
+        for (int q = 0; q < 4 && !rc; ++q) {
+            if (H.twi[q].empty()) continue;
+            u64 *d = nullptr;
+            rc = upload(H.twi[q], &d);
+            if (!rc) { D->T.twi[q] = d; D->owned.push_back(d); }
         }
-        for (int q = 0; q < 3; ++q) {
-            D->T.tw[q] = nullptr;
-            if (!H.tw[q].empty()) {
-                u64 *d = nullptr;
-                int rc = upload(H.tw[q], &d);
-                if (rc) return rc;
-                D->T.tw[q] = d;
-                D->owned.push_back(d);
-            }
+        for (int q = 0; q < 3 && !rc; ++q) {
+            if (H.tw[q].empty()) continue;
+            u64 *d = nullptr;
+            rc = upload(H.tw[q], &d);
+            if (!rc) { D->T.tw[q] = d; D->owned.push_back(d); }
         }
-        int rc = get_twl(dev, inv, &D->T.twl);
-        if (rc) return rc;
+        if (!rc) rc = get_twl(dev, inv, &D->T.twl);
+        if (rc) {                                          // give back what was uploaded before the failure
+            for (void *p : D->owned) (void)hipFree(p);
+            delete D;
+            return rc;
+        }
         it = g_tables.emplace(key, D).first;
     }
     *out = &it->second->T;
     return VI_OK;
 }
+
+// Coset multiplier tables are N words each and depend on the shift: the most recently used MAX_PRE per process are
+// kept, the least recently used one is freed when a new one is needed (hipFree waits for the kernels that may still
+// read it).
+constexpr size_t MAX_PRE = 16;
+u64 g_pre_clock = 0;
+std::map<std::tuple<int, int, int, u64>, u64> g_pre_used;            // key -> time of last use
 
 int get_pre(int logK, int logN, u64 shift, const u64 **out) {
     int dev = 0;
@@ -227,11 +238,25 @@ int get_pre(int logK, int logN, u64 shift, const u64 **out) {
     auto key = std::make_tuple(dev, logK, logN, shift);
     auto it = g_pre.find(key);
     if (it == g_pre.end()) {
+        if (g_pre.size() >= MAX_PRE) {
+            auto oldest = g_pre_used.begin();
+            for (auto u = g_pre_used.begin(); u != g_pre_used.end(); ++u)
+                if (u->second < oldest->second) oldest = u;
+            auto victim = g_pre.find(oldest->first);
+            int vdev = std::get<0>(victim->first);
+            if (vdev != dev) VI_HIP(hipSetDevice(vdev));
+            hipError_t e = hipFree(victim->second);
+            if (vdev != dev) VI_HIP(hipSetDevice(dev));
+            if (e != hipSuccess) return vi::fail(VI_EHIP, "hipFree of a coset table: %s", hipGetErrorString(e));
+            g_pre.erase(victim);
+            g_pre_used.erase(oldest);
+        }
         u64 *d = nullptr;
         int rc = upload(make_coset_pre(logK, logN, shift), &d);
         if (rc) return rc;
         it = g_pre.emplace(key, d).first;
     }
+    g_pre_used[key] = ++g_pre_clock;
     *out = it->second;
     return VI_OK;
 }

@@ -96,8 +96,9 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
             if (PROD || t < D.n_tables) {
                 const u64 *f = D.src[t];
                 if (MODE == 0) {
-                    lo_u[u][t] = f[i];
-                    hi_u[u][t] = f[half + i];
+                    // caller data: any 64-bit word is taken as its residue (the ladders below add canonical values)
+                    lo_u[u][t] = gl::canon(f[i]);
+                    hi_u[u][t] = gl::canon(f[half + i]);
                 } else if (MODE == 1) {
                     D.dst[t][i] = fold1(f[i], f[half + i], r);
                 } else {
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
             u64 lc = D.c0, ld = 0;
             for (int k = 0; k < D.n_lin; ++k) {
                 const u64 *f = D.src[D.lin_idx[k]];
-                const u64 c = D.lin_coeff[k], cur = f[i], dif = gl::sub(f[half + i], cur);
+                const u64 c = D.lin_coeff[k], cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
                 lc = gl::add(lc, gl::mul(c, cur));
                 ld = gl::add(ld, gl::mul(c, dif));
             }
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
             for (int x = 0; x < NSAMP; ++x) prod[x] = D.coeff[k];
             for (int j = D.term_off[k]; j < D.term_off[k + 1]; ++j) {
                 const u64 *f = D.src[D.fidx[j]];
-                u64 cur = f[i], dif = gl::sub(f[half + i], cur);
+                u64 cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
 #pragma unroll
                 for (int x = 0; x < NSAMP; ++x) {
                     if (x <= D.deg) prod[x] = gl::mul(prod[x], cur);
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
         }
         if (D.common >= 0) {
             const u64 *f = D.src[D.common];
-            u64 cur = f[i], dif = gl::sub(f[half + i], cur);
+            u64 cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
 #pragma unroll
             for (int x = 0; x < NSAMP; ++x) {
                 if (x <= D.deg) sx[x] = gl::mul(sx[x], cur);
@@ -448,7 +449,17 @@ int resident_blocks(K kernel, int max_per_cu) {
 
 template <int NT, int MODE, int U, bool PROD, int NS>
 int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
-    static const int cap = resident_blocks(k_round<NT, MODE, U, PROD, NS>, MODE == 2 ? 5 : 64);     // per instantiation, first use
+    // per instantiation and device, looked up on first use there (devices of one process may differ)
+    static std::mutex mu;
+    static int caps[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    int cap;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (!caps[dev]) caps[dev] = resident_blocks(k_round<NT, MODE, U, PROD, NS>, MODE == 2 ? 5 : 64);
+        cap = caps[dev];
+    }
     if (nb > cap) nb = cap;
     hipLaunchKernelGGL((k_round<NT, MODE, U, PROD, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
     return nb;
@@ -571,6 +582,16 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
     const bool eval = out_samples != nullptr;
     Desc D;
     if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
+    if (!eval && src && n_tables > VI_SC_MAX_TABLES) {
+        // folding alone has no limit on the number of tables: a descriptor's worth at a time
+        for (int t0 = 0; t0 < n_tables; t0 += VI_SC_MAX_TABLES) {
+            const int cnt = (n_tables - t0 < VI_SC_MAX_TABLES) ? (n_tables - t0) : VI_SC_MAX_TABLES;
+            int rc = vi_sumcheck_fold_eval(src + t0, dst + t0, cnt, half, r, nullptr, nullptr, nullptr, 0, nullptr, nullptr,
+                                           nullptr, 0, stream);
+            if (rc) return rc;
+        }
+        return VI_OK;
+    }
     int rc = fill_desc(D, src, dst, n_tables, term_off, factor_idx, coeffs, n_terms, eval, "vi_sumcheck_fold_eval");
     if (rc) return rc;
     if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: half = %lld", (long long)half);

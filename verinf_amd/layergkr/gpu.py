@@ -411,7 +411,65 @@ def _poly_eval(coeffs: Sequence[int], x: int, p: int) -> int:
     return acc
 
 
+# ---- dense Lagrange encoder (layergkr/gpu.py:80-122, 256-271) ------------------------------------------
+_LAGRANGE_GPU = {}
+
+
+def lagrange_gpu(cfg: Config):
+    """The ELL x N_LIG matrix L[c][j] = L_c(eta_j) = zeta_c (eta_j^K - 1) / (K (eta_j - zeta_c)) as a device tensor,
+    cached per geometry.  The two domains go up as vectors; the ELL * N_LIG differences are inverted on the device
+    with one batched inversion, so no entry is computed on the host."""
+    _require_gpu()
+    key = (cfg.ELL, cfg.K_DEG, cfg.N_LIG, torch.cuda.current_device())
+    if key not in _LAGRANGE_GPU:
+        k_inv = pow(cfg.K_DEG, P - 2, P)
+        eta, zeta, num = [], [], []
+        e, w_n = GLOBAL_G % P, cfg.W_N
+        for _ in range(cfg.N_LIG):
+            eta.append(e)
+            num.append((pow(e, cfg.K_DEG, P) - 1) * k_inv % P)        # (eta^K - 1) / K
+            e = e * w_n % P
+        z, w_k = 1, cfg.W_K
+        for _ in range(cfg.ELL):
+            zeta.append(z)
+            z = z * w_k % P
+        eta_t, num_t, zeta_t = _u64_row(eta), _u64_row(num), _u64_row(zeta)
+        zeta_cols = zeta_t.view(torch.int64).view(-1, 1).expand(cfg.ELL, cfg.N_LIG).contiguous().view(torch.uint64)
+        eta_rows = eta_t.view(torch.int64).view(1, -1).expand(cfg.ELL, cfg.N_LIG).contiguous().view(torch.uint64)
+        inv = cp.gl_inv_batched(cp.gl_sub(eta_rows, zeta_cols).view(-1)).view(cfg.ELL, cfg.N_LIG)
+        _LAGRANGE_GPU[key] = cp.gl_mul(cp.gl_mul_bcast(inv, num_t.view(-1)), zeta_cols)
+    return _LAGRANGE_GPU[key]
+
+
+def encode_batch_t(cfg: Config, messages):
+    """(rows x ELL) @ (ELL x N_LIG) over the field, result left on the device (gpu.py:256-271): the dense form of
+    the encoder, O(ELL * N_LIG) per row -- for small geometries and as a cross-check of encode_batch_ntt."""
+    _require_gpu()
+    return cp.gl_matmul(_to_device_rows(messages, cfg.ELL), lagrange_gpu(cfg))
+
+
+def encode_batch(cfg: Config, messages):
+    """The same as Python lists (gpu.py:92-111)."""
+    return [[int(v) for v in row] for row in encode_batch_t(cfg, messages).cpu().tolist()]
+
+
 def selftest(cfg: Config, n_rows: int = 4, seed: int = 1) -> Optional[str]:
-    """Gate of the encoder against the definition (the reference's `selftest`,
-    gpu.py:413-434, gates its dense matmul encoder; here the one encoder is the NTT one)."""
-    return selftest_ntt(cfg, n_rows=n_rows, seed=seed)
+    """Gate of the dense encoder and of the linear combination against the definition on the host
+    (prover.protocol.eval_zeta_form, Python integers), as gpu.py:413-434.  None on agreement."""
+    if not available():
+        return "no CUDA"
+    import random
+    from ..prover.protocol import eval_zeta_form
+    r = random.Random(seed)
+    msgs = [[r.randrange(P) for _ in range(cfg.ELL)] for _ in range(n_rows)]
+    got = encode_batch(cfg, msgs)
+    want = [[eval_zeta_form(cfg, m, cfg.eta(j)) for j in range(cfg.N_LIG)] for m in msgs]
+    for i in range(n_rows):
+        if want[i] != got[i]:
+            j = next(k for k in range(cfg.N_LIG) if want[i][k] != got[i][k])
+            return f"row {i} column {j}: definition {want[i][j]} != dense {got[i][j]}"
+    co = [r.randrange(P) for _ in range(n_rows)]
+    comb = [sum(c * row[j] for c, row in zip(co, want)) % P for j in range(cfg.N_LIG)]
+    if comb != [int(v) for v in linear_combination(cfg, want, co)]:
+        return "linear_combination disagrees"
+    return None

@@ -12,6 +12,7 @@ builds the Merkle tree there, and only the tree (32 bytes per node) and the open
 columns come back to the host.
 """
 from typing import List, Sequence, Tuple
+import torch
 
 from ..prover.protocol import (  # noqa: F401  (re-exported like the reference)
     Config, P, blake3_digest, eval_zeta_form, merkle_leaf, merkle_verify)
@@ -61,6 +62,13 @@ def _ntt_ok(cfg: Config) -> bool:
         else:
             _NTT_OK[key] = gpu.selftest_ntt_spot(cfg) is None
     return _NTT_OK[key]
+
+
+def lagrange_matrix(cfg: Config) -> List[List[int]]:
+    """L[j][c] = L_c(eta_j) as Python integers, N_LIG rows of ELL entries (rs.py:66-77): the device-built dense
+    matrix of gpu.lagrange_gpu brought to the host (the definition itself is prover.protocol.lagrange)."""
+    from . import gpu
+    return [[int(v) for v in row] for row in gpu.lagrange_gpu(cfg).view(torch.int64).t().contiguous().view(torch.uint64).cpu().tolist()]
 
 
 def encode_row(cfg: Config, message: Sequence[int]) -> Codeword:

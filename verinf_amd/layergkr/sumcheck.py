@@ -45,42 +45,51 @@ def _lagrange_interpolate(points: Sequence[Tuple[int, int]], x: int) -> int:
 
 
 # ---- mask tape -----------------------------------------------------------------------
-@dataclass
+# Interface of layergkr/sumcheck.py:74-111.  A masked round adds a scalar polynomial h of the round's degree d
+# to the samples.  h is fixed by d tape words and the running value mu: the tape supplies the coefficients of
+# x^1 .. x^d, and the constant term follows from h(0) + h(1) = 2 h_0 + (h_1 + ... + h_d) = mu.
 class MaskTape:
-    """Fresh field elements committed before any challenge."""
-    values: List[int]
-    pos: int = 0
+    """Field elements drawn (and committed to) before the first challenge, consumed front to back."""
+
+    def __init__(self, values, pos: int = 0):
+        self.values = list(values)
+        self.pos = pos
+
+    def remaining(self) -> int:
+        return len(self.values) - self.pos
 
     def take(self, n: int) -> List[int]:
-        if self.pos + n > len(self.values):
+        if n > self.remaining():
             raise RuntimeError("mask tape exhausted")
-        out = self.values[self.pos:self.pos + n]
-        self.pos += n
-        return out
+        start, self.pos = self.pos, self.pos + n
+        return self.values[start:self.pos]
 
 
 def mask_poly_coeffs(mu: int, u: Sequence[int]) -> List[int]:
-    """Ascending coefficients [a0, u_1..u_d] of h with h(0) + h(1) = mu."""
-    a0 = (mu - sum(u)) % FIELD_P * INV2 % FIELD_P
-    return [a0] + [x % FIELD_P for x in u]
+    """[h_0, h_1, ..., h_d], lowest degree first, for tape words u = (h_1 .. h_d) and running value mu."""
+    upper = [int(w) % FIELD_P for w in u]
+    h0 = (mu - sum(upper)) * INV2 % FIELD_P
+    return [h0, *upper]
 
 
 def poly_eval_coeffs(coeffs: Sequence[int], x: int) -> int:
-    acc = 0
-    for c in reversed(coeffs):
-        acc = (acc * x + c) % FIELD_P
-    return acc
+    """Value at x of the polynomial with the given coefficients, lowest degree first."""
+    value, power = 0, 1
+    for c in coeffs:
+        value = (value + c * power) % FIELD_P
+        power = power * x % FIELD_P
+    return value
 
 
 def solve_tape_for_target(mu: int, target_h: Sequence[int]) -> Optional[List[int]]:
-    """The unique tape producing mask polynomial `target_h`, or None if it is not in
-    the affine space h(0) + h(1) = mu."""
-    if not target_h:
+    """The tape words that make mask_poly_coeffs(mu, .) equal target_h, or None when target_h does not
+    satisfy h(0) + h(1) = mu (then no tape produces it).  The map tape -> h is injective: the words are
+    h's non-constant coefficients."""
+    h = [int(c) % FIELD_P for c in target_h]
+    if not h:
         return None
-    if (poly_eval_coeffs(target_h, 0) + poly_eval_coeffs(target_h, 1)) % FIELD_P != mu % FIELD_P:
-        return None
-    u = [c % FIELD_P for c in target_h[1:]]
-    return u if mask_poly_coeffs(mu, u) == [c % FIELD_P for c in target_h] else None
+    words = h[1:]
+    return words if mask_poly_coeffs(mu, words) == h else None
 
 
 # ---- proofs ----------------------------------------------------------------------------
