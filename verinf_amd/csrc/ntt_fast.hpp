@@ -154,7 +154,7 @@ inline bool pass_uniform(const PassArgs &A, int *n1_valid) {
     }
     const int lc = A.B + A.log_rho;
     if (A.pre || A.ndig < 1 || lc < lt || lt < A.log_rho || lt - A.log_rho > A.dig[0]) return false;
-    if (A.src_width != n) return false;
+    if (A.src_width != n || A.logn + A.log_rho > 28) return false;
     return (((i64)1 << A.log_rho) - 1) * A.src_coset_stride + n < ((i64)1 << 29);
 }
 
@@ -191,9 +191,42 @@ VI_HD TileU tile_uniform(const PassArgs &A, i64 tile) {
     return U;
 }
 
-// element `off` (a per-thread 32-bit element offset) of the run that starts at the uniform address `base`
-VI_HD const u64 *at32(const u64 *base, u32 off) { return (const u64 *)((const char *)base + (size_t)(u32)(off * 8u)); }
-VI_HD u64 *at32(u64 *base, u32 off) { return (u64 *)((char *)base + (size_t)(u32)(off * 8u)); }
+// A run of elements addressed as "uniform base + uniform element offset + per-thread element offset" (all three
+// below 2^29 elements).  On the device this is a raw buffer access: the base sits in a buffer resource in scalar
+// registers, the uniform offset in a scalar register and the thread offset in one vector register, so an access
+// costs no vector arithmetic at all and keeps no 64-bit address alive (global_load needs one register pair per
+// address, which the compiler hoists out of the coset loop).  On the host it is pointer arithmetic.
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __attribute__((__vector_size__(2 * sizeof(u32)))) u32 vi_u32x2;
+struct URun { __amdgpu_buffer_rsrc_t r; };
+__device__ __forceinline__ URun urun(const u64 *base) {
+    // raw buffer (stride 0), 4 GiB window, 32-bit data format
+    return URun{__builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)0xFFFFFFFFu, 0x00020000)};
+}
+__device__ __forceinline__ u64 uload(const URun &b, u32 uni, u32 off) {
+    const vi_u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(b.r, off * 8u, uni * 8u, 0);
+    return ((u64)v[1] << 32) | v[0];
+}
+__device__ __forceinline__ void ustore(const URun &b, u32 uni, u32 off, u64 x) {
+    const vi_u32x2 v = {(u32)x, (u32)(x >> 32)};
+    __builtin_amdgcn_raw_buffer_store_b64(v, b.r, off * 8u, uni * 8u, 0);
+}
+// not read again by this launch: non-temporal
+__device__ __forceinline__ void ustore_stream(const URun &b, u32 uni, u32 off, u64 x) {
+    const vi_u32x2 v = {(u32)x, (u32)(x >> 32)};
+#if defined(VI_PLAIN_STORES)
+    __builtin_amdgcn_raw_buffer_store_b64(v, b.r, off * 8u, uni * 8u, 0);
+#else
+    __builtin_amdgcn_raw_buffer_store_b64(v, b.r, off * 8u, uni * 8u, 2);
+#endif
+}
+#else
+struct URun { u64 *p; };
+inline URun urun(const u64 *base) { return URun{const_cast<u64 *>(base)}; }
+inline u64 uload(const URun &b, u32 uni, u32 off) { return b.p[(size_t)uni + off]; }
+inline void ustore(const URun &b, u32 uni, u32 off, u64 x) { b.p[(size_t)uni + off] = x; }
+inline void ustore_stream(const URun &b, u32 uni, u32 off, u64 x) { b.p[(size_t)uni + off] = x; }
+#endif
 
 // the per-thread part of the stage-1 source offset in a tile described by a TileU
 template <int A2>
@@ -229,8 +262,9 @@ VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &
         const u32 off = lane_src_off<A2>(A, U, c, n2);
         // an input past the source width reads input 0 instead (and is zeroed in fast_fix): the choice is the same
         // for every thread, so it is made on the scalar base
+        const URun src = urun(A.src + U.src_u);
 #pragma unroll
-        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = *at32(A.src + U.src_u + ((i64)(n1 < A.n1_valid ? n1 : 0) << U.sh1), off);
+        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = uload(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off);
         ok = A.n1_valid >= 16 ? 0xFFFFu : ((1u << A.n1_valid) - 1u);
         return;
     }
@@ -271,9 +305,9 @@ VI_HD void fast_pre_load(const PassArgs &A, i64 tile, int tid, int t_loop, u64 (
     if constexpr (UNI) {                                   // a strided pass: a final pass with pre-multipliers is never uniform
         const TileU U = tile_uniform<A2>(A, tile);
         const u32 off = lane_src_off<A2>(A, U, c, n2);
-        const u64 *pre = A.pre + ((i64)t_loop << A.logn) + U.pre_u;
+        const URun pre = urun(A.pre + ((i64)t_loop << A.logn) + U.pre_u);
 #pragma unroll
-        for (int n1 = 0; n1 < 16; ++n1) pw[n1] = *at32(pre + ((i64)n1 << U.sh1), off);
+        for (int n1 = 0; n1 < 16; ++n1) pw[n1] = uload(pre, (u32)n1 << U.sh1, off);
         return;
     }
     const ColRef R = col_ref(A, tile, c);
@@ -326,7 +360,8 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
     const int c = tid & ((1 << lt) - 1);
     if constexpr (UNI) {
         const TileU U = tile_uniform<A2>(A, tile);
-        u64 *dst = A.dst + U.dst_u + (A.is_final ? 0 : (i64)t_loop * A.dst_coset_stride);
+        const URun dst = urun(A.dst + U.dst_u + (A.is_final ? 0 : (i64)t_loop * A.dst_coset_stride));
+        const URun twr = urun(A.is_final ? A.dst : A.tw + U.tw_u);
 #pragma unroll
         for (int i = 0; i < 16 / E2; ++i) {
             const int k1 = (tid + i * NTHREADS) >> lt;
@@ -334,7 +369,7 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
             u64 x[E2], tw[E2];
             if (!A.is_final) {
 #pragma unroll
-                for (int k2 = 0; k2 < E2; ++k2) tw[k2] = *at32(A.tw + U.tw_u + ((i64)k2 << U.sh2), off);
+                for (int k2 = 0; k2 < E2; ++k2) tw[k2] = uload(twr, (u32)k2 << U.sh2, off);
             }
 #pragma unroll
             for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
@@ -346,7 +381,7 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
                 u64 v = x[k2];
                 if (!A.is_final) v = gl::mul(v, tw[k2]);
                 else if (A.scale != 1) v = gl::mul(v, A.scale);
-                VI_STREAM_STORE(at32(dst + ((i64)k2 << U.sh2), off), v);
+                ustore_stream(dst, (u32)k2 << U.sh2, off, v);
                 if ((k2 & 3) == 3) VI_SCHED_FENCE();
             }
         }
@@ -417,13 +452,13 @@ VI_HD void fused_stage2_inv(const PassArgs &A, i64 tile, int tid, const u64 *lds
         }
     }
     if (A.dst) {
-        u64 *dst = A.dst + U.dst_u;
+        const URun dst = urun(A.dst + U.dst_u);
 #pragma unroll
         for (int i = 0; i < 16 / E2; ++i) {
             const int k1 = (tid + i * NTHREADS) >> lt;
             const u32 off = (u32)c + ((u32)k1 << U.shk);
 #pragma unroll
-            for (int k2 = 0; k2 < E2; ++k2) *at32(dst + ((i64)k2 << U.sh2), off) = coef[i + (16 / E2) * k2];
+            for (int k2 = 0; k2 < E2; ++k2) ustore(dst, (u32)k2 << U.sh2, off, coef[i + (16 / E2) * k2]);
         }
     }
 }
@@ -438,13 +473,13 @@ VI_HD void fused_stage1_fwd(const PassArgs &A, i64 tile, int tid, int t, const u
     s1_coords<A2>(A, tid, c, n2);
     const TileU U = tile_uniform<A2>(A, tile);
     const u32 off = lane_src_off<A2>(A, U, c, n2);
-    const u64 *pre = A.pre + ((i64)t << A.logn) + U.pre_u;
+    const URun pre = urun(A.pre + ((i64)t << A.logn) + U.pre_u);
     u64 x[16];
 #pragma unroll
     for (int g = 0; g < 16; g += 4) {
         u64 pw[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) pw[j] = *at32(pre + ((i64)(g + j) << U.sh1), off);
+        for (int j = 0; j < 4; ++j) pw[j] = uload(pre, (u32)(g + j) << U.sh1, off);
 #pragma unroll
         for (int j = 0; j < 4; ++j) x[g + j] = gl::mul(coef[g + j], pw[j]);
         VI_SCHED_FENCE();
@@ -472,7 +507,8 @@ VI_HD void fused_stage2_fwd(const PassArgs &A, i64 tile, int tid, int t, const u
     const int st = (1 << lt) + 1;
     const int c = tid & ((1 << lt) - 1);
     const TileU U = tile_uniform<A2>(A, tile);
-    u64 *dst = A.dst + U.dst_u + (i64)t * A.dst_coset_stride;
+    const URun dst = urun(A.dst + U.dst_u + (i64)t * A.dst_coset_stride);
+    const URun twr = urun(A.tw + U.tw_u);
 #pragma unroll
     for (int i = 0; i < 16 / E2; ++i) {
         const int k1 = (tid + i * NTHREADS) >> lt;
@@ -487,9 +523,9 @@ VI_HD void fused_stage2_fwd(const PassArgs &A, i64 tile, int tid, int t, const u
         for (int g = 0; g < E2; g += G) {
             u64 tw[G];
 #pragma unroll
-            for (int j = 0; j < G; ++j) tw[j] = *at32(A.tw + U.tw_u + ((i64)(g + j) << U.sh2), off);
+            for (int j = 0; j < G; ++j) tw[j] = uload(twr, (u32)(g + j) << U.sh2, off);
 #pragma unroll
-            for (int j = 0; j < G; ++j) VI_STREAM_STORE(at32(dst + ((i64)(g + j) << U.sh2), off), gl::mul(x[g + j], tw[j]));
+            for (int j = 0; j < G; ++j) ustore_stream(dst, (u32)(g + j) << U.sh2, off, gl::mul(x[g + j], tw[j]));
             VI_SCHED_FENCE();
         }
     }
