@@ -96,6 +96,12 @@ def test_sum_of_products_shared_tables_and_coefficients(mods):
     ("first coefficient zero", 5, [(0, [0, 1, 2]), (5, [0, 3, 4]), (7, [0, 2])]),
     ("first coefficient one", 5, [(1, [0, 1, 2]), (5, [0, 3, 4]), (7, [0, 2]), (9, [0])]),
     ("first coefficient minus one", 5, [(P - 1, [0, 1, 2]), (5, [0, 3, 4]), (7, [0, 2]), (9, [0])]),
+    # the hadamard gate batch eq * a * b - eq * c (layergkr/relations.py:104-124) has its own unrolled kernel path:
+    # four distinct tables, one product of two and one linear term under a common factor, in any table order
+    ("hadamard gate", 4, [(3, [0, 1, 2]), (P - 5, [0, 3])]),
+    ("hadamard gate, unit coefficients", 4, [(1, [0, 1, 2]), (P - 1, [0, 3])]),
+    ("hadamard gate, other table order", 4, [(P - 5, [2, 1]), (7, [3, 1, 0])]),
+    ("hadamard gate, linear term first and zero", 4, [(0, [3, 2]), (9, [1, 3, 0])]),
     # more tables than a thread keeps in registers: the same forms with the factors read from memory
     ("many tables", 11, [(3, [0, 1, 2]), (P - 5, [0, 3]), (7, [0, 4, 5]), (11, [0, 6]), (13, [0, 7, 8]), (17, [0, 9]),
                          (19, [0, 10, 10]), (23, [0])]),

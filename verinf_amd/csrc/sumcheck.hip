@@ -53,6 +53,7 @@ struct Desc {
                                             // term's coefficient, or the first product term's coefficient of a
                                             // factored sum, whose other coefficients are divided by it
     int product;                            // one term whose factors are exactly the n_tables tables, once each
+    int gate;                               // four tables [common, f0, f1, lin]: common * (f0 * f1 + lin_coeff[0] * lin)
     int skip1;                              // S(1) is not summed: it is claim - S(0) (the round's known total)
     u64 claim;                              // S(0) + S(1) when skip1
 };
@@ -75,9 +76,12 @@ __device__ __forceinline__ u64 wave_sum(u64 v) {
 // three-factor benchmark instance): the term interpreter below -- scalar loads of the term
 // description and a register picked by index per factor -- gives way to a fully unrolled product.
 // NS: evaluation points the general path keeps per pair (4 when the degree is at most 3, else NSAMP)
-template <int NT, int MODE, int U, bool PROD, int NS>
+// SHAPE 2: the hadamard gate batch eq * (a * b + c' * c) (layergkr/relations.py:104-124: eq * a * b - eq * c with the
+// coefficients normalised on the host), tables ordered [eq, a, b, c] by the host: unrolled like the single product.
+template <int NT, int MODE, int U, int SHAPE, int NS>
 __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial, u64 *out,
                                                  u64 scale, int direct) {
+    constexpr bool PROD = SHAPE == 1, GATE = SHAPE == 2, FIXED = SHAPE != 0;
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const i64 count = (MODE == 2) ? (half >> 1) : half;
     const i64 stride = (i64)gridDim.x * BLOCK;
@@ -93,7 +97,7 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         if (i >= count) continue;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            if (PROD || t < D.n_tables) {
+            if (FIXED || t < D.n_tables) {
                 const u64 *f = D.src[t];
                 if (MODE == 0) {
                     // caller data: any 64-bit word is taken as its residue (the ladders below add canonical values)
@@ -122,7 +126,25 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         u64 cur[NT], dif[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-            if (PROD || t < D.n_tables) { cur[t] = lo[t]; dif[t] = gl::sub(hi[t], lo[t]); }
+            if (FIXED || t < D.n_tables) { cur[t] = lo[t]; dif[t] = gl::sub(hi[t], lo[t]); }
+        if constexpr (GATE) {
+            // S(x) = eq(x) * (a(x) b(x) + c'(x)), c' = lin_coeff * c carried as value and step
+            u64 lc = gl::mul(D.lin_coeff[0], cur[3]);
+            const u64 ld = gl::mul(D.lin_coeff[0], dif[3]);
+#pragma unroll
+            for (int x = 0; x <= 3; ++x) {
+                if (!(x == 1 && D.skip1)) {
+                    const u64 inner = gl::addc(gl::mul(cur[1], cur[2]), lc);
+                    acc[x] = gl::addc(acc[x], gl::mul(inner, cur[0]));
+                }
+                if (x < 3) {
+#pragma unroll
+                    for (int t = 0; t < 3; ++t) cur[t] = gl::addc(cur[t], dif[t]);
+                    lc = gl::addc(lc, ld);
+                }
+            }
+            continue;
+        }
         if (PROD) {
 #pragma unroll
             for (int x = 0; x <= NT; ++x) {
@@ -390,6 +412,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
     D.coeff_at_end = 0;
     D.out_scale = 1;
     D.product = 0;
+    D.gate = 0;
     D.skip1 = 0;
     D.claim = 0;
     if (!need_terms) return VI_OK;
@@ -417,6 +440,21 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         D.product = (seen == (1u << n_tables) - 1);
     }
     if (n_terms >= 2) factor_terms(D, term_off, factor_idx, n_terms);
+    // the hadamard gate batch: four distinct tables, common * (f0 * f1 + c * lin).  The tables are put in that order
+    // (sources and destinations together), so the kernel needs no indices.
+    if (n_terms >= 2 && n_tables == 4 && D.common >= 0 && D.n_terms == 1 && D.term_off[1] == 2 && D.n_lin == 1 &&
+        D.c0 == 0 && D.coeff[0] == 1) {
+        const int order[4] = {D.common, D.fidx[0], D.fidx[1], D.lin_idx[0]};
+        unsigned seen = 0;
+        for (int t = 0; t < 4; ++t) seen |= 1u << order[t];
+        if (seen == 0xFu) {
+            const u64 *s4[4];
+            u64 *d4[4];
+            for (int t = 0; t < 4; ++t) { s4[t] = D.src[order[t]]; d4[t] = D.dst[order[t]]; }
+            for (int t = 0; t < 4; ++t) { D.src[t] = s4[t]; D.dst[t] = d4[t]; }
+            D.gate = 1;
+        }
+    }
     return VI_OK;
 }
 
@@ -447,7 +485,7 @@ int resident_blocks(K kernel, int max_per_cu) {
     return nb > MAX_BLOCKS ? MAX_BLOCKS : nb;
 }
 
-template <int NT, int MODE, int U, bool PROD, int NS>
+template <int NT, int MODE, int U, int SHAPE, int NS>
 int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
     // per instantiation and device, looked up on first use there (devices of one process may differ)
     static std::mutex mu;
@@ -457,20 +495,22 @@ int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u6
     int cap;
     {
         std::lock_guard<std::mutex> lock(mu);
-        if (!caps[dev]) caps[dev] = resident_blocks(k_round<NT, MODE, U, PROD, NS>, MODE == 2 ? 5 : 64);
+        if (!caps[dev]) caps[dev] = resident_blocks(k_round<NT, MODE, U, SHAPE, NS>, MODE == 2 ? 5 : 64);
         cap = caps[dev];
     }
     if (nb > cap) nb = cap;
-    hipLaunchKernelGGL((k_round<NT, MODE, U, PROD, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    hipLaunchKernelGGL((k_round<NT, MODE, U, SHAPE, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
     return nb;
 }
 
 template <int NT, int MODE, int U>
 int launch_k(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
     if (MODE != 1 && NT <= 4 && D.product && D.n_tables == NT)
-        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4), NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
-    if (MODE != 1 && D.deg <= 3) return launch_kp<NT, MODE, U, false, (MODE != 1 ? 4 : NSAMP)>(D, half, r, partial, nb, out, scale, direct, s);
-    return launch_kp<NT, MODE, U, false, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
+        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4) ? 1 : 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
+    if (MODE != 1 && NT == 4 && D.gate && D.n_tables == 4)
+        return launch_kp<NT, MODE, U, (MODE != 1 && NT == 4) ? 2 : 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
+    if (MODE != 1 && D.deg <= 3) return launch_kp<NT, MODE, U, 0, (MODE != 1 ? 4 : NSAMP)>(D, half, r, partial, nb, out, scale, direct, s);
+    return launch_kp<NT, MODE, U, 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
 }
 
 template <int MODE, int U>
