@@ -97,7 +97,33 @@ int g_allow_fusion = 1;
 // runs passes[q] (and passes[q + 1] with it when the two fuse); returns how many passes it consumed
 int run_passes_at(const std::vector<PassArgs> &passes, size_t q);
 
+template <bool INV>
+void run_512(const PassArgs &A_in) {
+    PassArgs A = A_in;
+    A.is_final = 1;
+    i64 tiles = pass_tiles(A);
+    std::vector<u64> lds(fast_lds_words(A.a));
+    std::vector<u64> regs((size_t)NTHREADS * 16);
+    std::vector<u32> oks(NTHREADS);
+    for (i64 tile = 0; tile < tiles; ++tile) {
+        for (int tid = 0; tid < NTHREADS; ++tid)
+            fast_load<5, false>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
+        for (int tid = 0; tid < NTHREADS; ++tid) {
+            u64 pw[16] = {};
+            if (A.pre) fast_pre_load<5, false>(A, tile, tid, 0, pw);
+            fast_stage1<5, INV>(A, tile, tid, 0, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]), pw,
+                                A.twi, lds.data());
+        }
+        for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2_512<INV>(A, tile, tid, lds.data());
+    }
+}
+
 void run_pass(const PassArgs &A) {
+    if (g_use_fast && fast512_ok(A.a) && A.is_final && A.twi) {
+        if (A.inverse) run_512<true>(A);
+        else run_512<false>(A);
+        return;
+    }
     if (g_use_fast && fast_ok(A.a)) {
         switch ((A.a - FAST_A1) * 2 + (A.inverse ? 1 : 0)) {
             case 2: run_fast<1, false>(A); return;

@@ -102,6 +102,31 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
 }
 
 
+// 512-point rows: one pass, 16 x 32 (fast_stage2_512); eight rows (or row-coset pairs) per workgroup
+template <bool INV>
+__global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
+    PassArgs A = A_in;
+    A.is_final = 1;
+    constexpr int A2 = 5;
+    __shared__ u64 lds[TILE + (16 << A2)];
+    __shared__ u64 twi[16 << A2];
+    const int tid = threadIdx.x;
+    const i64 tile = blockIdx.x;
+    u64 tw_mine[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) tw_mine[i] = A.twi[tid + i * NTHREADS];
+    u64 reg[16], pw[16];
+    u32 ok;
+    if (A.pre) fast_pre_load<A2, false>(A, tile, tid, 0, pw);
+    fast_load<A2, false>(A, tile, tid, reg, ok);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) twi[tid + i * NTHREADS] = tw_mine[i];
+    __syncthreads();
+    fast_stage1<A2, INV>(A, tile, tid, 0, ok, reg, pw, twi, lds);
+    __syncthreads();
+    fast_stage2_512<INV>(A, tile, tid, lds);
+}
+
 // The last inverse pass and the first forward pass of a coset extension in one launch (fused_stage2_inv): the
 // coefficients stay in registers between the two, so they are neither written to nor read back from HBM (unless the
 // caller wants them), and the rho cosets are expanded by a loop inside the workgroup.
@@ -321,6 +346,9 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
         if (fast_ok(A.a) && A.twi) {
             if (!A.is_final && A.loop_cosets) grid.x <<= A.log_rho;       // tiles * rho <= 2^31 by max_rows_per_launch
             launch_fast(A, grid, block, s);
+        } else if (fast512_ok(A.a) && A.twi && A.is_final) {
+            if (A.inverse) hipLaunchKernelGGL(k_ntt_512<true>, grid, block, 0, s, A);
+            else hipLaunchKernelGGL(k_ntt_512<false>, grid, block, 0, s, A);
         } else {
             hipLaunchKernelGGL(k_ntt_pass, grid, block, 0, s, A);
         }

@@ -77,6 +77,7 @@ VI_HD void dft_reg(u64 (&x)[1 << A]) {
 constexpr int FAST_A1 = 4;
 constexpr int FAST_E1 = 16;
 VI_HD bool fast_ok(int a) { return a >= 5 && a <= 8; }
+VI_HD bool fast512_ok(int a) { return a == 9; }                  // 512 = 16 x 32: single-pass transforms only (fast_stage2_512)
 VI_HD int fast_lds_words(int a) { return TILE + (1 << a); }      // (L rows) x (T + 1)
 
 // per-thread description of the one column it serves in a stage
@@ -421,6 +422,49 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
     }
 }
 
+
+// Stage 2 of a 512-point single pass (16 x 32): the 32-point transforms over n2.  Two threads share one
+// transform, decimated in frequency: both read its 32 values, thread h = 0 forms the sixteen sums
+// x[j] + x[j + 16] and gets the even outputs from a 16-point transform, thread h = 1 forms the differences times
+// w_32^j (shifts) and gets the odd outputs -- no exchange between the two.  h is the top bit of the thread id, so a
+// wavefront is all sums or all differences.  Per-element addressing (a single pass is never a uniform pass).
+template <bool INV>
+VI_HD void fast_stage2_512(const PassArgs &A, i64 tile, int tid, const u64 *lds) {
+    constexpr int A2 = 5;
+    const int lt = logT(A);                                // 3: eight columns per tile
+    const int st = (1 << lt) + 1;
+    const int c = tid & ((1 << lt) - 1);
+    const int k1 = (tid >> lt) & 15, h = tid >> (lt + 4);
+    const ColRef R = col_ref(A, tile, c);
+    const int lc = A.B + A.log_rho;
+    u64 x[32], y[16];
+#pragma unroll
+    for (int n2 = 0; n2 < 32; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
+    if (h == 0) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) y[j] = gl::addc(x[j], x[j + 16]);
+    } else {
+        static_for<0, 16>([&](auto j_) {
+            constexpr int j = decltype(j_)::value;
+            constexpr int e = level_exp<5, INV>(4, j);         // w_32^j = 2^e
+            const u64 d = gl::sub(x[j], x[j + 16]);
+            if constexpr (e == 0) y[j] = d;
+            else if constexpr (e < 96) y[j] = gl::mul_pow2c<e>(d);
+            else y[j] = gl::neg(gl::mul_pow2c<e - 96>(d));
+        });
+    }
+    VI_SCHED_FENCE();
+    dft_reg<4, INV>(y);
+    VI_SCHED_FENCE();
+    if (!R.valid) return;
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+        const i64 k = k1 + 16 * (2 * m + h);
+        u64 v = y[m];
+        if (A.scale != 1) v = gl::mul(v, A.scale);
+        VI_STREAM_STORE(&A.dst[R.dst_base + (k << lc)], v);
+    }
+}
 
 // The last inverse pass and the first forward pass of a coset extension share their tiles when K = L * L: the last
 // inverse pass leaves, in the thread that ran the stage-2 transforms (column c, outputs k1 = q + E2 i, i < 16 / E2),

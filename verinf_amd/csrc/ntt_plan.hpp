@@ -36,7 +36,7 @@ struct HostTables {
     int logn, inverse;
     Split sp;
     std::vector<u64> tw[3];     // one per non-final pass: [(k << logR) + r] = w_M^(k r) (pass 0 also carries 1/n on the inverse)
-    std::vector<u64> twi[4];    // per pass with a digit of 2^5..2^8: w_L^(n2 k1) at [n2 * 16 + k1]
+    std::vector<u64> twi[4];    // per pass with a digit of 2^5..2^9: w_L^(n2 k1) at [n2 * 16 + k1]
     u64 scale;                  // 1/n when inverse and single pass, else 1
 };
 
@@ -66,7 +66,7 @@ inline HostTables make_tables(int logn, int inv) {
     }
     for (int q = 0; q < H.sp.p; ++q) {
         int a = H.sp.a[q];
-        if (!fast_ok(a)) continue;
+        if (!fast_ok(a) && !fast512_ok(a)) continue;
         u64 w = root_of_unity(a);
         if (inv) w = inverse(w);
         std::vector<u64> &t = H.twi[q];
