@@ -28,14 +28,17 @@ P = (1 << 64) - (1 << 32) + 1
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 
-# HBM bytes of one step of the default LDE leg (all k_ntt_fast launches of the step together): FETCH_SIZE and
-# WRITE_SIZE read by rocprofv3 in two counter runs of this script (3.80 GB read + 5.77 GB written per step),
-# each scaled by what the same counter reads for a 1 GiB device copy.  roofline.traffic is this figure divided
-# by the launches of a step, like roofline.achieved.
-LDE_TRAFFIC_BYTES_PER_STEP = 9.14e9
-# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU: per 512-row chunk 433.7 M + 285.7 M in the
-# two forward launches and 92.8 M + 71.3 M in the two inverse ones) and the rate at which 1024 SIMDs issue them at 2.4 GHz, one per four cycles
-LDE_VALU_INSTS_PER_STEP = 2 * (433_717_248 + 285_736_960 + 92_766_208 + 71_335_936)
+# HBM bytes of one step of the default LDE leg (its six launches together: per 512-row chunk the strided inverse
+# pass, the fused last-inverse / first-forward launch k_lde_mid, and the final forward pass): FETCH_SIZE and
+# WRITE_SIZE read by rocprofv3 in two counter runs of this script, each scaled by what the same counter reads for a
+# 1 GiB device copy (x 2.000 / x 1.000): 3.23 GB read + 4.83 GB written per step
+# (profiles/k_lde_mid_k_ntt_fast__coset_lde_1024x2p16_to_2p18.md).  roofline.traffic is this figure divided by the
+# launches of a step, like roofline.achieved.
+LDE_TRAFFIC_BYTES_PER_STEP = 8.06e9
+# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU, same profile: per 512-row chunk 58.6 M in
+# the strided inverse launch, 296.8 M in k_lde_mid and 187.6 M in the final forward launch) and the rate at which
+# 1024 SIMDs issue them at 2.4 GHz, one per four cycles
+LDE_VALU_INSTS_PER_STEP = 2 * (58_621_952 + 296_779_776 + 187_564_032)
 VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / 4
 
 
@@ -555,7 +558,7 @@ def main():
                      "frac": lde["achieved_gbs"] / HBM_PEAK_GBS, "traffic": LDE_TRAFFIC_BYTES_PER_STEP / lde["launches_per_step"],
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a copy probe "
                                        "(x2.000 / x1.000); not re-measured in this run",
-                     "kernel": "k_ntt_fast", "launches_per_step": lde["launches_per_step"],
+                     "kernel": "k_lde_mid + k_ntt_fast (the three launches of a row chunk)", "launches_per_step": lde["launches_per_step"],
                      "avg_launch_us": lde["kernel_avg_us"],
                      "algorithmic_bytes_per_launch": lde["alg_bytes_per_launch"],
                      # the same launches against the integer-VALU issue rate, which is what bounds this kernel

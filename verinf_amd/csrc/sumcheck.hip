@@ -138,8 +138,9 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
                     acc[x] = gl::addc(acc[x], gl::mul(inner, cur[0]));
                 }
                 if (x < 3) {
+                    // f(1) is the loaded upper value itself: the first step of the ladder costs nothing
 #pragma unroll
-                    for (int t = 0; t < 3; ++t) cur[t] = gl::addc(cur[t], dif[t]);
+                    for (int t = 0; t < 3; ++t) cur[t] = (x == 0) ? hi[t] : gl::addc(cur[t], dif[t]);
                     lc = gl::addc(lc, ld);
                 }
             }
@@ -155,8 +156,9 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
                     acc[x] = gl::addc(acc[x], NT == 1 ? gl::canon(prod) : prod);
                 }
                 if (x < NT) {
+                    // f(1) is the loaded upper value itself: the first step of the ladder costs nothing
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) cur[t] = gl::addc(cur[t], dif[t]);
+                    for (int t = 0; t < NT; ++t) cur[t] = (x == 0) ? hi[t] : gl::addc(cur[t], dif[t]);
                 }
             }
             continue;
