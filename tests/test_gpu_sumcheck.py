@@ -154,6 +154,24 @@ def test_tables_with_words_at_or_above_p_are_taken_as_residues(mods, v, nt, term
     assert [[y for _, y in s] for s in polys] == want_samples
 
 
+def test_tables_that_are_views_at_an_odd_word_offset(mods):
+    """The evaluation round loads two adjacent words per access when every table is 16-byte aligned; a table that
+    starts at an odd word (a slice of a larger tensor) must take the other path and give the same proof."""
+    gpu, _ = mods
+    v = 13
+    tabs = [rand_field(1 << v, 700 + j) for j in range(3)]
+    coins, coin = _coins(v, 31)
+    want_claim, want_samples, _ = O.sumcheck_prove(tabs, [(1, [0, 1, 2])], coins)
+    for shifted in ((1, 0, 0), (0, 1, 1), (1, 1, 1), (0, 0, 0)):
+        objs = []
+        for t, sh in zip(tabs, shifted):
+            buf = to_dev(np.concatenate([np.zeros(sh, dtype=np.uint64), t]))
+            objs.append(buf[sh:])
+            assert objs[-1].data_ptr() % 16 == (8 if sh else 0)
+        claim, polys, _, _ = gpu.prove_terms_gpu([(1, objs)], coin, P)
+        assert claim == want_claim and [[y for _, y in s] for s in polys] == want_samples, shifted
+
+
 def test_large_instance_matches_oracle(mods):
     """2^22 x 3 factors, degree 3, 22 rounds: every round's samples against the C oracle."""
     gpu, _ = mods

@@ -89,12 +89,28 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
 #pragma unroll
     for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
 
-    for (i64 i0 = (i64)blockIdx.x * BLOCK + threadIdx.x; i0 < count; i0 += stride * U) {
+    // U = 2 (evaluation-only rounds): a thread takes the adjacent indices 2j, 2j + 1 and loads each table's two
+    // lower and two upper words as one 16-byte access each (the host selects it only for even counts and 16-byte
+    // aligned tables)
+    const i64 trips = (U == 2) ? (count >> 1) : count;
+    for (i64 i0 = (i64)blockIdx.x * BLOCK + threadIdx.x; i0 < trips; i0 += stride) {
       u64 lo_u[U][NT], hi_u[U][NT];
+      if constexpr (U == 2) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const i64 i = i0 + u * stride;
-        if (i >= count) continue;
+        for (int t = 0; t < NT; ++t) {
+            if (FIXED || t < D.n_tables) {
+                const ulonglong2 lo2 = *reinterpret_cast<const ulonglong2 *>(D.src[t] + 2 * i0);
+                const ulonglong2 hi2 = *reinterpret_cast<const ulonglong2 *>(D.src[t] + half + 2 * i0);
+                lo_u[0][t] = gl::canon(lo2.x);
+                lo_u[U - 1][t] = gl::canon(lo2.y);
+                hi_u[0][t] = gl::canon(hi2.x);
+                hi_u[U - 1][t] = gl::canon(hi2.y);
+            }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < (U == 2 ? 0 : U); ++u) {
+        const i64 i = i0;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             if (FIXED || t < D.n_tables) {
@@ -119,7 +135,6 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
       if (MODE == 1) continue;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (i0 + u * stride >= count) continue;
         u64 (&lo)[NT] = lo_u[u];
         u64 (&hi)[NT] = hi_u[u];
         // f(x) for x = 0, 1, 2, ... by repeated addition of (hi - lo)
@@ -531,7 +546,11 @@ template <int MODE>
 int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
                  hipStream_t s) {
     // two indices in flight for the load-light evaluation round on few tables
-    if (MODE == 0 && D.n_tables <= 4 && nb > 1) return launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, s);
+    if (MODE == 0 && D.n_tables <= 4 && nb > 1 && (half & 1) == 0) {
+        bool aligned = true;
+        for (int t = 0; t < D.n_tables; ++t) aligned = aligned && ((uintptr_t)D.src[t] & 15) == 0;
+        if (aligned) return launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, s);
+    }
     return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, s);
 }
 
