@@ -360,6 +360,19 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
 // rows per launch so that grids stay below 2^31 tiles
 i64 max_rows_per_launch(int logn) { return ((i64)1 << 40) >> logn; }
 
+// rows per chunk of a coset extension: within the grid limit, and small enough that the coset planes of the forward
+// intermediate stay inside the 2^29-element window the final pass's scalar-base addressing covers (a larger chunk
+// would still be correct, on the per-element path)
+i64 max_lde_chunk(int logK, int logN) {
+    i64 cap = max_rows_per_launch(logN);
+    const i64 K = (i64)1 << logK, rho = (i64)1 << (logN - logK);
+    if (rho > 1 && logK <= 26) {
+        const i64 fit = (((i64)1 << 29) - K - 1) / ((rho - 1) * K);
+        if (fit >= 8 && fit < cap) cap = fit;
+    }
+    return cap;
+}
+
 }  // namespace
 
 extern "C" {
@@ -422,7 +435,7 @@ int64_t vi_coset_lde_launches(int64_t m, int64_t K, int64_t N, size_t ws_bytes) 
     if (!one || m <= 0 || ws_bytes < one) return 0;
     i64 chunk = (i64)(ws_bytes / one);
     if (chunk > m) chunk = m;
-    if (chunk > max_rows_per_launch(vi::ilog2(N))) chunk = max_rows_per_launch(vi::ilog2(N));
+    if (chunk > max_lde_chunk(vi::ilog2(K), vi::ilog2(N))) chunk = max_lde_chunk(vi::ilog2(K), vi::ilog2(N));
     const i64 n_chunks = (m + chunk - 1) / chunk;         // balancing keeps the chunk count
     chunk = (m + n_chunks - 1) / n_chunks;
     // the pass list of one chunk, planned with placeholder addresses (only their being null or not matters)
@@ -487,7 +500,7 @@ int coset_lde_impl(const char *who, const uint64_t *in, int64_t m, int64_t width
     if (!ws || chunk < 1)
         return vi::fail(VI_ENOMEM, "%s: workspace of %zu bytes is below the one-row minimum %zu", who, ws_bytes, one);
     if (chunk > m) chunk = m;
-    if (chunk > max_rows_per_launch(logN)) chunk = max_rows_per_launch(logN);
+    if (chunk > max_lde_chunk(logK, logN)) chunk = max_lde_chunk(logK, logN);
     chunk = (m + ((m + chunk - 1) / chunk) - 1) / ((m + chunk - 1) / chunk);   // same chunk count, even sizes
     const Tables *Ti = nullptr, *Tf = nullptr;
     const u64 *pre = nullptr;

@@ -420,6 +420,9 @@ def lagrange_gpu(cfg: Config):
     cached per geometry.  The two domains go up as vectors; the ELL * N_LIG differences are inverted on the device
     with one batched inversion, so no entry is computed on the host."""
     _require_gpu()
+    if cfg.ELL * cfg.N_LIG > (1 << 27):
+        raise RuntimeError(f"lagrange_gpu: the dense {cfg.ELL} x {cfg.N_LIG} matrix would take "
+                           f"{cfg.ELL * cfg.N_LIG * 8 / 2**30:.0f} GiB; use encode_batch_ntt at this geometry")
     key = (cfg.ELL, cfg.K_DEG, cfg.N_LIG, torch.cuda.current_device())
     if key not in _LAGRANGE_GPU:
         k_inv = pow(cfg.K_DEG, P - 2, P)
