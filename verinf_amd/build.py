@@ -21,9 +21,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Wall", "-Wno-unused-function"]
 
 
-def build(verbose: bool = False, out: str = LIB, extra_flags=()) -> str:
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + list(extra_flags) + ["-shared", "-o", out] + [os.path.join(CSRC, s) for s in SOURCES]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -31,6 +29,22 @@ def build(verbose: bool = False, out: str = LIB, extra_flags=()) -> str:
     log = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + log)
+    return log
+
+
+def build(verbose: bool = False, out: str = LIB, extra_flags=()) -> str:
+    """Compile every translation unit (in parallel, one hipcc each) and link the shared library."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    jobs = max(1, min(len(SOURCES), int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
+    with tempfile.TemporaryDirectory(prefix="verinf_build_") as tmp:
+        objs = [os.path.join(tmp, s.replace(".hip", ".o")) for s in SOURCES]
+        cmds = [[hipcc] + FLAGS + list(extra_flags) + ["-c", "-o", o, os.path.join(CSRC, s)] for s, o in zip(SOURCES, objs)]
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            logs = list(pool.map(lambda c: _run(c, verbose), cmds))
+        logs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs, verbose))
+    log = "\n".join(l for l in logs if l.strip())
     if log.strip():
         print(log)                      # compiler warnings
     return out
