@@ -61,7 +61,8 @@ int main() {
         {8, 10, 16, 1, 1},   {9, 11, 9, 300, 512}, {10, 12, 5, 1024, 1024}, {10, 12, 4, 513, 600}, {10, 10, 3, 1000, 1024},
         {12, 14, 3, 4096, 4096}, {12, 14, 2, 2048, 4096}, {12, 15, 1, 4095, 4095}, {13, 15, 2, 8192, 8200},
         {14, 16, 2, 8192, 16384}, {14, 16, 1, 16384, 16384}, {16, 18, 1, 65536, 65536}, {16, 17, 1, 40000, 40000},
-        {16, 16, 1, 65536, 65536}, {8, 10, 0, 256, 256},
+        {16, 16, 1, 65536, 65536}, {8, 10, 0, 256, 256}, {12, 14, 2, 5, 8}, {14, 16, 2, 100, 128}, {14, 16, 2, 2816, 2816},
+        {16, 18, 1, 4097, 4100}, {16, 18, 1, 4095, 4095}, {12, 14, 3, 257, 257},
     };
     // per-element addressing, scalar-base addressing where it applies, and the fused middle launch of the LDE
     for (int mode = 0; mode < 3; ++mode) {

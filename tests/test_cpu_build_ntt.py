@@ -112,7 +112,8 @@ def test_ntt_25_bit_split_is_well_formed(emu):
 @pytest.mark.parametrize("logK,logN,m,w", [(5, 6, 4, 16), (7, 8, 9, 64), (9, 10, 3, 256), (3, 5, 700, 8),
                                            (12, 14, 2, 4096), (13, 15, 2, 5000), (14, 16, 1, 8192),
                                            (16, 18, 1, 65536), (10, 10, 3, 1000), (4, 7, 5, 11),
-                                           (10, 12, 5, 1024), (11, 13, 3, 2000), (11, 12, 2, 2048)])
+                                           (10, 12, 5, 1024), (11, 13, 3, 2000), (11, 12, 2, 2048),
+                                           (14, 16, 2, 2816), (12, 14, 3, 257), (16, 18, 1, 4097), (12, 14, 2, 63)])
 def test_lde_passes_match_oracle(emu, logK, logN, m, w):
     msgs = _rand((m, w), 200 + logK)
     want = O.coset_lde_rows(msgs, 1 << logK, 1 << logN, 7)

@@ -147,9 +147,13 @@ inline bool pass_uniform(const PassArgs &A, int *n1_valid) {
         const int lc = A.B + A.logR;
         if (lc < lt || A.logR < lt) return false;
         if (A.src_width == n) return true;
-        // a narrower source: only on the first pass (B = 0, so the index of input n1 is below (n1 + 1) << sh1)
+        // a narrower source: only on the first pass (B = 0, so input n1 of a thread has the index
+        // (n1 << sh1) + its 32-bit thread offset).  The first n1_valid inputs exist for every thread, input n1_valid for
+        // the threads whose index inside that plane is below the remainder of the width (src_width mod 2^sh1), the others for none.
         const int sh1 = a2 + A.logR;
-        if (A.B != 0 || A.src_width < 1 || (A.src_width & (((i64)1 << sh1) - 1)) != 0) return false;
+        // (at least the first plane whole, so that word 0 of a tile always exists for the loads that stand in for
+        // missing inputs)
+        if (A.B != 0 || (A.src_width >> sh1) < 1) return false;
         *n1_valid = (int)(A.src_width >> sh1);
         return true;
     }
@@ -267,6 +271,15 @@ VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &
 #pragma unroll
         for (int n1 = 0; n1 < 16; ++n1) reg[n1] = uload(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off);
         ok = A.n1_valid >= 16 ? 0xFFFFu : ((1u << A.n1_valid) - 1u);
+        if (A.n1_valid < 16) {
+            // the plane the width ends in: this thread's input there exists if its offset is below the remainder
+            const u32 rem = (u32)(A.src_width - ((i64)A.n1_valid << U.sh1));
+            const bool mine = (u32)U.pre_u + off < rem;           // pre_u: index of the tile's first column inside the row
+            const u64 v = uload(src, 0u, mine ? off + ((u32)A.n1_valid << U.sh1) : 0u);     // the others read word 0 of the tile
+#pragma unroll
+            for (int n1 = 0; n1 < 16; ++n1) reg[n1] = (n1 == A.n1_valid) ? v : reg[n1];
+            ok |= mine ? (1u << A.n1_valid) : 0u;
+        }
         return;
     }
     const ColRef R = col_ref(A, tile, c);
