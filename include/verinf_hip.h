@@ -53,6 +53,13 @@ int vi_gl_binop_bcast(int op, const uint64_t *a, const uint64_t *b, int64_t peri
  * op 0: out = -a;  op 1: out = a^arg;  op 2: out = a^(p-2) (arg ignored). */
 int vi_gl_unop(int op, const uint64_t *a, uint64_t arg, uint64_t *out, int64_t n, void *stream);
 
+/* Test hook (no counterpart in the reference): one device field primitive of the transform and sumcheck kernels
+ * applied elementwise, so that the test-suite can drive it with chosen operands.
+ * op 0: modular add of canonical a, b;  1: a - b;  2 / 3: sum / difference of the butterfly (a, b);
+ * 4: a mod p of any word;  5: a * b of any words;  6: (hi = b, lo = a) mod p;
+ * 100 + e, 0 <= e < 96: canonical a times 2^e (the compile-time shift twiddle). */
+int vi_gl_probe(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream);
+
 /* Replaces gl_axpy (cuda_primitives.py:282-288, 1104-1106; gl_extras.cuh:33-41):
  * y[i] += alpha * x[i], in place. */
 int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *stream);

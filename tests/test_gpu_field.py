@@ -135,3 +135,42 @@ def test_inverse_of_arrays_with_zeros_and_ragged_lengths(cp, n):
     red = to_dev(a % np.uint64(P))
     prod = to_np(cp.gl_mul(red, to_dev(got)))
     assert np.array_equal(prod, (to_np(red) != 0).astype(np.uint64))
+
+
+def test_device_field_primitives_one_by_one():
+    """The hand-scheduled sequences the transform and sumcheck kernels are built from (modular add, sub, the
+    interleaved butterfly, canonicalisation, the product, the 128-bit reduction and all 95 compile-time shift
+    twiddles), each on operands chosen around every carry they test: 0, 1, p - 1, p - 2, 2^32 +- 1, 2^63, words whose
+    halves are all ones, and random words, in all pairs; against Python integers."""
+    from verinf_amd import _lib
+    L = _lib.lib()
+    r = random.Random(77)
+    edge = [0, 1, 2, P - 1, P - 2, P - 3, (1 << 32) - 1, 1 << 32, (1 << 32) + 1, (1 << 63), (1 << 63) - 1,
+            0xFFFFFFFF00000000, 0xFFFFFFFEFFFFFFFF, 0x00000001FFFFFFFF, 0x0000000100000000, 0xFFFFFFFE00000001,
+            0xFFFFFFFE00000002, 0x8000000080000000, 0x7FFFFFFF7FFFFFFF]
+    edge += [(1 << s) % P for s in range(64)] + [((1 << s) - 1) % P for s in range(1, 64)]
+    canon = [x % P for x in edge] + [r.randrange(P) for _ in range(200)]
+    anyw = canon + [P, P + 1, (1 << 64) - 1, (1 << 64) - 2, P + (1 << 31)] + [r.randrange(1 << 64) for _ in range(100)]
+
+    def run(op, xs, ys):
+        a = to_dev(np.array(xs, dtype=np.uint64))
+        b = to_dev(np.array(ys, dtype=np.uint64))
+        out = torch.empty_like(a)
+        _lib.check(L.vi_gl_probe(op, a.data_ptr(), b.data_ptr(), out.data_ptr(), a.numel(), _lib.stream_ptr()))
+        return [int(v) for v in to_np(out)]
+
+    xs = [x for x in canon for _ in canon]
+    ys = [y for _ in canon for y in canon]
+    assert run(0, xs, ys) == [(x + y) % P for x, y in zip(xs, ys)]
+    assert run(1, xs, ys) == [(x - y) % P for x, y in zip(xs, ys)]
+    assert run(2, xs, ys) == [(x + y) % P for x, y in zip(xs, ys)]
+    assert run(3, xs, ys) == [(x - y) % P for x, y in zip(xs, ys)]
+    xa = [x for x in anyw for _ in anyw]
+    ya = [y for _ in anyw for y in anyw]
+    assert run(5, xa, ya) == [x * y % P for x, y in zip(xa, ya)]
+    assert run(6, xa, ya) == [((y << 64) + x) % P for x, y in zip(xa, ya)]
+    assert run(4, anyw, anyw) == [x % P for x in anyw]
+    for e in range(96):
+        assert run(100 + e, canon, canon) == [(x << e) % P for x in canon], e
+    with pytest.raises(RuntimeError):
+        _lib.check(L.vi_gl_probe(7, 0, 0, 0, 1, None))

@@ -18,7 +18,7 @@ LIB_PATH = os.environ.get("VERINF_HIP_LIB") or os.path.join(_HERE, "libverinf_hi
 
 EXPORTS = [
     "vi_last_error", "vi_version",
-    "vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy",
+    "vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_probe",
     "vi_gl_sum_workspace_bytes", "vi_gl_sum",
     "vi_gl_matmul_workspace_bytes", "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
     "vi_ntt_workspace_bytes", "vi_ntt_batched",
@@ -61,6 +61,7 @@ def lib():
     L.vi_gl_binop_bcast.argtypes = [c_int, vp, vp, i64, vp, i64, vp]
     L.vi_gl_unop.argtypes = [c_int, vp, u64, vp, i64, vp]
     L.vi_gl_axpy.argtypes = [vp, u64, vp, i64, vp]
+    L.vi_gl_probe.argtypes = [c_int, vp, vp, vp, i64, vp]
     L.vi_gl_sum_workspace_bytes.restype = sz
     L.vi_gl_sum_workspace_bytes.argtypes = [i64]
     L.vi_gl_sum.argtypes = [vp, i64, vp, vp, sz, vp]
@@ -111,7 +112,7 @@ def lib():
     L.vi_mle_eval.argtypes = [vp, i64, i64, POINTER(u64), c_int, vp, vp, sz, vp]
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
-    for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_sum",
+    for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_probe", "vi_gl_sum",
                  "vi_gl_matmul", "vi_gl_matvec", "vi_poly_eval",
                  "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_kquant_to_field_transposed", "vi_sumcheck_eval", "vi_sumcheck_eval_static",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",

@@ -54,6 +54,35 @@ __global__ __launch_bounds__(BLOCK) void k_unop(int op, const u64 *a, u64 arg, u
     }
 }
 
+// One device field primitive applied elementwise, for the test-suite: the transforms use these through fully
+// unrolled code with compile-time exponents, so this is the only place they can be driven with chosen operands.
+template <int E>
+__device__ __forceinline__ u64 shift_by(u64 v, int e) {
+    if constexpr (E >= 96) return 0;
+    else {
+        if (e == E) return gl::mul_pow2c<E>(v);
+        return shift_by<E + 1>(v, e);
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void k_probe(int op, const u64 *a, const u64 *b, u64 *out, i64 n) {
+    i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) {
+        const u64 x = a[i], y = b ? b[i] : 0;
+        u64 s, d, r;
+        gl::bfly(x, y, s, d);
+        if (op == 0) r = gl::addc(x, y);
+        else if (op == 1) r = gl::sub(x, y);
+        else if (op == 2) r = s;
+        else if (op == 3) r = d;
+        else if (op == 4) r = gl::canon(x);
+        else if (op == 5) r = gl::mul(x, y);
+        else if (op == 6) r = gl::reduce128(x, y);
+        else r = shift_by<0>(x, op - 100);
+        out[i] = r;
+    }
+}
+
 // Inverses of a whole array by Montgomery's trick in registers (the batching of
 // layergkr/field.py:84-101 at the scale of one thread): a thread takes INV_E elements, one
 // from each of INV_E equal slabs of the array so that a wavefront's accesses stay contiguous,
@@ -211,6 +240,18 @@ int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *
     if (!y || !x) return vi::fail(VI_EINVAL, "vi_gl_axpy: null pointer");
     hipLaunchKernelGGL(k_axpy, dim3(grid_for(n)), dim3(BLOCK), 0, (hipStream_t)stream, y, (u64)alpha, x, (i64)n);
     VI_LAUNCH_CHECK("k_axpy");
+    return VI_OK;
+}
+
+int vi_gl_probe(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream) {
+    const bool shift = op >= 100 && op < 196;
+    if (!shift && (op < 0 || op > 6)) return vi::fail(VI_EINVAL, "vi_gl_probe: op = %d", op);
+    if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_probe: n = %lld", (long long)n);
+    if (n == 0) return VI_OK;
+    const bool needs_b = !shift && op != 4;
+    if (!a || !out || (needs_b && !b)) return vi::fail(VI_EINVAL, "vi_gl_probe: null pointer");
+    hipLaunchKernelGGL(k_probe, dim3(grid_for(n)), dim3(BLOCK), 0, (hipStream_t)stream, op, a, needs_b ? b : nullptr, out, (i64)n);
+    VI_LAUNCH_CHECK("k_probe");
     return VI_OK;
 }
 
