@@ -202,10 +202,14 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
  * and returns 0, or non-zero to abort (the call then returns VI_EINVAL).
  *   tables        n_tables device tables of `size` = 2^v words (left untouched)
  *   work          n_tables device buffers of size/2 words (the folded tables live here)
- *   host_samples  >= 8 words of PINNED host memory the kernels write each round's samples to
+ *   host_samples  VI_SC_HOST_WORDS (16) words of PINNED host memory (hipHostMalloc): words 0..7 receive each
+ *                 round's samples and word 8 the count of rounds that have arrived; the host thread waits
+ *                 on that word (and queries the stream from time to time) rather than synchronising the stream
+ *                 every round.  One buffer per proof in flight.
  *   out_samples   host, v * (deg+1) words: S_round(x) for x = 0..deg (no mask applied)
  *   out_challenges host, v words: the challenges, reduced mod p
  * The final fold (after the last round) is not performed, as nothing reads it. */
+#define VI_SC_HOST_WORDS 16
 typedef int (*vi_coin_fn)(int round, const uint64_t *samples, int n_samples, uint64_t *challenge, void *user);
 int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
                       const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,

@@ -18,6 +18,7 @@
 //
 // Variable order is most-significant first, pairs are (i, half + i)
 // (layergkr/sumcheck.py:51-54).
+#include <atomic>
 #include <mutex>
 
 #include "common.hpp"
@@ -72,6 +73,8 @@ __device__ __forceinline__ u64 wave_sum(u64 v) {
 // loads per table and index, so two indices are kept in flight to cover HBM latency.
 // `direct`: a single-workgroup launch writes the finished samples itself (small rounds
 // need no second launch).
+// `flag`: when non-zero (and direct), out[NSAMP] = flag is stored after the samples have reached system scope, so a
+// host that owns `out` as pinned memory can wait on that word instead of on the stream.
 // PROD: the sum is a single product of all NT tables (a matmul contraction, eq * a * b, the
 // three-factor benchmark instance): the term interpreter below -- scalar loads of the term
 // description and a register picked by index per factor -- gives way to a fully unrolled product.
@@ -80,7 +83,7 @@ __device__ __forceinline__ u64 wave_sum(u64 v) {
 // coefficients normalised on the host), tables ordered [eq, a, b, c] by the host: unrolled like the single product.
 template <int NT, int MODE, int U, int SHAPE, int NS>
 __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, u64 *partial, u64 *out,
-                                                 u64 scale, int direct) {
+                                                 u64 scale, int direct, u64 flag) {
     constexpr bool PROD = SHAPE == 1, GATE = SHAPE == 2, FIXED = SHAPE != 0;
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const i64 count = (MODE == 2) ? (half >> 1) : half;
@@ -253,19 +256,32 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
         if (lane == 0) red[w][x] = v;
     }
     __syncthreads();
-    if (threadIdx.x < NSAMP) {
-        u64 v = red[0][threadIdx.x];
-        for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
-        if (direct) {
-            if (D.skip1 && threadIdx.x == 1) {           // S(1) = claim - S(0)
-                u64 s0 = red[0][0];
-                for (int i = 1; i < BLOCK / 64; ++i) s0 = gl::add(s0, red[i][0]);
-                out[1] = gl::sub(D.claim, scale == 1 ? s0 : gl::mul(s0, scale));
-            } else if ((int)threadIdx.x <= D.deg) {
-                out[threadIdx.x] = scale == 1 ? v : gl::mul(v, scale);
-            }
-        } else {
+    if (!direct) {
+        if (threadIdx.x < NSAMP) {
+            u64 v = red[0][threadIdx.x];
+            for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
             partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
+        }
+        return;
+    }
+    // single workgroup: thread 0 finishes every sample, so that its one fence orders all of them before the flag
+    if (threadIdx.x == 0) {
+        u64 s0 = 0;
+        for (int x = 0; x <= D.deg; ++x) {
+            u64 v;
+            if (D.skip1 && x == 1) {                     // S(1) = claim - S(0)
+                v = gl::sub(D.claim, s0);
+            } else {
+                v = red[0][x];
+                for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][x]);
+                if (scale != 1) v = gl::mul(v, scale);
+            }
+            if (x == 0) s0 = v;
+            out[x] = v;
+        }
+        if (flag) {
+            __threadfence_system();
+            __hip_atomic_store(out + NSAMP, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
     }
 }
@@ -341,8 +357,9 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
 
 // cross-block tree: one workgroup adds the per-block partials of every sample
 // skip1: sample 1 was not summed; it is claim - sample 0
+// flag: as in k_round
 __global__ __launch_bounds__(BLOCK) void k_final(const u64 *partial, int nb, int deg, u64 scale, int skip1, u64 claim,
-                                                 u64 *out) {
+                                                 u64 *out, u64 flag) {
     __shared__ u64 red[BLOCK / 64];
     u64 s0 = 0;
     for (int x = 0; x <= deg; ++x) {
@@ -363,6 +380,10 @@ __global__ __launch_bounds__(BLOCK) void k_final(const u64 *partial, int nb, int
             if (x == 0) s0 = v;
         }
         __syncthreads();
+    }
+    if (flag && threadIdx.x == 0) {                      // every sample above was stored by this thread
+        __threadfence_system();
+        __hip_atomic_store(out + NSAMP, flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
 
@@ -503,7 +524,7 @@ int resident_blocks(K kernel, int max_per_cu) {
 }
 
 template <int NT, int MODE, int U, int SHAPE, int NS>
-int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
+int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, u64 flag, hipStream_t s) {
     // per instantiation and device, looked up on first use there (devices of one process may differ)
     static std::mutex mu;
     static int caps[64] = {0};
@@ -516,42 +537,42 @@ int launch_kp(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u6
         cap = caps[dev];
     }
     if (nb > cap) nb = cap;
-    hipLaunchKernelGGL((k_round<NT, MODE, U, SHAPE, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct);
+    hipLaunchKernelGGL((k_round<NT, MODE, U, SHAPE, NS>), dim3(nb), dim3(BLOCK), 0, s, D, half, r, partial, out, scale, direct, flag);
     return nb;
 }
 
 template <int NT, int MODE, int U>
-int launch_k(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, hipStream_t s) {
+int launch_k(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct, u64 flag, hipStream_t s) {
     if (MODE != 1 && NT <= 4 && D.product && D.n_tables == NT)
-        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4) ? 1 : 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
+        return launch_kp<NT, MODE, U, (MODE != 1 && NT <= 4) ? 1 : 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, flag, s);
     if (MODE != 1 && NT == 4 && D.gate && D.n_tables == 4)
-        return launch_kp<NT, MODE, U, (MODE != 1 && NT == 4) ? 2 : 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
-    if (MODE != 1 && D.deg <= 3) return launch_kp<NT, MODE, U, 0, (MODE != 1 ? 4 : NSAMP)>(D, half, r, partial, nb, out, scale, direct, s);
-    return launch_kp<NT, MODE, U, 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, s);
+        return launch_kp<NT, MODE, U, (MODE != 1 && NT == 4) ? 2 : 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, flag, s);
+    if (MODE != 1 && D.deg <= 3) return launch_kp<NT, MODE, U, 0, (MODE != 1 ? 4 : NSAMP)>(D, half, r, partial, nb, out, scale, direct, flag, s);
+    return launch_kp<NT, MODE, U, 0, NSAMP>(D, half, r, partial, nb, out, scale, direct, flag, s);
 }
 
 template <int MODE, int U>
 int launch_round_u(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
-                   hipStream_t s) {
+                   u64 flag, hipStream_t s) {
     int nt = D.n_tables;
-    if (nt <= 1) return launch_k<1, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
-    if (nt <= 2) return launch_k<2, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
-    if (nt <= 3) return launch_k<3, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
-    if (nt <= 4) return launch_k<4, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
-    return launch_k<REG_TABLES, MODE, U>(D, half, r, partial, nb, out, scale, direct, s);
+    if (nt <= 1) return launch_k<1, MODE, U>(D, half, r, partial, nb, out, scale, direct, flag, s);
+    if (nt <= 2) return launch_k<2, MODE, U>(D, half, r, partial, nb, out, scale, direct, flag, s);
+    if (nt <= 3) return launch_k<3, MODE, U>(D, half, r, partial, nb, out, scale, direct, flag, s);
+    if (nt <= 4) return launch_k<4, MODE, U>(D, half, r, partial, nb, out, scale, direct, flag, s);
+    return launch_k<REG_TABLES, MODE, U>(D, half, r, partial, nb, out, scale, direct, flag, s);
 }
 
 // returns the number of workgroups actually launched (= partials written)
 template <int MODE>
 int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out, u64 scale, int direct,
-                 hipStream_t s) {
+                 u64 flag, hipStream_t s) {
     // two indices in flight for the load-light evaluation round on few tables
     if (MODE == 0 && D.n_tables <= 4 && nb > 1 && (half & 1) == 0) {
         bool aligned = true;
         for (int t = 0; t < D.n_tables; ++t) aligned = aligned && ((uintptr_t)D.src[t] & 15) == 0;
-        if (aligned) return launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, s);
+        if (aligned) return launch_round_u<MODE, 2>(D, half, r, partial, nb, out, scale, direct, flag, s);
     }
-    return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, s);
+    return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, flag, s);
 }
 
 }  // namespace
@@ -564,7 +585,7 @@ namespace {
 
 int sumcheck_eval_on(const char *who, const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
                      const int *factor_idx, const uint64_t *coeffs, int n_terms, uint64_t *out_samples, u64 *partial,
-                     void *stream) {
+                     u64 flag, void *stream) {
     Desc D;
     int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, who);
     if (rc) return rc;
@@ -574,14 +595,14 @@ int sumcheck_eval_on(const char *who, const uint64_t *const *tables, int n_table
     int nb = blocks_for(half);
     const u64 scale = D.out_scale;
     if (n_tables <= REG_TABLES && half <= DIRECT_MAX) {
-        launch_round<0>(D, half, 0, partial, 1, out_samples, scale, 1, s);
+        launch_round<0>(D, half, 0, partial, 1, out_samples, scale, 1, flag, s);
         VI_LAUNCH_CHECK("sumcheck eval");
         return VI_OK;
     }
-    if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, partial, nb, nullptr, 1, 0, s);
+    if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, partial, nb, nullptr, 1, 0, 0, s);
     else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, partial);
     VI_LAUNCH_CHECK("sumcheck eval");
-    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, D.deg, scale, 0, (u64)0, out_samples);
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, D.deg, scale, 0, (u64)0, out_samples, flag);
     VI_LAUNCH_CHECK("sumcheck final");
     return VI_OK;
 }
@@ -593,7 +614,7 @@ int vi_sumcheck_eval(const uint64_t *const *tables, int n_tables, int64_t half, 
                      uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream) {
     if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
     return sumcheck_eval_on("vi_sumcheck_eval", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, out_samples,
-                            (u64 *)ws, stream);
+                            (u64 *)ws, 0, stream);
 }
 
 // The per-workgroup partial sums of vi_sumcheck_eval_static: MAX_BLOCKS x NSAMP words (128 KiB) per GPU for the
@@ -633,13 +654,28 @@ int vi_sumcheck_eval_static(const uint64_t *const *tables, int n_tables, int64_t
     // every workgroup of the launch overwrites its own NSAMP words and the final kernel reads exactly those, so
     // nothing of an earlier call has to be cleared
     return sumcheck_eval_on("vi_sumcheck_eval_static", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms,
-                            out_samples, partial, stream);
+                            out_samples, partial, 0, stream);
+}
+
+namespace {
+int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables, int64_t half, uint64_t r,
+                 const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, const uint64_t *claim,
+                 uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream);
 }
 
 int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
                           int64_t half, uint64_t r, const int *term_off, const int *factor_idx,
                           const uint64_t *coeffs, int n_terms, const uint64_t *claim,
                           uint64_t *out_samples, void *ws, size_t ws_bytes, void *stream) {
+    return fold_eval_on(src, dst, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, claim, out_samples, ws, ws_bytes,
+                        0, stream);
+}
+
+namespace {
+// flag: non-zero = the kernel that finishes the samples also stores out_samples[NSAMP] = flag after them
+int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables, int64_t half, uint64_t r,
+                 const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, const uint64_t *claim,
+                 uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream) {
     const bool eval = out_samples != nullptr;
     Desc D;
     if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
@@ -670,7 +706,7 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
             Desc E = D;
             E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
             for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
-            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, s);
+            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, 0, s);
             VI_LAUNCH_CHECK("sumcheck fold");
         }
         return VI_OK;
@@ -679,18 +715,18 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
     const u64 scale = D.out_scale;
     if (n_tables <= REG_TABLES) {
         if ((half >> 1) <= DIRECT_MAX) {
-            launch_round<2>(D, half, r, (u64 *)ws, 1, out_samples, scale, 1, s);
+            launch_round<2>(D, half, r, (u64 *)ws, 1, out_samples, scale, 1, flag, s);
             VI_LAUNCH_CHECK("sumcheck fold+eval");
             return VI_OK;
         }
-        nb = launch_round<2>(D, half, r, (u64 *)ws, blocks_for(half >> 1), nullptr, 1, 0, s);
+        nb = launch_round<2>(D, half, r, (u64 *)ws, blocks_for(half >> 1), nullptr, 1, 0, 0, s);
         VI_LAUNCH_CHECK("sumcheck fold+eval");
     } else {
         for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {
             Desc E = D;
             E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
             for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
-            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, s);
+            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, 0, s);
             VI_LAUNCH_CHECK("sumcheck fold");
         }
         Desc E = D;
@@ -699,25 +735,56 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
         hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws);
         VI_LAUNCH_CHECK("sumcheck eval");
     }
-    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, D.skip1, D.claim, out_samples);
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, D.skip1, D.claim, out_samples, flag);
     VI_LAUNCH_CHECK("sumcheck final");
     return VI_OK;
 }
 
+// Lagrange weights of the points 0..n-1: winv[i] = 1 / prod_{k != i} (i - k)
+void lagrange_weights(int n, u64 *winv) {
+    for (int i = 0; i < n; ++i) {
+        u64 den = 1;
+        for (int k = 0; k < n; ++k)
+            if (k != i) den = gl::mul(den, gl::sub((u64)i, (u64)k));
+        winv[i] = gl::pow(den, gl::P - 2);
+    }
+}
+
 // value at x of the polynomial through (0, y[0]), ..., (n-1, y[n-1])
-static u64 interpolate_at(const u64 *y, int n, u64 x) {
+u64 interpolate_at(const u64 *y, const u64 *winv, int n, u64 x) {
     u64 total = 0;
     for (int i = 0; i < n; ++i) {
-        u64 num = y[i], den = 1;
-        for (int k = 0; k < n; ++k) {
-            if (k == i) continue;
-            num = gl::mul(num, gl::sub(x, (u64)k));
-            den = gl::mul(den, gl::sub((u64)i, (u64)k));
-        }
-        total = gl::add(total, gl::mul(num, gl::pow(den, gl::P - 2)));
+        u64 num = gl::mul(y[i], winv[i]);
+        for (int k = 0; k < n; ++k)
+            if (k != i) num = gl::mul(num, gl::sub(x, (u64)k));
+        total = gl::add(total, num);
     }
     return total;
 }
+
+// Waits until the kernel that finishes a round's samples has stored `seq` behind them.  The word is polled (a stream
+// synchronisation costs several microseconds more per round); every 2^16 polls the stream is queried, so a failed
+// launch or a stream that drained without the store ends the wait with an error instead of spinning.
+int wait_for_samples(const volatile u64 *flag, u64 seq, hipStream_t s) {
+    for (unsigned spins = 1;; ++spins) {
+        if (*flag == seq) break;
+        __builtin_ia32_pause();
+        if ((spins & 0xFFFF) == 0) {
+            hipError_t e = hipStreamQuery(s);
+            if (e == hipErrorNotReady) {
+                (void)hipGetLastError();                 // "not ready" is no error for the launch checks that follow
+                continue;
+            }
+            if (e != hipSuccess) return vi::fail(VI_EHIP, "vi_sumcheck_prove: %s while waiting for a round", hipGetErrorString(e));
+            // drained: host memory that is not coherent while a kernel runs shows the store now
+            if (*flag == seq) break;
+            return vi::fail(VI_EHIP, "vi_sumcheck_prove: the stream drained without the round's samples");
+        }
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
+    return VI_OK;
+}
+}  // namespace
 
 int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
                       const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
@@ -725,34 +792,48 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
                       uint64_t *out_challenges, void *ws, size_t ws_bytes, void *stream) {
     if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: size must be a power of two >= 2, got %lld", (long long)size);
     if (!coin || !host_samples || !out_samples || !out_challenges || !work) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: null pointer");
+    if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_prove: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
     Desc D;
     int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, "vi_sumcheck_prove");
     if (rc) return rc;
     const int ns = D.deg + 1;
+    u64 winv[NSAMP];
+    lagrange_weights(ns, winv);
     hipStream_t s = (hipStream_t)stream;
     int64_t half = size / 2;
-    rc = vi_sumcheck_eval(tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, host_samples, ws, ws_bytes, stream);
+    // host_samples[NSAMP] is the arrival word: round k's kernel stores k + 1 there behind its samples
+    volatile u64 *arrived = host_samples + NSAMP;
+    *arrived = 0;
+    std::atomic_thread_fence(std::memory_order_seq_cst);
+    rc = sumcheck_eval_on("vi_sumcheck_prove", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, host_samples,
+                          (u64 *)ws, 1, stream);
     if (rc) return rc;
     const uint64_t *const *src = tables;
     int round = 0;
     for (;;) {
-        VI_HIP(hipStreamSynchronize(s));
+        rc = wait_for_samples(arrived, (u64)round + 1, s);
+        if (rc) return rc;
         u64 y[NSAMP];
-        for (int x = 0; x < ns; ++x) y[x] = out_samples[(size_t)round * ns + x] = host_samples[x];
+        for (int x = 0; x < ns; ++x) y[x] = out_samples[(size_t)round * ns + x] = ((const volatile u64 *)host_samples)[x];
         uint64_t r = 0;
         int stop = coin(round, y, ns, &r, user);
-        if (stop) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: coin callback asked to stop in round %d", round);
+        if (stop) {
+            hipStreamSynchronize(s);
+            return vi::fail(VI_EINVAL, "vi_sumcheck_prove: coin callback asked to stop in round %d", round);
+        }
         r %= gl::P;
         out_challenges[round] = r;
         ++round;
         if (half < 2) break;
-        const uint64_t claim = interpolate_at(y, ns, r);
-        rc = vi_sumcheck_fold_eval(src, work, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, &claim,
-                                   host_samples, ws, ws_bytes, stream);
+        const uint64_t claim = interpolate_at(y, winv, ns, r);
+        rc = fold_eval_on(src, work, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, &claim, host_samples, ws,
+                          ws_bytes, (u64)round + 1, stream);
         if (rc) return rc;
         src = work;
         half /= 2;
     }
+    // the last round's kernel has stored its samples; wait for it to retire so that the caller may release buffers
+    VI_HIP(hipStreamSynchronize(s));
     return VI_OK;
 }
 

@@ -347,7 +347,7 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
             return (total + mu) % field_p, [], [], mu
 
         # The round loop runs inside the library (vi_sumcheck_prove): per round one fused
-        # launch, one stream synchronisation, the samples read from pinned host memory, and
+        # launch, a wait on a word of pinned host memory that the kernel stores behind its samples, and
         # this callback -- the only Python left in the loop -- which applies the optional
         # scalar mask and asks the verifier coin for the challenge.
         samples_host = _pinned_samples()
@@ -392,15 +392,16 @@ _PINNED = threading.local()
 
 
 def _pinned_samples():
-    """8 pinned host words the round kernels write their samples into.  One buffer per host thread and stream:
-    a proof waits for each round's samples before it goes on, so a thread needs one per stream it drives, and
+    """16 pinned host words (VI_SC_HOST_WORDS of the library header): the round kernels write their samples
+    into the first 8 and the count of rounds that have arrived into the ninth.  One buffer per host thread and
+    stream: a proof waits for each round's samples before it goes on, so a thread needs one per stream it drives, and
     two threads (or two streams) never see each other's samples."""
     bufs = getattr(_PINNED, "bufs", None)
     if bufs is None:
         bufs = _PINNED.bufs = {}
     key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
     if key not in bufs:
-        bufs[key] = torch.zeros(8, dtype=torch.uint64).pin_memory()
+        bufs[key] = torch.zeros(16, dtype=torch.uint64).pin_memory()
     return bufs[key]
 
 
