@@ -156,10 +156,12 @@ int vi_kquant_to_field_transposed(int qtype, const uint8_t *raw, int64_t d_out, 
  *   S(x) = sum_k coeffs[k] * sum_{i<half} prod_j (f_j[i] + x (f_j[half+i] - f_j[i])).
  *
  * The descriptor arrays (tables, term_off, factor_idx, coeffs) are HOST memory;
- * they are passed to the kernel by value (limits: VI_SC_MAX_TABLES, VI_SC_MAX_TERMS,
- * VI_SC_MAX_FACTORS).  out_samples: deg+1 words the GPU can write -- device memory or
- * pinned host memory (hipHostMalloc), the latter saves the copy back.  ws: device
- * scratch of vi_sumcheck_workspace_bytes() bytes. */
+ * they are passed to the kernel by value, VI_SC_MAX_TABLES / _TERMS / _FACTORS at a
+ * time: a larger sum (like the reference's, any number of tables and terms; at most 7
+ * factors per term) is evaluated in groups of consecutive terms, one launch each --
+ * only vi_sumcheck_eval_static keeps to a single descriptor.  out_samples: deg+1 words
+ * the GPU can write -- device memory or pinned host memory (hipHostMalloc), the latter
+ * saves the copy back.  ws: device scratch of vi_sumcheck_workspace_bytes() bytes. */
 #define VI_SC_MAX_TABLES 32
 #define VI_SC_MAX_TERMS 32
 #define VI_SC_MAX_FACTORS 64

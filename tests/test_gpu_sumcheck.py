@@ -124,6 +124,95 @@ def test_more_tables_than_fit_in_registers(mods):
     _check(gpu, tabs, terms, 13, as_tensor=True)
 
 
+def _layer_gate_batch(n_had, n_resc, n_bool, n_aff, v, seed):
+    """The shape of relations.prove_batch (layergkr/relations.py:104-124) over many gates: eq(z, .) in every term,
+    lambda-weighted hadamard (eq*a*b - eq*c), rescale (three linear terms), booleanity (eq*b*b - eq*b: a factor
+    twice in one term) and affine gates.  -> (tables, terms over table indices)"""
+    r = random.Random(seed)
+    tabs = [rand_field(1 << v, seed * 1000)]                     # stands in for eq(z, .)
+    terms = []
+
+    def new_table():
+        tabs.append(rand_field(1 << v, seed * 1000 + len(tabs)))
+        return len(tabs) - 1
+
+    for _ in range(n_had):
+        lam, a, b, c = r.randrange(P), new_table(), new_table(), new_table()
+        terms += [(lam, [0, a, b]), ((lam * (P - 1)) % P, [0, c])]
+    for _ in range(n_resc):
+        lam, raw, q, rem = r.randrange(P), new_table(), new_table(), new_table()
+        terms += [(lam, [0, raw]), ((lam * (P - 4096)) % P, [0, q]), ((lam * (P - 1)) % P, [0, rem])]
+    for _ in range(n_bool):
+        lam, b = r.randrange(P), new_table()
+        terms += [(lam, [0, b, b]), ((lam * (P - 1)) % P, [0, b])]
+    for _ in range(n_aff):
+        lam, x0, x1, y = r.randrange(P), new_table(), new_table(), new_table()
+        terms += [(lam, [0, x0]), (lam, [0, x1]), ((lam * (P - 1)) % P, [0, y])]
+    return tabs, terms
+
+
+@pytest.mark.parametrize("v", [1, 4, 9, 13])
+def test_gate_batch_of_a_whole_layer_beyond_one_descriptor(mods, v):
+    """97 tables and 88 terms: more than a kernel's descriptor holds (32 tables, 32 terms, 64 factors), so the
+    library evaluates the sum in groups of terms; the reference's prove_terms_gpu has no such limit."""
+    gpu, _ = mods
+    tabs, terms = _layer_gate_batch(n_had=12, n_resc=10, n_bool=6, n_aff=8, v=v, seed=21)
+    assert len(tabs) > 32 and len(terms) > 32
+    _check(gpu, tabs, terms, 22, as_tensor=True)
+
+
+def test_term_groups_cut_at_the_factor_and_table_limits(mods):
+    gpu, _ = mods
+    # ten terms of seven factors: 70 factors over 20 tables -- only the factor count exceeds a descriptor
+    tabs = [rand_field(1 << 6, 400 + j) for j in range(20)]
+    terms = [(j + 2, [(j + i) % 20 for i in range(7)]) for j in range(10)]
+    _check(gpu, tabs, terms, 23, as_tensor=True)
+    # forty single-table terms over forty tables: the table and term counts exceed it, the factor count does not
+    tabs = [rand_field(1 << 10, 440 + j) for j in range(40)]
+    terms = [(3 * j + 1, [j]) for j in range(40)]
+    _check(gpu, tabs, terms, 24, as_tensor=True)
+    # a term whose tables straddle two groups, and mixed degrees in each
+    tabs = [rand_field(1 << 8, 480 + j) for j in range(36)]
+    terms = [(j + 1, [j, j + 1]) for j in range(35)] + [(7, [0, 17, 35]), (P - 1, [35])]
+    _check(gpu, tabs, terms, 25, as_tensor=True)
+
+
+def test_large_sum_through_the_c_abi_round_by_round(mods):
+    """vi_sumcheck_eval and vi_sumcheck_fold_eval on 97 tables / 88 terms against the oracle's rounds 0 and 1;
+    the entry point that allocates nothing keeps to one descriptor and says so."""
+    import ctypes
+    from verinf_amd import _lib
+    L = _lib.lib()
+    tabs, terms = _layer_gate_batch(n_had=12, n_resc=10, n_bool=6, n_aff=8, v=11, seed=31)
+    n = len(tabs)
+    dev = [to_dev(t) for t in tabs]
+    dst = [torch.empty(1 << 10, dtype=torch.uint64, device="cuda") for _ in tabs]
+    src_p = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dev])
+    dst_p = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dst])
+    off, idx = [0], []
+    for _, fs in terms:
+        idx += fs
+        off.append(len(idx))
+    term_off, factor_idx = (ctypes.c_int * len(off))(*off), (ctypes.c_int * len(idx))(*idx)
+    coeffs = (ctypes.c_uint64 * len(terms))(*[c for c, _ in terms])
+    out = torch.zeros(8, dtype=torch.uint64, device="cuda")
+    ws = torch.empty(L.vi_sumcheck_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    r = 0x123456789ABCDEF0 % P
+    _, samples, _ = O.sumcheck_prove(tabs, terms, [r] + [1] * 10)
+    _lib.check(L.vi_sumcheck_eval(src_p, n, 1 << 10, term_off, factor_idx, coeffs, len(terms), out.data_ptr(),
+                                  ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    assert [int(x) for x in out.cpu().tolist()[:4]] == samples[0]
+    claim = (ctypes.c_uint64 * 1)(0)
+    _lib.check(L.vi_sumcheck_fold_eval(src_p, dst_p, n, 1 << 10, r, term_off, factor_idx, coeffs, len(terms), claim,
+                                       out.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+    assert [int(x) for x in out.cpu().tolist()[:4]] == samples[1]
+    for t, d in zip(tabs, dst):
+        assert np.array_equal(to_np(d), O.fold(t, r))
+    rc = L.vi_sumcheck_eval_static(src_p, n, 1 << 10, term_off, factor_idx, coeffs, len(terms), out.data_ptr(),
+                                   _lib.stream_ptr())
+    assert rc != 0 and "n_tables" in L.vi_last_error().decode()
+
+
 def test_degree_above_three_and_limits(mods):
     gpu, _ = mods
     tabs = [rand_field(1 << 7, 70 + j) for j in range(6)]

@@ -20,6 +20,7 @@
 // (layergkr/sumcheck.py:51-54).
 #include <atomic>
 #include <mutex>
+#include <vector>
 
 #include "common.hpp"
 #include "gl_field.hpp"
@@ -288,7 +289,9 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
 
 // tables kept in memory: for problems with more than REG_TABLES distinct tables.
 // The fold (if any) has already been done by k_round<*, 1>.
-__global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 *partial) {
+// A problem too large for one descriptor is evaluated as several launches over groups of its terms: each multiplies
+// its block sums by its own `scale` and, from the second group on (`accumulate`), adds them to what the slots hold.
+__global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 *partial, int accumulate, u64 scale) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const i64 stride = (i64)gridDim.x * BLOCK;
     u64 acc[NSAMP];
@@ -351,7 +354,9 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
     if (threadIdx.x < NSAMP) {
         u64 v = red[0][threadIdx.x];
         for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
-        partial[(i64)blockIdx.x * NSAMP + threadIdx.x] = v;
+        if (scale != 1) v = gl::mul(v, scale);
+        u64 *slot = partial + (i64)blockIdx.x * NSAMP + threadIdx.x;
+        *slot = accumulate ? gl::add(v, *slot) : v;
     }
 }
 
@@ -434,7 +439,8 @@ void factor_terms(Desc &D, const int *term_off, const int *factor_idx, int n_ter
 }
 
 int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_tables, const int *term_off,
-              const int *factor_idx, const uint64_t *coeffs, int n_terms, bool need_terms, const char *who) {
+              const int *factor_idx, const uint64_t *coeffs, int n_terms, bool need_terms, const char *who,
+              bool mem_path = false) {
     if (n_tables < 1 || n_tables > VI_SC_MAX_TABLES) return vi::fail(VI_EINVAL, "%s: n_tables = %d (1..%d)", who, n_tables, VI_SC_MAX_TABLES);
     D.n_tables = n_tables;
     for (int t = 0; t < n_tables; ++t) {
@@ -471,13 +477,14 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         D.fidx[j] = (unsigned char)factor_idx[j];
     }
     D.coeff_at_end = (n_terms == 1);
-    if (n_terms == 1 && n_tables <= REG_TABLES) D.out_scale = D.coeff[0];     // k_eval_mem applies it per term instead
+    if (n_terms == 1 && n_tables <= REG_TABLES && !mem_path) D.out_scale = D.coeff[0];     // k_eval_mem applies it per term instead
     if (n_terms == 1 && term_off[1] == n_tables && n_tables <= 4) {
         unsigned seen = 0;
         for (int j = 0; j < n_tables; ++j) seen |= 1u << factor_idx[j];
         D.product = (seen == (1u << n_tables) - 1);
     }
     if (n_terms >= 2) factor_terms(D, term_off, factor_idx, n_terms);
+    if (mem_path) return VI_OK;             // k_eval_mem walks the terms by index: no fixed shapes, no table order
     // the hadamard gate batch: four distinct tables, common * (f0 * f1 + c * lin).  The tables are put in that order
     // (sources and destinations together), so the kernel needs no indices.
     if (n_terms >= 2 && n_tables == 4 && D.common >= 0 && D.n_terms == 1 && D.term_off[1] == 2 && D.n_lin == 1 &&
@@ -575,6 +582,102 @@ int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out,
     return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, flag, s);
 }
 
+// ---- problems beyond one descriptor -------------------------------------------------------------------------
+// A descriptor travels to the kernel by value, which bounds it (VI_SC_MAX_TABLES / _TERMS / _FACTORS).  A larger
+// sum -- the batched gate check of a whole layer (layergkr/relations.py:104-124) has a few tables per gate and
+// eq(z, .) in every term -- is cut into groups of consecutive terms that each fit one descriptor; the groups are
+// evaluated one launch each over tables in memory and add into the same per-workgroup slots.
+
+struct TermGroup {
+    std::vector<int> tables;                // indices into the caller's table list, in order of first use
+    std::vector<int> term_off, fidx;        // the group's terms over positions in `tables`
+    std::vector<u64> coeffs;
+};
+
+inline bool fits_one_desc(int n_tables, const int *term_off, int n_terms) {
+    return n_tables <= VI_SC_MAX_TABLES && n_terms <= VI_SC_MAX_TERMS && term_off && term_off[0] == 0 &&
+           term_off[n_terms] <= VI_SC_MAX_FACTORS;
+}
+
+// argument checks for a term list of any length; *deg = the largest factor count
+int check_terms(const char *who, const uint64_t *const *tables, int n_tables, const int *term_off, const int *factor_idx,
+                const uint64_t *coeffs, int n_terms, int *deg) {
+    if (n_tables < 1 || !tables) return vi::fail(VI_EINVAL, "%s: n_tables = %d", who, n_tables);
+    for (int t = 0; t < n_tables; ++t)
+        if (!tables[t]) return vi::fail(VI_EINVAL, "%s: null table %d", who, t);
+    if (n_terms < 1) return vi::fail(VI_EINVAL, "%s: n_terms = %d", who, n_terms);
+    if (!term_off || !factor_idx || !coeffs) return vi::fail(VI_EINVAL, "%s: null term descriptor", who);
+    if (term_off[0] != 0) return vi::fail(VI_EINVAL, "%s: term_off[0] = %d", who, term_off[0]);
+    *deg = 0;
+    for (int k = 0; k < n_terms; ++k) {
+        const int nf = term_off[k + 1] - term_off[k];
+        if (nf < 1 || nf > MAX_DEG) return vi::fail(VI_EINVAL, "%s: term %d has %d factors (1..%d)", who, k, nf, MAX_DEG);
+        if (nf > *deg) *deg = nf;
+    }
+    for (int j = 0; j < term_off[n_terms]; ++j)
+        if (factor_idx[j] < 0 || factor_idx[j] >= n_tables) return vi::fail(VI_EINVAL, "%s: factor index %d out of range", who, factor_idx[j]);
+    return VI_OK;
+}
+
+// consecutive terms, as many per group as one descriptor holds (a single term always fits: <= MAX_DEG factors)
+void split_terms(int n_tables, const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                 std::vector<TermGroup> &groups) {
+    std::vector<int> local(n_tables, -1);
+    groups.clear();
+    groups.emplace_back();
+    groups.back().term_off.push_back(0);
+    for (int k = 0; k < n_terms; ++k) {
+        const int nf = term_off[k + 1] - term_off[k];
+        for (int attempt = 0;; ++attempt) {
+            TermGroup &G = groups.back();
+            int fresh = 0;
+            for (int j = term_off[k]; j < term_off[k + 1]; ++j) {
+                bool earlier = false;
+                for (int i = term_off[k]; i < j; ++i) earlier = earlier || factor_idx[i] == factor_idx[j];
+                if (local[factor_idx[j]] < 0 && !earlier) ++fresh;
+            }
+            const bool fits = (int)G.coeffs.size() < VI_SC_MAX_TERMS && (int)G.fidx.size() + nf <= VI_SC_MAX_FACTORS &&
+                              (int)G.tables.size() + fresh <= VI_SC_MAX_TABLES;
+            if (fits || attempt == 1) break;
+            for (int t : G.tables) local[t] = -1;          // close the group, open the next
+            groups.emplace_back();
+            groups.back().term_off.push_back(0);
+        }
+        TermGroup &G = groups.back();
+        for (int j = term_off[k]; j < term_off[k + 1]; ++j) {
+            const int t = factor_idx[j];
+            if (local[t] < 0) {
+                local[t] = (int)G.tables.size();
+                G.tables.push_back(t);
+            }
+            G.fidx.push_back(local[t]);
+        }
+        G.term_off.push_back((int)G.fidx.size());
+        G.coeffs.push_back(coeffs[k]);
+    }
+}
+
+// samples of sum over all groups at x = 0..deg from `tables` (pairs (i, half + i)); partial: MAX_BLOCKS * NSAMP words
+int eval_groups(const char *who, const uint64_t *const *tables, const std::vector<TermGroup> &groups, int deg, i64 half,
+                u64 *partial, u64 *out_samples, u64 flag, hipStream_t s) {
+    const int nb = blocks_for(half);
+    for (size_t g = 0; g < groups.size(); ++g) {
+        const TermGroup &G = groups[g];
+        const uint64_t *src[VI_SC_MAX_TABLES];
+        for (size_t t = 0; t < G.tables.size(); ++t) src[t] = tables[G.tables[t]];
+        Desc D;
+        int rc = fill_desc(D, src, nullptr, (int)G.tables.size(), G.term_off.data(), G.fidx.data(), G.coeffs.data(),
+                           (int)G.coeffs.size(), true, who, true);
+        if (rc) return rc;
+        D.deg = deg;                        // every group yields all the samples of the whole sum
+        hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, half, partial, g > 0 ? 1 : 0, D.out_scale);
+        VI_LAUNCH_CHECK("sumcheck eval (term group)");
+    }
+    hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, deg, (u64)1, 0, (u64)0, out_samples, flag);
+    VI_LAUNCH_CHECK("sumcheck final");
+    return VI_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -585,13 +688,24 @@ namespace {
 
 int sumcheck_eval_on(const char *who, const uint64_t *const *tables, int n_tables, int64_t half, const int *term_off,
                      const int *factor_idx, const uint64_t *coeffs, int n_terms, uint64_t *out_samples, u64 *partial,
-                     u64 flag, void *stream) {
-    Desc D;
-    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, who);
-    if (rc) return rc;
+                     u64 flag, void *stream, const std::vector<TermGroup> *groups = nullptr, bool may_split = true) {
     if (half < 1) return vi::fail(VI_EINVAL, "%s: half = %lld", who, (long long)half);
     if (!out_samples) return vi::fail(VI_EINVAL, "%s: null out_samples", who);
     hipStream_t s = (hipStream_t)stream;
+    if (may_split && n_terms >= 1 && term_off && !fits_one_desc(n_tables, term_off, n_terms)) {
+        int deg = 0;
+        int rc = check_terms(who, tables, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
+        if (rc) return rc;
+        std::vector<TermGroup> mine;
+        if (!groups) {
+            split_terms(n_tables, term_off, factor_idx, coeffs, n_terms, mine);
+            groups = &mine;
+        }
+        return eval_groups(who, tables, *groups, deg, half, partial, out_samples, flag, s);
+    }
+    Desc D;
+    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, who);
+    if (rc) return rc;
     int nb = blocks_for(half);
     const u64 scale = D.out_scale;
     if (n_tables <= REG_TABLES && half <= DIRECT_MAX) {
@@ -600,7 +714,7 @@ int sumcheck_eval_on(const char *who, const uint64_t *const *tables, int n_table
         return VI_OK;
     }
     if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, partial, nb, nullptr, 1, 0, 0, s);
-    else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, partial);
+    else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, partial, 0, (u64)1);
     VI_LAUNCH_CHECK("sumcheck eval");
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, D.deg, scale, 0, (u64)0, out_samples, flag);
     VI_LAUNCH_CHECK("sumcheck final");
@@ -654,13 +768,14 @@ int vi_sumcheck_eval_static(const uint64_t *const *tables, int n_tables, int64_t
     // every workgroup of the launch overwrites its own NSAMP words and the final kernel reads exactly those, so
     // nothing of an earlier call has to be cleared
     return sumcheck_eval_on("vi_sumcheck_eval_static", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms,
-                            out_samples, partial, 0, stream);
+                            out_samples, partial, 0, stream, nullptr, false);
 }
 
 namespace {
 int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables, int64_t half, uint64_t r,
                  const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, const uint64_t *claim,
-                 uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream);
+                 uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream,
+                 const std::vector<TermGroup> *groups = nullptr);
 }
 
 int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
@@ -675,7 +790,8 @@ namespace {
 // flag: non-zero = the kernel that finishes the samples also stores out_samples[NSAMP] = flag after them
 int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables, int64_t half, uint64_t r,
                  const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, const uint64_t *claim,
-                 uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream) {
+                 uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream,
+                 const std::vector<TermGroup> *groups) {
     const bool eval = out_samples != nullptr;
     Desc D;
     if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
@@ -688,6 +804,24 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
             if (rc) return rc;
         }
         return VI_OK;
+    }
+    if (eval && src && n_terms >= 1 && term_off && !fits_one_desc(n_tables, term_off, n_terms)) {
+        // more than one descriptor holds: fold every table, then evaluate the folded tables group by group
+        const char *who = "vi_sumcheck_fold_eval";
+        int deg = 0;
+        int rc = check_terms(who, src, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
+        if (rc) return rc;
+        if (half < 2) return vi::fail(VI_EINVAL, "%s: no next round after half = %lld; pass out_samples = NULL", who, (long long)half);
+        if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "%s: workspace below %zu bytes", who, vi_sumcheck_workspace_bytes());
+        rc = vi_sumcheck_fold_eval(src, dst, n_tables, half, r, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, stream);
+        if (rc) return rc;
+        std::vector<TermGroup> mine;
+        if (!groups) {
+            split_terms(n_tables, term_off, factor_idx, coeffs, n_terms, mine);
+            groups = &mine;
+        }
+        return eval_groups(who, (const uint64_t *const *)dst, *groups, deg, half >> 1, (u64 *)ws, out_samples, flag,
+                           (hipStream_t)stream);
     }
     int rc = fill_desc(D, src, dst, n_tables, term_off, factor_idx, coeffs, n_terms, eval, "vi_sumcheck_fold_eval");
     if (rc) return rc;
@@ -732,7 +866,7 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
         Desc E = D;
         for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
         nb = blocks_for(half >> 1);
-        hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws);
+        hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws, 0, (u64)1);
         VI_LAUNCH_CHECK("sumcheck eval");
     }
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, D.skip1, D.claim, out_samples, flag);
@@ -793,10 +927,16 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
     if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: size must be a power of two >= 2, got %lld", (long long)size);
     if (!coin || !host_samples || !out_samples || !out_challenges || !work) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: null pointer");
     if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_prove: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
-    Desc D;
-    int rc = fill_desc(D, tables, nullptr, n_tables, term_off, factor_idx, coeffs, n_terms, true, "vi_sumcheck_prove");
+    int deg = 0;
+    int rc = check_terms("vi_sumcheck_prove", tables, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
     if (rc) return rc;
-    const int ns = D.deg + 1;
+    for (int t = 0; t < n_tables; ++t)
+        if (!work[t]) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: null work buffer %d", t);
+    // a sum beyond one descriptor is cut into groups of terms once for all rounds
+    std::vector<TermGroup> groups;
+    const bool split = !fits_one_desc(n_tables, term_off, n_terms);
+    if (split) split_terms(n_tables, term_off, factor_idx, coeffs, n_terms, groups);
+    const int ns = deg + 1;
     u64 winv[NSAMP];
     lagrange_weights(ns, winv);
     hipStream_t s = (hipStream_t)stream;
@@ -806,7 +946,7 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
     *arrived = 0;
     std::atomic_thread_fence(std::memory_order_seq_cst);
     rc = sumcheck_eval_on("vi_sumcheck_prove", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, host_samples,
-                          (u64 *)ws, 1, stream);
+                          (u64 *)ws, 1, stream, split ? &groups : nullptr);
     if (rc) return rc;
     const uint64_t *const *src = tables;
     int round = 0;
@@ -818,7 +958,7 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
         uint64_t r = 0;
         int stop = coin(round, y, ns, &r, user);
         if (stop) {
-            hipStreamSynchronize(s);
+            (void)hipStreamSynchronize(s);     // the last kernel retires before the caller releases its buffers
             return vi::fail(VI_EINVAL, "vi_sumcheck_prove: coin callback asked to stop in round %d", round);
         }
         r %= gl::P;
@@ -827,7 +967,7 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
         if (half < 2) break;
         const uint64_t claim = interpolate_at(y, winv, ns, r);
         rc = fold_eval_on(src, work, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, &claim, host_samples, ws,
-                          ws_bytes, (u64)round + 1, stream);
+                          ws_bytes, (u64)round + 1, stream, split ? &groups : nullptr);
         if (rc) return rc;
         src = work;
         half /= 2;
