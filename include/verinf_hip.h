@@ -162,9 +162,9 @@ int vi_kquant_to_field_transposed(int qtype, const uint8_t *raw, int64_t d_out, 
  * only vi_sumcheck_eval_static keeps to a single descriptor.  out_samples: deg+1 words
  * the GPU can write -- device memory or pinned host memory (hipHostMalloc), the latter
  * saves the copy back.  ws: device scratch of vi_sumcheck_workspace_bytes() bytes. */
-#define VI_SC_MAX_TABLES 32
-#define VI_SC_MAX_TERMS 32
-#define VI_SC_MAX_FACTORS 64
+#define VI_SC_MAX_TABLES 64
+#define VI_SC_MAX_TERMS 64
+#define VI_SC_MAX_FACTORS 128
 size_t vi_sumcheck_workspace_bytes(void);
 
 /* samples of the current round (sumcheck.py:194-205 / gpu.py:384-394) */

@@ -153,32 +153,37 @@ def _layer_gate_batch(n_had, n_resc, n_bool, n_aff, v, seed):
 
 @pytest.mark.parametrize("v", [1, 4, 9, 13])
 def test_gate_batch_of_a_whole_layer_beyond_one_descriptor(mods, v):
-    """97 tables and 88 terms: more than a kernel's descriptor holds (32 tables, 32 terms, 64 factors), so the
+    """97 tables and 90 terms: more than a kernel's descriptor holds (64 tables, 64 terms, 128 factors), so the
     library evaluates the sum in groups of terms; the reference's prove_terms_gpu has no such limit."""
     gpu, _ = mods
     tabs, terms = _layer_gate_batch(n_had=12, n_resc=10, n_bool=6, n_aff=8, v=v, seed=21)
-    assert len(tabs) > 32 and len(terms) > 32
+    assert len(tabs) > 64 and len(terms) > 64
     _check(gpu, tabs, terms, 22, as_tensor=True)
 
 
 def test_term_groups_cut_at_the_factor_and_table_limits(mods):
     gpu, _ = mods
-    # ten terms of seven factors: 70 factors over 20 tables -- only the factor count exceeds a descriptor
+    # twenty terms of seven factors: 140 factors over 20 tables -- only the factor count exceeds a descriptor
     tabs = [rand_field(1 << 6, 400 + j) for j in range(20)]
-    terms = [(j + 2, [(j + i) % 20 for i in range(7)]) for j in range(10)]
+    terms = [(j + 2, [(j + i) % 20 for i in range(7)]) for j in range(20)]
     _check(gpu, tabs, terms, 23, as_tensor=True)
-    # forty single-table terms over forty tables: the table and term counts exceed it, the factor count does not
-    tabs = [rand_field(1 << 10, 440 + j) for j in range(40)]
-    terms = [(3 * j + 1, [j]) for j in range(40)]
+    # seventy single-table terms over seventy tables: the table and term counts exceed it, the factor count does not
+    tabs = [rand_field(1 << 10, 440 + j) for j in range(70)]
+    terms = [(3 * j + 1, [j]) for j in range(70)]
     _check(gpu, tabs, terms, 24, as_tensor=True)
     # a term whose tables straddle two groups, and mixed degrees in each
-    tabs = [rand_field(1 << 8, 480 + j) for j in range(36)]
-    terms = [(j + 1, [j, j + 1]) for j in range(35)] + [(7, [0, 17, 35]), (P - 1, [35])]
+    tabs = [rand_field(1 << 8, 520 + j) for j in range(72)]
+    terms = [(j + 1, [j, j + 1]) for j in range(71)] + [(7, [0, 35, 71]), (P - 1, [71])]
     _check(gpu, tabs, terms, 25, as_tensor=True)
+    # exactly one descriptor's worth of tables and terms, and one more
+    for n in (64, 65):
+        tabs = [rand_field(1 << 7, 600 + j) for j in range(n)]
+        terms = [(j + 5, [j, (j + 1) % n]) for j in range(n)]
+        _check(gpu, tabs, terms, 26 + n, as_tensor=True)
 
 
 def test_large_sum_through_the_c_abi_round_by_round(mods):
-    """vi_sumcheck_eval and vi_sumcheck_fold_eval on 97 tables / 88 terms against the oracle's rounds 0 and 1;
+    """vi_sumcheck_eval and vi_sumcheck_fold_eval on 97 tables / 90 terms against the oracle's rounds 0 and 1;
     the entry point that allocates nothing keeps to one descriptor and says so."""
     import ctypes
     from verinf_amd import _lib

@@ -291,8 +291,12 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
 // The fold (if any) has already been done by k_round<*, 1>.
 // A problem too large for one descriptor is evaluated as several launches over groups of its terms: each multiplies
 // its block sums by its own `scale` and, from the second group on (`accumulate`), adds them to what the slots hold.
+// Small rounds are bound by the latency of one thread's chain of loads (two per factor slot), so the grid's y dimension
+// deals the terms out: workgroup row ty takes the terms k = ty (mod gridDim.y) of the bracket -- the constant c0 goes
+// to row 0 -- and multiplies its share by the common factor; the shares add up in k_final like any other partials.
 __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 *partial, int accumulate, u64 scale) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
+    const int ty = blockIdx.y, ny = gridDim.y;
     const i64 stride = (i64)gridDim.x * BLOCK;
     u64 acc[NSAMP];
 #pragma unroll
@@ -301,8 +305,8 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
         // the factored form described at Desc, every factor fetched from its table
         u64 sx[NSAMP];
         {
-            u64 lc = D.c0, ld = 0;
-            for (int k = 0; k < D.n_lin; ++k) {
+            u64 lc = ty == 0 ? D.c0 : 0, ld = 0;
+            for (int k = ty; k < D.n_lin; k += ny) {
                 const u64 *f = D.src[D.lin_idx[k]];
                 const u64 c = D.lin_coeff[k], cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
                 lc = gl::add(lc, gl::mul(c, cur));
@@ -314,7 +318,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
                 if (D.n_lin) lc = gl::add(lc, ld);
             }
         }
-        for (int k = 0; k < D.n_terms; ++k) {
+        for (int k = ty; k < D.n_terms; k += ny) {
             u64 prod[NSAMP];
 #pragma unroll
             for (int x = 0; x < NSAMP; ++x) prod[x] = D.coeff[k];
@@ -355,9 +359,29 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
         u64 v = red[0][threadIdx.x];
         for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
         if (scale != 1) v = gl::mul(v, scale);
-        u64 *slot = partial + (i64)blockIdx.x * NSAMP + threadIdx.x;
+        u64 *slot = partial + ((i64)blockIdx.y * gridDim.x + blockIdx.x) * NSAMP + threadIdx.x;
         *slot = accumulate ? gl::add(v, *slot) : v;
     }
+}
+
+// fold of many tables in one launch: blockIdx.y = table, the x dimension strides over the lower half
+constexpr int FOLD_MANY = 64;
+struct FoldDesc {
+    const u64 *src[FOLD_MANY];
+    u64 *dst[FOLD_MANY];
+};
+__global__ __launch_bounds__(BLOCK) void k_fold_many(const FoldDesc F, i64 half, u64 r) {
+    const u64 *src = F.src[blockIdx.y];
+    u64 *dst = F.dst[blockIdx.y];
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x;
+    for (; i + stride < half; i += 2 * stride) {         // two independent indices in flight
+        const u64 lo0 = src[i], hi0 = src[half + i];
+        const u64 lo1 = src[i + stride], hi1 = src[half + i + stride];
+        dst[i] = fold1(lo0, hi0, r);
+        dst[i + stride] = fold1(lo1, hi1, r);
+    }
+    if (i < half) dst[i] = fold1(src[i], src[half + i], r);
 }
 
 // cross-block tree: one workgroup adds the per-block partials of every sample
@@ -582,6 +606,36 @@ int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out,
     return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, flag, s);
 }
 
+// k_eval_mem over `half` pairs: returns the number of partial slots written (x workgroups times term rows)
+int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 scale, hipStream_t s) {
+    const int nbx = blocks_for(half);
+    int ny = 1;
+    while (ny < 16 && nbx * ny * 2 <= 1024) ny *= 2;     // deal the terms out while the grid is below ~4 workgroups per CU
+    hipLaunchKernelGGL(k_eval_mem, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
+    return nbx * ny;
+}
+
+// fold `n` tables by r: up to REG_TABLES through the register kernel, more through k_fold_many (FOLD_MANY per launch)
+int fold_tables(const uint64_t *const *src, uint64_t *const *dst, int n, i64 half, u64 r, hipStream_t s) {
+    for (int t = 0; t < n; ++t)
+        if (!src[t] || !dst[t]) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null table %d", t);
+    int nbx = blocks_for((half + 1) / 2);
+    for (int t0 = 0; t0 < n; t0 += FOLD_MANY) {
+        const int cnt = (n - t0 < FOLD_MANY) ? (n - t0) : FOLD_MANY;
+        FoldDesc F;
+        for (int t = 0; t < FOLD_MANY; ++t) {
+            F.src[t] = t < cnt ? src[t0 + t] : nullptr;
+            F.dst[t] = t < cnt ? dst[t0 + t] : nullptr;
+        }
+        // a few thousand workgroups fill the chip; beyond that a workgroup takes more indices
+        int bx = nbx;
+        while (bx > 1 && (i64)bx * cnt > 8192) bx = (bx + 1) / 2;
+        hipLaunchKernelGGL(k_fold_many, dim3(bx, cnt), dim3(BLOCK), 0, s, F, half, r);
+        VI_LAUNCH_CHECK("sumcheck fold (many tables)");
+    }
+    return VI_OK;
+}
+
 // ---- problems beyond one descriptor -------------------------------------------------------------------------
 // A descriptor travels to the kernel by value, which bounds it (VI_SC_MAX_TABLES / _TERMS / _FACTORS).  A larger
 // sum -- the batched gate check of a whole layer (layergkr/relations.py:104-124) has a few tables per gate and
@@ -660,7 +714,7 @@ void split_terms(int n_tables, const int *term_off, const int *factor_idx, const
 // samples of sum over all groups at x = 0..deg from `tables` (pairs (i, half + i)); partial: MAX_BLOCKS * NSAMP words
 int eval_groups(const char *who, const uint64_t *const *tables, const std::vector<TermGroup> &groups, int deg, i64 half,
                 u64 *partial, u64 *out_samples, u64 flag, hipStream_t s) {
-    const int nb = blocks_for(half);
+    int nb = 0;
     for (size_t g = 0; g < groups.size(); ++g) {
         const TermGroup &G = groups[g];
         const uint64_t *src[VI_SC_MAX_TABLES];
@@ -670,7 +724,7 @@ int eval_groups(const char *who, const uint64_t *const *tables, const std::vecto
                            (int)G.coeffs.size(), true, who, true);
         if (rc) return rc;
         D.deg = deg;                        // every group yields all the samples of the whole sum
-        hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, half, partial, g > 0 ? 1 : 0, D.out_scale);
+        nb = launch_eval_mem(D, half, partial, g > 0 ? 1 : 0, D.out_scale, s);    // the same grid for every group
         VI_LAUNCH_CHECK("sumcheck eval (term group)");
     }
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, deg, (u64)1, 0, (u64)0, out_samples, flag);
@@ -714,7 +768,7 @@ int sumcheck_eval_on(const char *who, const uint64_t *const *tables, int n_table
         return VI_OK;
     }
     if (n_tables <= REG_TABLES) nb = launch_round<0>(D, half, 0, partial, nb, nullptr, 1, 0, 0, s);
-    else hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, D, (i64)half, partial, 0, (u64)1);
+    else nb = launch_eval_mem(D, half, partial, 0, 1, s);
     VI_LAUNCH_CHECK("sumcheck eval");
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, D.deg, scale, 0, (u64)0, out_samples, flag);
     VI_LAUNCH_CHECK("sumcheck final");
@@ -795,15 +849,10 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
     const bool eval = out_samples != nullptr;
     Desc D;
     if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
-    if (!eval && src && n_tables > VI_SC_MAX_TABLES) {
-        // folding alone has no limit on the number of tables: a descriptor's worth at a time
-        for (int t0 = 0; t0 < n_tables; t0 += VI_SC_MAX_TABLES) {
-            const int cnt = (n_tables - t0 < VI_SC_MAX_TABLES) ? (n_tables - t0) : VI_SC_MAX_TABLES;
-            int rc = vi_sumcheck_fold_eval(src + t0, dst + t0, cnt, half, r, nullptr, nullptr, nullptr, 0, nullptr, nullptr,
-                                           nullptr, 0, stream);
-            if (rc) return rc;
-        }
-        return VI_OK;
+    if (!eval && src && n_tables > REG_TABLES) {
+        // folding alone has no limit on the number of tables
+        if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: half = %lld", (long long)half);
+        return fold_tables(src, dst, n_tables, half, r % gl::P, (hipStream_t)stream);
     }
     if (eval && src && n_terms >= 1 && term_off && !fits_one_desc(n_tables, term_off, n_terms)) {
         // more than one descriptor holds: fold every table, then evaluate the folded tables group by group
@@ -835,14 +884,9 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
         D.claim = *claim % gl::P;
     }
     hipStream_t s = (hipStream_t)stream;
-    if (!eval) {
-        for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {       // any number of tables, REG_TABLES per launch
-            Desc E = D;
-            E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
-            for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
-            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, 0, s);
-            VI_LAUNCH_CHECK("sumcheck fold");
-        }
+    if (!eval) {                                                  // at most REG_TABLES tables: one launch
+        launch_round<1>(D, half, r, nullptr, blocks_for(half), nullptr, 1, 0, 0, s);
+        VI_LAUNCH_CHECK("sumcheck fold");
         return VI_OK;
     }
     int nb;
@@ -856,17 +900,11 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
         nb = launch_round<2>(D, half, r, (u64 *)ws, blocks_for(half >> 1), nullptr, 1, 0, 0, s);
         VI_LAUNCH_CHECK("sumcheck fold+eval");
     } else {
-        for (int t0 = 0; t0 < n_tables; t0 += REG_TABLES) {
-            Desc E = D;
-            E.n_tables = (n_tables - t0 < REG_TABLES) ? (n_tables - t0) : REG_TABLES;
-            for (int t = 0; t < E.n_tables; ++t) { E.src[t] = D.src[t0 + t]; E.dst[t] = D.dst[t0 + t]; }
-            launch_round<1>(E, half, r, nullptr, blocks_for(half), nullptr, 1, 0, 0, s);
-            VI_LAUNCH_CHECK("sumcheck fold");
-        }
+        rc = fold_tables(src, dst, n_tables, half, r, s);
+        if (rc) return rc;
         Desc E = D;
         for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
-        nb = blocks_for(half >> 1);
-        hipLaunchKernelGGL(k_eval_mem, dim3(nb), dim3(BLOCK), 0, s, E, (i64)(half >> 1), (u64 *)ws, 0, (u64)1);
+        nb = launch_eval_mem(E, half >> 1, (u64 *)ws, 0, 1, s);
         VI_LAUNCH_CHECK("sumcheck eval");
     }
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)ws, nb, D.deg, scale, D.skip1, D.claim, out_samples, flag);
