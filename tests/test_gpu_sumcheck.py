@@ -151,10 +151,11 @@ def _layer_gate_batch(n_had, n_resc, n_bool, n_aff, v, seed):
     return tabs, terms
 
 
-@pytest.mark.parametrize("v", [1, 4, 9, 13])
+@pytest.mark.parametrize("v", [1, 4, 9, 13, 20])
 def test_gate_batch_of_a_whole_layer_beyond_one_descriptor(mods, v):
     """97 tables and 90 terms: more than a kernel's descriptor holds (64 tables, 64 terms, 128 factors), so the
-    library evaluates the sum in groups of terms; the reference's prove_terms_gpu has no such limit."""
+    library evaluates the sum in groups of terms; the reference's prove_terms_gpu has no such limit.  At 2^20 the
+    first rounds evaluate in one row of workgroups, the later ones deal the terms over several rows."""
     gpu, _ = mods
     tabs, terms = _layer_gate_batch(n_had=12, n_resc=10, n_bool=6, n_aff=8, v=v, seed=21)
     assert len(tabs) > 64 and len(terms) > 64
@@ -216,6 +217,51 @@ def test_large_sum_through_the_c_abi_round_by_round(mods):
     rc = L.vi_sumcheck_eval_static(src_p, n, 1 << 10, term_off, factor_idx, coeffs, len(terms), out.data_ptr(),
                                    _lib.stream_ptr())
     assert rc != 0 and "n_tables" in L.vi_last_error().decode()
+
+
+def test_tables_in_memory_at_full_grid_size(mods):
+    """11 and 40 tables at 2^20 (one descriptor): the first rounds fill the capped grid of the evaluation kernel and
+    of the many-table fold, the later ones deal the terms over rows of workgroups."""
+    gpu, _ = mods
+    r = random.Random(15)
+    tabs = [rand_field(1 << 20, 700 + j) for j in range(11)]
+    terms = [(r.randrange(P), [j, (j + 1) % 11]) for j in range(11)] + [(3, [0, 5, 10])]
+    _check(gpu, tabs, terms, 16, as_tensor=True)
+    tabs = [rand_field(1 << 20, 720 + j) for j in range(40)]
+    terms = [(r.randrange(P), [0, j, j + 1]) for j in range(1, 39, 2)] + [(r.randrange(P), [0, j]) for j in range(1, 40)]
+    _check(gpu, tabs, terms, 17, as_tensor=True)
+
+
+def test_fold_eval_in_place_with_unused_tables_c_abi(mods):
+    """vi_sumcheck_fold_eval, dst == src, at 2^20: 70 tables of which five occur in no term (they are folded all
+    the same), the sum beyond one descriptor; and the same tables through one descriptor's worth of terms."""
+    import ctypes
+    from verinf_amd import _lib
+    L = _lib.lib()
+    n, v = 70, 20
+    tabs = [rand_field(1 << v, 800 + j) for j in range(n)]
+    used = [j for j in range(n) if j % 14 != 3]
+    r = 0x0FEDCBA987654321 % P
+    folded = [O.fold(t, r) for t in tabs]
+    for terms in ([(j + 2, [used[j], used[(j + 1) % len(used)]]) for j in range(len(used))],       # 65 terms: two groups
+                  [(j + 2, [used[j], used[j + 1], used[j + 2]]) for j in range(0, 30, 3)]):           # one descriptor
+        dev = [to_dev(t) for t in tabs]
+        ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dev])
+        off, idx = [0], []
+        for _, fs in terms:
+            idx += fs
+            off.append(len(idx))
+        term_off, factor_idx = (ctypes.c_int * len(off))(*off), (ctypes.c_int * len(idx))(*idx)
+        coeffs = (ctypes.c_uint64 * len(terms))(*[c for c, _ in terms])
+        out = torch.zeros(8, dtype=torch.uint64, device="cuda")
+        ws = torch.empty(L.vi_sumcheck_workspace_bytes(), dtype=torch.uint8, device="cuda")
+        _lib.check(L.vi_sumcheck_fold_eval(ptrs, ptrs, n, 1 << (v - 1), r, term_off, factor_idx, coeffs, len(terms), None,
+                                           out.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr()))
+        deg = max(len(fs) for _, fs in terms)
+        _, samples, _ = O.sumcheck_prove(folded, terms, [1] * (v - 1))
+        assert [int(x) for x in out.cpu().tolist()[:deg + 1]] == samples[0]
+        for t, f in zip(dev, folded):
+            assert np.array_equal(to_np(t)[: 1 << (v - 1)], f)
 
 
 def test_degree_above_three_and_limits(mods):

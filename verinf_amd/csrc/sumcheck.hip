@@ -302,15 +302,36 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
 #pragma unroll
     for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride) {
-        // the factored form described at Desc, every factor fetched from its table
+        // the factored form described at Desc, every factor fetched from its table.  Loads go out in batches ahead
+        // of the arithmetic that uses them (the common factor first, used last; four linear terms; two factor slots
+        // of a product): one thread's loads are otherwise a chain of round trips to memory.  A slot past the end of
+        // its list repeats a valid load (a cache hit) with coefficient 0 or is skipped by a wavefront-uniform test.
         u64 sx[NSAMP];
+        u64 com_lo = 0, com_hi = 0;
+        if (D.common >= 0) {
+            const u64 *f = D.src[D.common];
+            com_lo = f[i];
+            com_hi = f[half + i];
+        }
         {
             u64 lc = ty == 0 ? D.c0 : 0, ld = 0;
-            for (int k = ty; k < D.n_lin; k += ny) {
-                const u64 *f = D.src[D.lin_idx[k]];
-                const u64 c = D.lin_coeff[k], cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
-                lc = gl::add(lc, gl::mul(c, cur));
-                ld = gl::add(ld, gl::mul(c, dif));
+            for (int k0 = ty; k0 < D.n_lin; k0 += 4 * ny) {
+                u64 a[4], b[4], c[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int k = k0 + u * ny;
+                    const bool on = k < D.n_lin;
+                    const u64 *f = D.src[D.lin_idx[on ? k : k0]];
+                    a[u] = f[i];
+                    b[u] = f[half + i];
+                    c[u] = on ? D.lin_coeff[k] : 0;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const u64 cur = gl::canon(a[u]), dif = gl::sub(gl::canon(b[u]), cur);
+                    lc = gl::add(lc, gl::mul(c[u], cur));
+                    ld = gl::add(ld, gl::mul(c[u], dif));
+                }
             }
 #pragma unroll
             for (int x = 0; x < NSAMP; ++x) {
@@ -322,13 +343,25 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
             u64 prod[NSAMP];
 #pragma unroll
             for (int x = 0; x < NSAMP; ++x) prod[x] = D.coeff[k];
-            for (int j = D.term_off[k]; j < D.term_off[k + 1]; ++j) {
-                const u64 *f = D.src[D.fidx[j]];
-                u64 cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
+            const int j1 = D.term_off[k + 1];
+            for (int j = D.term_off[k]; j < j1; j += 2) {
+                const bool two = j + 1 < j1;
+                const u64 *f0 = D.src[D.fidx[j]], *f1 = D.src[D.fidx[two ? j + 1 : j]];
+                const u64 a0 = f0[i], b0 = f0[half + i], a1 = f1[i], b1 = f1[half + i];
+                u64 cur = gl::canon(a0), dif = gl::sub(gl::canon(b0), cur);
 #pragma unroll
                 for (int x = 0; x < NSAMP; ++x) {
                     if (x <= D.deg) prod[x] = gl::mul(prod[x], cur);
                     cur = gl::add(cur, dif);
+                }
+                if (two) {
+                    cur = gl::canon(a1);
+                    dif = gl::sub(gl::canon(b1), cur);
+#pragma unroll
+                    for (int x = 0; x < NSAMP; ++x) {
+                        if (x <= D.deg) prod[x] = gl::mul(prod[x], cur);
+                        cur = gl::add(cur, dif);
+                    }
                 }
             }
 #pragma unroll
@@ -336,8 +369,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
                 if (x <= D.deg) sx[x] = gl::add(sx[x], prod[x]);
         }
         if (D.common >= 0) {
-            const u64 *f = D.src[D.common];
-            u64 cur = gl::canon(f[i]), dif = gl::sub(gl::canon(f[half + i]), cur);
+            u64 cur = gl::canon(com_lo), dif = gl::sub(gl::canon(com_hi), cur);
 #pragma unroll
             for (int x = 0; x < NSAMP; ++x) {
                 if (x <= D.deg) sx[x] = gl::mul(sx[x], cur);
@@ -608,7 +640,19 @@ int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out,
 
 // k_eval_mem over `half` pairs: returns the number of partial slots written (x workgroups times term rows)
 int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 scale, hipStream_t s) {
-    const int nbx = blocks_for(half);
+    // a grid-stride loop: no more workgroups than are resident at once (see resident_blocks), looked up per device
+    static std::mutex mu;
+    static int caps[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    int cap;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem, 64);
+        cap = caps[dev];
+    }
+    int nbx = blocks_for(half);
+    if (nbx > cap) nbx = cap;
     int ny = 1;
     while (ny < 16 && nbx * ny * 2 <= 1024) ny *= 2;     // deal the terms out while the grid is below ~4 workgroups per CU
     hipLaunchKernelGGL(k_eval_mem, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
