@@ -264,6 +264,26 @@ def test_fold_eval_in_place_with_unused_tables_c_abi(mods):
             assert np.array_equal(to_np(t)[: 1 << (v - 1)], f)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_term_structures_match_oracle(mods, seed):
+    """Seeded random sums: 1..100 tables, 1..100 terms of 1..4 factors (repeats allowed), a table shared by all
+    terms or not, tables nobody uses, 2^1..2^11 entries -- the register path, one descriptor in memory, and groups."""
+    gpu, _ = mods
+    r = random.Random(9000 + seed)
+    n_tables = r.choice([1, 2, 3, 4, 5, 8, 9, 17, 33, 64, 65, 100])
+    n_terms = r.choice([1, 2, 3, 7, 31, 64, 65, 100])
+    v = r.randrange(1, 12)
+    shared = r.random() < 0.5
+    tabs = [rand_field(1 << v, 9100 + 101 * seed + j) for j in range(n_tables)]
+    terms = []
+    for _ in range(n_terms):
+        fs = [r.randrange(n_tables) for _ in range(r.randrange(1, 5))]
+        if shared:
+            fs[r.randrange(len(fs))] = 0
+        terms.append((r.choice([1, 2, P - 1, r.randrange(P)]), fs))
+    _check(gpu, tabs, terms, 9200 + seed, as_tensor=True)
+
+
 def test_degree_above_three_and_limits(mods):
     gpu, _ = mods
     tabs = [rand_field(1 << 7, 70 + j) for j in range(6)]
