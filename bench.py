@@ -178,6 +178,72 @@ def bench_sumcheck(torch, v=26, cpu=True):
     return res
 
 
+def bench_gate_batch(torch, v=22, cpu=True):
+    """The gate batch of a whole layer in the shape of relations.prove_batch (layergkr/relations.py:104-124): one
+    eq table in every term, lambda-weighted hadamard (eq*a*b - eq*c), rescale (three linear terms), booleanity
+    (eq*b*b - eq*b) and affine gates -- 97 tables, 90 terms, degree 3, more than one kernel descriptor holds, so
+    the tables are walked in memory and the terms in groups.  Proved at 2^v, checked through the verifier, and at
+    2^14 compared with the C oracle round by round."""
+    from verinf_amd.layergkr import gpu
+    from verinf_amd.layergkr import sumcheck as sc
+    r = random.Random(41)
+
+    def problem(vv):
+        tabs = [rand_field(torch, (1 << vv,), 4000)]
+        terms = []
+
+        def t():
+            tabs.append(rand_field(torch, (1 << vv,), 4000 + len(tabs)))
+            return len(tabs) - 1
+
+        for kind, count in (("had", 12), ("resc", 10), ("bool", 6), ("aff", 8)):
+            for _ in range(count):
+                lam = r.randrange(P)
+                neg = lam * (P - 1) % P
+                if kind == "had":
+                    a, b, c = t(), t(), t()
+                    terms += [(lam, [0, a, b]), (neg, [0, c])]
+                elif kind == "resc":
+                    raw, q, rem = t(), t(), t()
+                    terms += [(lam, [0, raw]), (lam * (P - 4096) % P, [0, q]), (neg, [0, rem])]
+                elif kind == "bool":
+                    b = t()
+                    terms += [(lam, [0, b, b]), (neg, [0, b])]
+                else:
+                    x0, x1, y = t(), t(), t()
+                    terms += [(lam, [0, x0]), (lam, [0, x1]), (neg, [0, y])]
+        return tabs, terms
+
+    coins = [r.randrange(P) for _ in range(v)]
+    tabs, terms = problem(v)
+    obj_terms = [(c, [tabs[i] for i in fs]) for c, fs in terms]
+    best = None
+    for _ in range(4):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        proof = sc.prove_terms(obj_terms, lambda i: coins[i])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        best = dt if best is None or dt < best else best
+    ok, why = sc.verify_terms(proof, obj_terms, lambda i: coins[i])
+    table_bytes = len(tabs) * (8 << v)
+    res = {"tables": len(tabs), "terms": len(terms), "log2_size": v, "ms": best * 1e3,
+           "table_gb": table_bytes / 1e9, "verifier_accepts": bool(ok), "verifier_says": why}
+    del tabs, obj_terms, proof
+    if cpu:
+        from oracle import oracle as O
+        vs = 14
+        tabs, terms = problem(vs)
+        claim, polys, _, _ = gpu.prove_terms_gpu([(c, [tabs[i] for i in fs]) for c, fs in terms], lambda i: coins[i], P)
+        c0 = time.perf_counter()
+        want_claim, want_samples, _ = O.sumcheck_prove([x.cpu().numpy() for x in tabs], terms, coins)
+        dt = time.perf_counter() - c0
+        res["cpu_baseline"] = {"ms": dt * 1e3, "cores": O.num_threads(), "kind": "port",
+                               "sample": f"the same batch at 2^{vs}",
+                               "bit_exact_vs_gpu": bool(claim == want_claim and [[y for _, y in s] for s in polys] == want_samples)}
+    return res
+
+
 def bench_kquant(torch, steps=20, cpu=True):
     from verinf_amd.prover import kquant_cuda as kq
     nb = 4096 * 11008 // 256
@@ -512,7 +578,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
     ap.add_argument("--copy-probe", action="store_true")
     ap.add_argument("--ws-mb", type=int, default=0, help="override the LDE workspace size (MiB); 0 = library default")
-    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer", "hash"], default=None,
+    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer", "hash", "gatebatch"], default=None,
                     help="run just one of the extra legs and print its JSON (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -536,6 +602,9 @@ def main():
     if args.only == "hash":
         print(json.dumps(bench_hash(torch)))
         return
+    if args.only == "gatebatch":
+        print(json.dumps(bench_gate_batch(torch)))
+        return
 
     lde, msgs, out = bench_lde(torch, args.steps, args.warmup, args.ws_mb)
     cpu = cpu_baseline_lde(torch, msgs, out, args.cpu_rows, args.cpu_reps)
@@ -544,6 +613,8 @@ def main():
     extra = {}
     if not args.no_extra:
         extra["sumcheck_3x2^26_deg3"] = bench_sumcheck(torch)
+        torch.cuda.empty_cache()
+        extra["gate_batch_97_tables_2^22_deg3"] = bench_gate_batch(torch)
         torch.cuda.empty_cache()
         extra["kquant_q4k_4096x11008"] = bench_kquant(torch)
         torch.cuda.empty_cache()
