@@ -1,10 +1,12 @@
 // Batched Goldilocks NTT and coset low-degree extension for gfx950.
 //
-// One kernel, k_ntt_pass, runs every pass of the multi-pass transform described in
-// ntt_pass.hpp: gather a tile of T columns x L points into LDS, run the radix-2
-// levels of the length-L sub-transforms there, multiply by the inter-pass
-// twiddles precomputed in HBM and scatter.  The host side (ntt_plan.hpp) decides
-// the digit split, owns the cached tables and strings passes together into
+// A transform is one or more passes over digits of its length (ntt_pass.hpp): gather a tile of T columns x L points,
+// transform the L-point columns, multiply by the inter-pass twiddles precomputed in HBM and scatter.  Digits of
+// 32..256 points run in k_ntt_fast (two register-blocked 16 / 2..16-point transforms with one LDS crossing,
+// ntt_fast.hpp), 512 points in k_ntt_512, and the last inverse pass of an LDE together with the first forward pass in
+// k_lde_mid (the coefficients never leave the registers); k_ntt_pass, radix-2 levels in LDS, is left with digits
+// below 32 points.  The host side (ntt_plan.hpp) decides the digit split, owns the cached tables and strings
+// passes together into
 //   * vi_ntt_batched  -- in-place natural-order transform of (m, n) rows
 //     (prover/cuda_primitives.py:388-409);
 //   * vi_coset_lde    -- values at w_K^c -> codeword on shift*<w_N>
