@@ -205,7 +205,7 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
  *   tables        n_tables device tables of `size` = 2^v words (left untouched)
  *   work          n_tables device buffers of size/2 words (the folded tables live here)
  *   host_samples  VI_SC_HOST_WORDS (16) words of PINNED host memory (hipHostMalloc): words 0..7 receive each
- *                 round's samples and word 8 the count of rounds that have arrived; the host thread waits
+ *                 round's samples and word 8 a tag of the call and round that has arrived; the host thread waits
  *                 on that word (and queries the stream from time to time) rather than synchronising the stream
  *                 every round.  One buffer per proof in flight.
  *   out_samples   host, v * (deg+1) words: S_round(x) for x = 0..deg (no mask applied)

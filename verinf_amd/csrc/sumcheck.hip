@@ -1023,17 +1023,20 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
     lagrange_weights(ns, winv);
     hipStream_t s = (hipStream_t)stream;
     int64_t half = size / 2;
-    // host_samples[NSAMP] is the arrival word: round k's kernel stores k + 1 there behind its samples
+    // host_samples[NSAMP] is the arrival word: round k's kernel stores (call number << 32) + k + 1 there behind its
+    // samples, so that nothing an earlier call may have left in flight on this buffer can pass for a round of this one
+    static std::atomic<u64> calls{0};
+    const u64 tag = (calls.fetch_add(1) + 1) << 32;
     volatile u64 *arrived = host_samples + NSAMP;
     *arrived = 0;
     std::atomic_thread_fence(std::memory_order_seq_cst);
     rc = sumcheck_eval_on("vi_sumcheck_prove", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, host_samples,
-                          (u64 *)ws, 1, stream, split ? &groups : nullptr);
+                          (u64 *)ws, tag + 1, stream, split ? &groups : nullptr);
     if (rc) return rc;
     const uint64_t *const *src = tables;
     int round = 0;
     for (;;) {
-        rc = wait_for_samples(arrived, (u64)round + 1, s);
+        rc = wait_for_samples(arrived, tag + (u64)round + 1, s);
         if (rc) return rc;
         u64 y[NSAMP];
         for (int x = 0; x < ns; ++x) y[x] = out_samples[(size_t)round * ns + x] = ((const volatile u64 *)host_samples)[x];
@@ -1049,7 +1052,7 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
         if (half < 2) break;
         const uint64_t claim = interpolate_at(y, winv, ns, r);
         rc = fold_eval_on(src, work, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, &claim, host_samples, ws,
-                          ws_bytes, (u64)round + 1, stream, split ? &groups : nullptr);
+                          ws_bytes, tag + (u64)round + 1, stream, split ? &groups : nullptr);
         if (rc) return rc;
         src = work;
         half /= 2;

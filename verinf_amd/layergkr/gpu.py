@@ -393,7 +393,7 @@ _PINNED = threading.local()
 
 def _pinned_samples():
     """16 pinned host words (VI_SC_HOST_WORDS of the library header): the round kernels write their samples
-    into the first 8 and the count of rounds that have arrived into the ninth.  One buffer per host thread and
+    into the first 8 and a tag of the round that has arrived into the ninth.  One buffer per host thread and
     stream: a proof waits for each round's samples before it goes on, so a thread needs one per stream it drives, and
     two threads (or two streams) never see each other's samples."""
     bufs = getattr(_PINNED, "bufs", None)
