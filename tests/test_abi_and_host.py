@@ -57,6 +57,28 @@ def test_size_queries_and_argument_validation_without_a_device(L):
     assert L.vi_kquant_to_field(8, None, 1, 4096.0, None, None) == -1 and b"qtype" in L.vi_last_error()
     assert L.vi_gl_binop(0, None, None, None, 0, None) == 0
     assert L.vi_ntt_batched(None, 0, 16, 0, None, 0, None) == 0
+    # sumcheck term lists of any length are checked on the host: here 100 tables and 100 terms (beyond one kernel
+    # descriptor), with one defect each
+    n = 100
+    fake = (ctypes.c_void_p * n)(*[0x1000 + 8 * i for i in range(n)])             # never dereferenced
+    ws, out = ctypes.c_void_p(0x2000), ctypes.c_void_p(0x3000)
+    ws_bytes = L.vi_sumcheck_workspace_bytes()
+
+    def sc_eval(offsets, indices, tables=fake, n_tables=n, half=8):
+        off = (ctypes.c_int * len(offsets))(*offsets)
+        idx = (ctypes.c_int * max(len(indices), 1))(*indices)
+        co = (ctypes.c_uint64 * (len(offsets) - 1))(*([1] * (len(offsets) - 1)))
+        return L.vi_sumcheck_eval(tables, n_tables, half, off, idx, co, len(offsets) - 1, out, ws, ws_bytes, None)
+
+    good_off, good_idx = list(range(0, 2 * n + 1, 2)), [j % n for j in range(2 * n)]
+    assert sc_eval(good_off, good_idx[:-1] + [n]) == -1 and b"factor index" in L.vi_last_error()
+    assert sc_eval(good_off[:-1] + [2 * n + 7], good_idx + [0] * 7) == -1 and b"factors" in L.vi_last_error()
+    assert sc_eval([1] + good_off[1:], good_idx) == -1 and b"term_off" in L.vi_last_error()
+    assert sc_eval(good_off, good_idx, half=0) == -1 and b"half" in L.vi_last_error()
+    holed = (ctypes.c_void_p * n)(*[0 if i == 57 else 0x1000 + 8 * i for i in range(n)])
+    assert sc_eval(good_off, good_idx, tables=holed) == -1 and b"null table 57" in L.vi_last_error()
+    assert L.vi_sumcheck_eval_static(fake, n, 8, (ctypes.c_int * (n + 1))(*good_off), (ctypes.c_int * (2 * n))(*good_idx),
+                                     (ctypes.c_uint64 * n)(*([1] * n)), n, out, None) != 0
 
 
 def test_missing_library_fails_loudly(monkeypatch):
