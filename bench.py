@@ -568,6 +568,50 @@ def copy_probe(torch):
     print(json.dumps({"copy_probe_bytes_read": 1 << 30, "copy_probe_bytes_written": 1 << 30, "launches": 5}))
 
 
+def valu_probe(torch, iters=400, reps=3):
+    """Issue rate of each integer VALU instruction class on the whole chip (vi_valu_probe): wave-instructions per
+    second from HIP events around the launch, the shader clock during the loop from the two counters the kernel
+    reads, and from both the cycles a SIMD spends per instruction."""
+    import ctypes
+    from verinf_amd import _lib
+    L = _lib.lib()
+    props = torch.cuda.get_device_properties(0)
+    cus = props.multi_processor_count
+    blocks = cus * 8                                   # 8 wavefronts on every SIMD
+    out = torch.empty(blocks * 256, dtype=torch.int64, device="cuda")
+    clocks = torch.zeros(blocks * 4, dtype=torch.int64, device="cuda")
+    wall_khz = L.vi_wall_clock_khz()
+    rows = []
+    for kind in range(L.vi_valu_probe_count()):
+        n = ctypes.c_int64(0)
+        best_ms, mhz = None, None
+        for rep in range(reps + 1):
+            s, e = _events(torch)
+            s.record()
+            _lib.check(L.vi_valu_probe(kind, 20 if rep == 0 else iters, blocks, out.data_ptr(), clocks.data_ptr(),
+                                       ctypes.byref(n), _lib.stream_ptr()))
+            e.record()
+            torch.cuda.synchronize()
+            if rep == 0:
+                continue
+            ms = s.elapsed_time(e)
+            if best_ms is None or ms < best_ms:
+                best_ms = ms
+                c = clocks.view(-1, 4).cpu()
+                ticks, ref = (c[:, 1] - c[:, 0]).double(), (c[:, 3] - c[:, 2]).double()
+                mhz = float((ticks / ref).median()) * wall_khz / 1e3 if wall_khz else None
+        rate = n.value / (best_ms * 1e-3)
+        row = {"instruction": L.vi_valu_probe_name(kind).decode(), "ms": best_ms, "wave_instr_per_s": rate,
+               "counter_ratio_mhz": mhz}
+        if mhz:
+            row["simd_cycles_per_instr"] = cus * 4 * mhz * 1e6 / rate
+        rows.append(row)
+    return {"device": props.name, "compute_units": cus, "simds": cus * 4, "wavefronts_per_simd": 8, "iters": iters,
+            "wall_clock_khz": wall_khz, "rows": rows,
+            "note": "counter_ratio_mhz = (shader-clock ticks / constant-rate ticks) x the constant counter's rate, median "
+                    "over workgroups; if the two counters tick at one rate on this part it reads that rate, not the clock"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -577,6 +621,7 @@ def main():
     ap.add_argument("--cpu-reps", type=int, default=5, help="passes of the CPU baseline over its sample")
     ap.add_argument("--no-extra", action="store_true", help="skip the sumcheck / K-quant legs")
     ap.add_argument("--copy-probe", action="store_true")
+    ap.add_argument("--valu-probe", action="store_true", help="issue rate of the integer VALU instruction classes")
     ap.add_argument("--ws-mb", type=int, default=0, help="override the LDE workspace size (MiB); 0 = library default")
     ap.add_argument("--only", choices=["sumcheck", "kquant", "layer", "hash", "gatebatch"], default=None,
                     help="run just one of the extra legs and print its JSON (for profiling)")
@@ -589,6 +634,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     if args.copy_probe:
         copy_probe(torch)
+        return
+    if args.valu_probe:
+        print(json.dumps(valu_probe(torch)))
         return
     if args.only == "sumcheck":
         print(json.dumps(bench_sumcheck(torch)))

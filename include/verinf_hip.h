@@ -204,19 +204,39 @@ int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int 
  * and returns 0, or non-zero to abort (the call then returns VI_EINVAL).
  *   tables        n_tables device tables of `size` = 2^v words (left untouched)
  *   work          n_tables device buffers of size/2 words (the folded tables live here)
- *   host_samples  VI_SC_HOST_WORDS (16) words of PINNED host memory (hipHostMalloc): words 0..7 receive each
- *                 round's samples and word 8 a tag of the call and round that has arrived; the host thread waits
+ *   host_samples  host_words >= VI_SC_HOST_WORDS (16) words of PINNED host memory (hipHostMalloc): words 0..7 receive
+ *                 each round's samples and word 8 a tag of the call and round that has arrived; the host thread waits
  *                 on that word (and queries the stream from time to time) rather than synchronising the stream
- *                 every round.  One buffer per proof in flight.
+ *                 every round.  One buffer per proof in flight.  A smaller host_words is rejected (VI_EINVAL).
  *   out_samples   host, v * (deg+1) words: S_round(x) for x = 0..deg (no mask applied)
  *   out_challenges host, v words: the challenges, reduced mod p
- * The final fold (after the last round) is not performed, as nothing reads it. */
+ * The final fold (after the last round) is not performed, as nothing reads it.  The call returns, also with an
+ * error, only after every kernel it has queued has retired.  Use it when the coin needs a round's samples; the
+ * reference's own coin takes the round number alone, which vi_sumcheck_prove_coins serves without host waits. */
 #define VI_SC_HOST_WORDS 16
 typedef int (*vi_coin_fn)(int round, const uint64_t *samples, int n_samples, uint64_t *challenge, void *user);
 int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
                       const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
-                      vi_coin_fn coin, void *user, uint64_t *host_samples, uint64_t *out_samples,
+                      vi_coin_fn coin, void *user, uint64_t *host_samples, size_t host_words, uint64_t *out_samples,
                       uint64_t *out_challenges, void *ws, size_t ws_bytes, void *stream);
+
+/* The same proof with every challenge known up front, which is what the reference's interface provides: its prover
+ * calls `coin(rnd)` with the round number only (layergkr/gpu.py:403, layergkr/sumcheck.py:217) and its callers draw
+ * the coins before the proof starts (layergkr/full_layer.py:222-224, layergkr/relations.py:122-123,
+ * layergkr/layer.py:123-125).  All rounds are queued on the stream without a host round trip, and the call returns
+ * without waiting.  A single product of up to four distinct tables and the hadamard gate batch eq * (a * b + c' * c)
+ * run three rounds per pass over the tables and every round of the last few thousand entries in one workgroup; other
+ * sums keep one launch per round.
+ *   challenges    host, v = log2(size) words (reduced mod p by the callee)
+ *   samples       v rows of 8 words the GPU can write (device memory or pinned host memory): S_round(x) at
+ *                 samples[8 * round + x], x = 0..deg, complete once the stream has reached the end of the call's work
+ *   work          n_tables device buffers of size/2 words; tables are left untouched
+ *   ws            vi_sumcheck_prove_coins_workspace_bytes(size) bytes of device scratch
+ * At most 40 rounds. */
+size_t vi_sumcheck_prove_coins_workspace_bytes(int64_t size);
+int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                            const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                            const uint64_t *challenges, uint64_t *samples, void *ws, size_t ws_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * BLAKE3 column digests and Merkle levels of a committed codeword matrix.
@@ -302,6 +322,21 @@ int vi_gl_spmv(const uint64_t *values, const uint64_t *col_idx, const uint64_t *
                const uint64_t *x, const uint8_t *seed, const uint8_t *label, int label_len, uint64_t *y, void *stream);
 int vi_lookup_multiplicities(const uint64_t *x, int64_t n_x, const uint64_t *table, int64_t n_table, int table_is_range,
                              uint64_t *mult, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Measurement hook (no counterpart in the reference): the issue rate of the integer VALU instructions the field
+ * arithmetic and the hashing consist of, which is the bound their kernels are put against.
+ * vi_valu_probe launches `blocks` workgroups of 256 threads that each run `iters` times a block of one instruction
+ * class (kind < vi_valu_probe_count(), named by vi_valu_probe_name) on independent registers; the caller times the
+ * launch.  *wave_instructions receives the VALU instructions issued, counted per wavefront.  out: blocks * 256
+ * words, clocks: blocks * 4 words of device memory; clocks[4b .. 4b+3] = the shader-clock counter at the start and
+ * the end of workgroup b, then the constant-rate counter (vi_wall_clock_khz() ticks per millisecond) at the same
+ * two moments: their ratio is the clock the SIMDs ran at. */
+int vi_valu_probe_count(void);
+const char *vi_valu_probe_name(int kind);
+int vi_wall_clock_khz(void);
+int vi_valu_probe(int kind, int iters, int blocks, uint64_t *out, uint64_t *clocks, int64_t *wave_instructions,
+                  void *stream);
 
 #ifdef __cplusplus
 }

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol(L):
     raw = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(raw, n), n
-    assert L.vi_version() == b"0.1"
+    assert L.vi_version() == b"0.2"
 
 
 def test_size_queries_and_argument_validation_without_a_device(L):

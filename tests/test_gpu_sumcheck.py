@@ -43,6 +43,16 @@ def _check(gpu, tables_np, terms_idx, seed, as_tensor):
     if as_tensor:
         for t, o in zip(tables_np, objs):
             assert np.array_equal(to_np(o), t), "caller's tensor was modified"
+    if v <= 13:
+        # the loop that hands every round's samples to the coin (one launch and one host wait per round)
+        seen = []
+
+        def coin_with_samples(i, samples):
+            seen.append(samples)
+            return coins[i]
+
+        assert gpu.prove_terms_gpu_interactive(terms, coin_with_samples, P) == (claim, polys, chals, mu)
+        assert seen == polys
 
 
 def test_sumcheck_golden(mods, golden_dir):
@@ -305,13 +315,47 @@ def test_tables_with_words_at_or_above_p_are_taken_as_residues(mods, v, nt, term
     for j, t in enumerate(raw):
         for pos, word in ((0, P), (1, P + 1), (t.size - 1, (1 << 64) - 1), (t.size // 2, P + 12345), (t.size // 2 + 1, P)):
             t[(pos + j) % t.size] = np.uint64(word)
+        # a word at or above p in the lower half opposite a tiny one in the upper half: hi - lo borrows twice unless
+        # lo is reduced first
+        h = t.size // 2
+        if h >= 4:
+            for pos, lo, hi in ((2, (1 << 64) - 1, 0), (3, P + 1, 0)):
+                t[(pos + j) % h] = np.uint64(lo)
+                t[h + (pos + j) % h] = np.uint64(hi)
     residues = [np.array([int(x) % P for x in t], dtype=np.uint64) for t in raw]
     coins, coin = _coins(v, 77)
     objs = [to_dev(t) for t in raw]
-    claim, polys, chals, _ = gpu.prove_terms_gpu([(c, [objs[i] for i in fs]) for c, fs in terms], coin, P)
+    obj_terms = [(c, [objs[i] for i in fs]) for c, fs in terms]
+    claim, polys, chals, _ = gpu.prove_terms_gpu(obj_terms, coin, P)
     want_claim, want_samples, _ = O.sumcheck_prove(residues, terms, coins)
     assert claim == want_claim
     assert [[y for _, y in s] for s in polys] == want_samples
+    assert gpu.prove_terms_gpu_interactive(obj_terms, lambda i, _s: coins[i], P)[:2] == (claim, polys)
+
+
+def test_fold_of_words_at_or_above_p_c_abi(mods):
+    """vi_sumcheck_fold_eval on caller words: (lo, hi) = (2^64 - 1, 0) and (p + 1, 0) fold like their residues, for
+    few tables (register kernel) and for many (the many-table fold)."""
+    import ctypes
+    from verinf_amd import _lib
+    L = _lib.lib()
+    r = 0x0123456789ABCDEF % P
+    for n in (2, 12):
+        tabs = [rand_field(1 << 8, 950 + j) for j in range(n)]
+        raw = [t.copy() for t in tabs]
+        for j, t in enumerate(raw):
+            t[j], t[128 + j] = np.uint64((1 << 64) - 1), np.uint64(0)
+            t[20 + j], t[148 + j] = np.uint64(P + 1), np.uint64(0)
+            t[40 + j], t[168 + j] = np.uint64(5), np.uint64((1 << 64) - 2)
+        residues = [np.array([int(x) % P for x in t], dtype=np.uint64) for t in raw]
+        dev = [to_dev(t) for t in raw]
+        dst = [torch.empty(128, dtype=torch.uint64, device="cuda") for _ in raw]
+        src_p = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dev])
+        dst_p = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dst])
+        _lib.check(L.vi_sumcheck_fold_eval(src_p, dst_p, n, 128, r, None, None, None, 0, None, None, None, 0,
+                                           _lib.stream_ptr()))
+        for d, t in zip(dst, residues):
+            assert np.array_equal(to_np(d), O.fold(t, r))
 
 
 def test_tables_that_are_views_at_an_odd_word_offset(mods):
@@ -456,26 +500,100 @@ def test_verifier_accepts_and_rejects_device_table_proofs(mods):
 
 
 def test_baseline_shape_three_tables_of_2p26(mods):
-    """The benchmark instance at full size (three tables of 2^26, degree 3, 26 rounds), through the
-    properties that do not need a CPU run: the claim is the sum of the elementwise product, every
-    round satisfies S(0) + S(1) = previous claim, and the last claim equals the product of the three
-    multilinear extensions at the challenge point (all checked by the verifier, the terminal values
-    on the device); a tampered table is rejected."""
+    """The benchmark instance at full size (three tables of 2^26 uniform field elements, degree 3, 26 rounds):
+    the claim and every round's samples against the C oracle on the same tables, then the properties -- the claim
+    is the sum of the elementwise product, every round satisfies S(0) + S(1) = previous claim, and the last claim
+    equals the product of the three multilinear extensions at the challenge point (all checked by the verifier,
+    the terminal values on the device); a tampered table is rejected."""
     gpu, sc = mods
+    from tests.gpu_util import rand_field_dev
     v = 26
-    g = torch.Generator(device="cuda").manual_seed(26)
-    tabs = [torch.randint(0, 1 << 62, (1 << v,), generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
-            for _ in range(3)]
-    coins = [random.Random(5).randrange(P) for _ in range(v)]
+    tabs = [rand_field_dev((1 << v,), 260 + j) for j in range(3)]
+    rnd = random.Random(5)
+    coins = [rnd.randrange(P) for _ in range(v)]
     terms = [(1, tabs)]
     proof = sc.prove_terms(terms, lambda i: coins[i])
     assert len(proof.round_polys) == v and all(len(s) == 4 for s in proof.round_polys)
+    want_claim, want_samples, _ = O.sumcheck_prove([t.cpu().numpy() for t in tabs], [(1, [0, 1, 2])], coins)
+    assert proof.claim == want_claim
+    assert [[y for _, y in s] for s in proof.round_polys] == want_samples
     assert proof.claim == int(gpu.gl_sum(cp_mul(cp_mul(tabs[0], tabs[1]), tabs[2])).cpu().item())
     ok, why = sc.verify_terms(proof, terms, lambda i: coins[i])
     assert ok, why
     tabs[1].view(torch.int64)[(1 << v) - 3] += 1
     ok, why = sc.verify_terms(proof, terms, lambda i: coins[i])
     assert not ok and "terminal" in why
+
+
+def test_coins_and_masks_drawn_up_front_match_the_interactive_loop(mods):
+    """prove_terms_gpu calls mask and coin for all rounds before the first launch, in the reference's order
+    (mask, coin, mask, coin, ...): with a coin and a mask tape that share one random.Random -- so that any other
+    call order would draw other values -- it returns what the round-by-round loop returns, for a shape with its
+    own multi-round kernels and for a general sum."""
+    gpu, sc = mods
+    for v, nt, terms_idx in ((14, 3, [(7, [0, 1, 2])]), (13, 4, [(3, [0, 1, 2]), (P - 5, [0, 3])]),
+                            (9, 6, [(3, [0, 1]), (P - 5, [2]), (7, [3]), (11, [4, 5, 0])]), (1, 2, [(1, [0, 1])])):
+        tabs = [to_dev(rand_field(1 << v, 1200 + j)) for j in range(nt)]
+        terms = [(c, [tabs[i] for i in fs]) for c, fs in terms_idx]
+        deg = max(len(fs) for _, fs in terms_idx)
+
+        def run(prover, wrap):
+            shared = random.Random(77)
+            calls = []
+
+            def coin(i):
+                calls.append(("coin", i))
+                return shared.randrange(1 << 64)
+
+            def mask(d, mu):
+                calls.append(("mask", mu))
+                assert d == deg
+                return sc.mask_poly_coeffs(mu, [shared.randrange(P) for _ in range(d)])
+
+            return prover(terms, wrap(coin), P, mask=mask, mu0=31337), calls
+
+        up_front, calls_a = run(gpu.prove_terms_gpu, lambda c: c)
+        looped, calls_b = run(gpu.prove_terms_gpu_interactive, lambda c: (lambda i, _samples: c(i)))
+        assert up_front == looped
+        assert calls_a == calls_b and [k for k, _ in calls_a] == ["mask", "coin"] * v
+        # and the masked proof verifies: S(0) + S(1) of every round is the previous round's value at its challenge
+        claim, polys, chals, mu = up_front
+        cur = claim
+        for s, r in zip(polys, chals):
+            ys = [y for _, y in s]
+            assert (ys[0] + ys[1]) % P == cur
+            cur = _lagrange_at(ys, r)
+        assert cur == (_terminal(tabs, terms_idx, chals) + mu) % P
+
+
+def _terminal(tabs, terms_idx, chals):
+    """sum_k c_k prod_j f_j(r): the tables folded on the host in Python integers"""
+    vals = []
+    for t in tabs:
+        f = [int(x) for x in to_np(t)]
+        for r in chals:
+            h = len(f) // 2
+            f = [(f[i] + r * (f[h + i] - f[i])) % P for i in range(h)]
+        vals.append(f[0])
+    total = 0
+    for c, fs in terms_idx:
+        prod = c
+        for i in fs:
+            prod = prod * vals[i] % P
+        total += prod
+    return total % P
+
+
+def _lagrange_at(ys, r):
+    n, total = len(ys), 0
+    for i, y in enumerate(ys):
+        num, den = y, 1
+        for k in range(n):
+            if k != i:
+                num = num * (r - k) % P
+                den = den * (i - k) % P
+        total += num * pow(den, P - 2, P)
+    return total % P
 
 
 def cp_mul(x, y):

@@ -12,4 +12,4 @@ Layout mirrors the reference modules this package stands in for:
 Everything computes through libverinf_hip.so (hand-written HIP, C ABI in
 include/verinf_hip.h); there is no CPU fallback.
 """
-__version__ = "0.1"
+__version__ = "0.2"

@@ -27,11 +27,12 @@ EXPORTS = [
     "vi_kquant_to_field",
     "vi_kquant_to_field_transposed",
     "vi_sumcheck_workspace_bytes", "vi_sumcheck_eval", "vi_sumcheck_eval_static", "vi_sumcheck_fold_eval",
-    "vi_sumcheck_prove",
+    "vi_sumcheck_prove", "vi_sumcheck_prove_coins_workspace_bytes", "vi_sumcheck_prove_coins",
     "vi_hash_columns_workspace_bytes", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
     "vi_merkle_level", "vi_merkle_tree_nodes", "vi_merkle_tree", "vi_row_prg",
     "vi_eq_vector", "vi_mle_eval_workspace_bytes", "vi_mle_eval",
     "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities",
+    "vi_valu_probe_count", "vi_valu_probe_name", "vi_wall_clock_khz", "vi_valu_probe",
 ]
 
 COIN_FN = ctypes.CFUNCTYPE(c_int, c_int, POINTER(c_uint64), c_int, POINTER(c_uint64), c_void_p)
@@ -91,8 +92,13 @@ def lib():
     L.vi_sumcheck_fold_eval.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, u64, ip, ip,
                                         POINTER(u64), c_int, POINTER(u64), vp, vp, sz, vp]
     L.vi_sumcheck_prove.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int,
-                                    COIN_FN, vp, vp, POINTER(u64), POINTER(u64), vp, sz, vp]
+                                    COIN_FN, vp, vp, sz, POINTER(u64), POINTER(u64), vp, sz, vp]
     L.vi_sumcheck_prove.restype = c_int
+    L.vi_sumcheck_prove_coins_workspace_bytes.restype = sz
+    L.vi_sumcheck_prove_coins_workspace_bytes.argtypes = [i64]
+    L.vi_sumcheck_prove_coins.argtypes = [POINTER(vp), POINTER(vp), c_int, i64, ip, ip, POINTER(u64), c_int,
+                                          POINTER(u64), vp, vp, sz, vp]
+    L.vi_sumcheck_prove_coins.restype = c_int
     L.vi_hash_columns_workspace_bytes.restype = sz
     L.vi_hash_columns_workspace_bytes.argtypes = [i64, i64]
     L.vi_hash_columns.argtypes = [vp, i64, i64, i64, vp, vp, sz, vp]
@@ -110,6 +116,9 @@ def lib():
     L.vi_mle_eval_workspace_bytes.restype = sz
     L.vi_mle_eval_workspace_bytes.argtypes = [i64]
     L.vi_mle_eval.argtypes = [vp, i64, i64, POINTER(u64), c_int, vp, vp, sz, vp]
+    L.vi_valu_probe_name.restype = c_char_p
+    L.vi_valu_probe_name.argtypes = [c_int]
+    L.vi_valu_probe.argtypes = [c_int, c_int, c_int, vp, vp, POINTER(i64), vp]
     for name in EXPORTS:
         getattr(L, name)                     # AttributeError here = stale build
     for name in ("vi_gl_binop", "vi_gl_binop_bcast", "vi_gl_unop", "vi_gl_axpy", "vi_gl_probe", "vi_gl_sum",
@@ -117,7 +126,7 @@ def lib():
                  "vi_ntt_batched", "vi_coset_lde", "vi_coset_lde_coeffs", "vi_coset_extend", "vi_kquant_to_field", "vi_kquant_to_field_transposed", "vi_sumcheck_eval", "vi_sumcheck_eval_static",
                  "vi_sumcheck_fold_eval", "vi_hash_columns", "vi_hash_columns_update", "vi_hash_columns_finalize",
                  "vi_merkle_level", "vi_merkle_tree_nodes", "vi_merkle_tree", "vi_row_prg", "vi_eq_vector", "vi_mle_eval",
-                 "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities"):
+                 "vi_challenge", "vi_gl_spmv", "vi_lookup_multiplicities", "vi_valu_probe"):
         getattr(L, name).restype = c_int
     _lib = L
     return L

@@ -11,7 +11,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["field_ops.hip", "linalg.hip", "ntt.hip", "kquant.hip", "sumcheck.hip", "blake3.hip", "mle.hip"]
+SOURCES = ["field_ops.hip", "linalg.hip", "ntt.hip", "kquant.hip", "sumcheck.hip", "blake3.hip", "mle.hip", "valu_probe.hip"]
 LIB = os.path.join(HERE, "libverinf_hip.so")
 
 # -ffp-contract=off: the K-quant decode must round every fp32 operation separately.

@@ -180,7 +180,7 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 extern "C" {
 
 const char *vi_last_error(void) { return vi::err_buf(); }
-const char *vi_version(void) { return "0.1"; }
+const char *vi_version(void) { return "0.2"; }
 
 int vi_gl_binop(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream) {
     if (op < 0 || op > 2) return vi::fail(VI_EINVAL, "vi_gl_binop: op %d", op);

@@ -58,6 +58,8 @@ struct Desc {
     int gate;                               // four tables [common, f0, f1, lin]: common * (f0 * f1 + lin_coeff[0] * lin)
     int skip1;                              // S(1) is not summed: it is claim - S(0) (the round's known total)
     u64 claim;                              // S(0) + S(1) when skip1
+    int canon_src;                          // the fold reads caller data: words are reduced mod p on load (sub() and the
+                                            // ladders want canonical operands); 0 for tables this library has folded
 };
 
 __device__ __forceinline__ u64 fold1(u64 lo, u64 hi, u64 r) { return gl::add(lo, gl::mul(r, gl::sub(hi, lo))); }
@@ -124,10 +126,13 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
                     lo_u[u][t] = gl::canon(f[i]);
                     hi_u[u][t] = gl::canon(f[half + i]);
                 } else if (MODE == 1) {
-                    D.dst[t][i] = fold1(f[i], f[half + i], r);
+                    u64 a0 = f[i], b0 = f[half + i];
+                    if (D.canon_src) { a0 = gl::canon(a0); b0 = gl::canon(b0); }
+                    D.dst[t][i] = fold1(a0, b0, r);
                 } else {
                     const i64 h2 = half >> 1;
                     u64 a0 = f[i], a1 = f[i + h2], b0 = f[half + i], b1 = f[half + i + h2];
+                    if (D.canon_src) { a0 = gl::canon(a0); a1 = gl::canon(a1); b0 = gl::canon(b0); b1 = gl::canon(b1); }
                     lo_u[u][t] = fold1(a0, b0, r);
                     hi_u[u][t] = fold1(a1, b1, r);
                     D.dst[t][i] = lo_u[u][t];
@@ -402,18 +407,24 @@ struct FoldDesc {
     const u64 *src[FOLD_MANY];
     u64 *dst[FOLD_MANY];
 };
-__global__ __launch_bounds__(BLOCK) void k_fold_many(const FoldDesc F, i64 half, u64 r) {
+// canon_src: the tables are caller data, reduced mod p on load (the kernel is bound by memory either way)
+__global__ __launch_bounds__(BLOCK) void k_fold_many(const FoldDesc F, i64 half, u64 r, int canon_src) {
     const u64 *src = F.src[blockIdx.y];
     u64 *dst = F.dst[blockIdx.y];
     const i64 stride = (i64)gridDim.x * BLOCK;
     i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x;
     for (; i + stride < half; i += 2 * stride) {         // two independent indices in flight
-        const u64 lo0 = src[i], hi0 = src[half + i];
-        const u64 lo1 = src[i + stride], hi1 = src[half + i + stride];
+        u64 lo0 = src[i], hi0 = src[half + i];
+        u64 lo1 = src[i + stride], hi1 = src[half + i + stride];
+        if (canon_src) { lo0 = gl::canon(lo0); hi0 = gl::canon(hi0); lo1 = gl::canon(lo1); hi1 = gl::canon(hi1); }
         dst[i] = fold1(lo0, hi0, r);
         dst[i + stride] = fold1(lo1, hi1, r);
     }
-    if (i < half) dst[i] = fold1(src[i], src[half + i], r);
+    if (i < half) {
+        u64 lo0 = src[i], hi0 = src[half + i];
+        if (canon_src) { lo0 = gl::canon(lo0); hi0 = gl::canon(hi0); }
+        dst[i] = fold1(lo0, hi0, r);
+    }
 }
 
 // cross-block tree: one workgroup adds the per-block partials of every sample
@@ -515,6 +526,7 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
     D.gate = 0;
     D.skip1 = 0;
     D.claim = 0;
+    D.canon_src = 1;
     if (!need_terms) return VI_OK;
     if (n_terms < 1 || n_terms > VI_SC_MAX_TERMS) return vi::fail(VI_EINVAL, "%s: n_terms = %d (1..%d)", who, n_terms, VI_SC_MAX_TERMS);
     if (!term_off || !factor_idx || !coeffs) return vi::fail(VI_EINVAL, "%s: null term descriptor", who);
@@ -660,7 +672,7 @@ int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 s
 }
 
 // fold `n` tables by r: up to REG_TABLES through the register kernel, more through k_fold_many (FOLD_MANY per launch)
-int fold_tables(const uint64_t *const *src, uint64_t *const *dst, int n, i64 half, u64 r, hipStream_t s) {
+int fold_tables(const uint64_t *const *src, uint64_t *const *dst, int n, i64 half, u64 r, hipStream_t s, int canon_src = 1) {
     for (int t = 0; t < n; ++t)
         if (!src[t] || !dst[t]) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null table %d", t);
     int nbx = blocks_for((half + 1) / 2);
@@ -674,7 +686,7 @@ int fold_tables(const uint64_t *const *src, uint64_t *const *dst, int n, i64 hal
         // a few thousand workgroups fill the chip; beyond that a workgroup takes more indices
         int bx = nbx;
         while (bx > 1 && (i64)bx * cnt > 8192) bx = (bx + 1) / 2;
-        hipLaunchKernelGGL(k_fold_many, dim3(bx, cnt), dim3(BLOCK), 0, s, F, half, r);
+        hipLaunchKernelGGL(k_fold_many, dim3(bx, cnt), dim3(BLOCK), 0, s, F, half, r, canon_src);
         VI_LAUNCH_CHECK("sumcheck fold (many tables)");
     }
     return VI_OK;
@@ -755,9 +767,10 @@ void split_terms(int n_tables, const int *term_off, const int *factor_idx, const
     }
 }
 
-// samples of sum over all groups at x = 0..deg from `tables` (pairs (i, half + i)); partial: MAX_BLOCKS * NSAMP words
+// samples of sum over all groups at x = 0..deg from `tables` (pairs (i, half + i)); partial: MAX_BLOCKS * NSAMP words.
+// nb_out != NULL: the per-workgroup sums are left in `partial` (*nb_out rows) for a later kernel to add up.
 int eval_groups(const char *who, const uint64_t *const *tables, const std::vector<TermGroup> &groups, int deg, i64 half,
-                u64 *partial, u64 *out_samples, u64 flag, hipStream_t s) {
+                u64 *partial, u64 *out_samples, u64 flag, hipStream_t s, int *nb_out = nullptr) {
     int nb = 0;
     for (size_t g = 0; g < groups.size(); ++g) {
         const TermGroup &G = groups[g];
@@ -770,6 +783,10 @@ int eval_groups(const char *who, const uint64_t *const *tables, const std::vecto
         D.deg = deg;                        // every group yields all the samples of the whole sum
         nb = launch_eval_mem(D, half, partial, g > 0 ? 1 : 0, D.out_scale, s);    // the same grid for every group
         VI_LAUNCH_CHECK("sumcheck eval (term group)");
+    }
+    if (nb_out) {
+        *nb_out = nb;
+        return VI_OK;
     }
     hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)partial, nb, deg, (u64)1, 0, (u64)0, out_samples, flag);
     VI_LAUNCH_CHECK("sumcheck final");
@@ -873,7 +890,7 @@ namespace {
 int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables, int64_t half, uint64_t r,
                  const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, const uint64_t *claim,
                  uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream,
-                 const std::vector<TermGroup> *groups = nullptr);
+                 const std::vector<TermGroup> *groups = nullptr, int canon_src = 1);
 }
 
 int vi_sumcheck_fold_eval(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
@@ -889,14 +906,14 @@ namespace {
 int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables, int64_t half, uint64_t r,
                  const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, const uint64_t *claim,
                  uint64_t *out_samples, void *ws, size_t ws_bytes, u64 flag, void *stream,
-                 const std::vector<TermGroup> *groups) {
+                 const std::vector<TermGroup> *groups, int canon_src) {
     const bool eval = out_samples != nullptr;
     Desc D;
     if (!dst) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: null dst");
     if (!eval && src && n_tables > REG_TABLES) {
         // folding alone has no limit on the number of tables
         if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: half = %lld", (long long)half);
-        return fold_tables(src, dst, n_tables, half, r % gl::P, (hipStream_t)stream);
+        return fold_tables(src, dst, n_tables, half, r % gl::P, (hipStream_t)stream, canon_src);
     }
     if (eval && src && n_terms >= 1 && term_off && !fits_one_desc(n_tables, term_off, n_terms)) {
         // more than one descriptor holds: fold every table, then evaluate the folded tables group by group
@@ -906,7 +923,8 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
         if (rc) return rc;
         if (half < 2) return vi::fail(VI_EINVAL, "%s: no next round after half = %lld; pass out_samples = NULL", who, (long long)half);
         if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "%s: workspace below %zu bytes", who, vi_sumcheck_workspace_bytes());
-        rc = vi_sumcheck_fold_eval(src, dst, n_tables, half, r, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, stream);
+        rc = fold_eval_on(src, dst, n_tables, half, r, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, 0, 0, stream,
+                          nullptr, canon_src);
         if (rc) return rc;
         std::vector<TermGroup> mine;
         if (!groups) {
@@ -918,6 +936,7 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
     }
     int rc = fill_desc(D, src, dst, n_tables, term_off, factor_idx, coeffs, n_terms, eval, "vi_sumcheck_fold_eval");
     if (rc) return rc;
+    D.canon_src = canon_src;
     if (half < 1) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: half = %lld", (long long)half);
     if (eval && half < 2) return vi::fail(VI_EINVAL, "vi_sumcheck_fold_eval: no next round after half = 1; pass out_samples = NULL");
     if (eval && (!ws || ws_bytes < vi_sumcheck_workspace_bytes())) return vi::fail(VI_ENOMEM, "vi_sumcheck_fold_eval: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
@@ -944,7 +963,7 @@ int fold_eval_on(const uint64_t *const *src, uint64_t *const *dst, int n_tables,
         nb = launch_round<2>(D, half, r, (u64 *)ws, blocks_for(half >> 1), nullptr, 1, 0, 0, s);
         VI_LAUNCH_CHECK("sumcheck fold+eval");
     } else {
-        rc = fold_tables(src, dst, n_tables, half, r, s);
+        rc = fold_tables(src, dst, n_tables, half, r, s, canon_src);
         if (rc) return rc;
         Desc E = D;
         for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
@@ -1004,10 +1023,11 @@ int wait_for_samples(const volatile u64 *flag, u64 seq, hipStream_t s) {
 
 int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
                       const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
-                      vi_coin_fn coin, void *user, uint64_t *host_samples, uint64_t *out_samples,
+                      vi_coin_fn coin, void *user, uint64_t *host_samples, size_t host_words, uint64_t *out_samples,
                       uint64_t *out_challenges, void *ws, size_t ws_bytes, void *stream) {
     if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: size must be a power of two >= 2, got %lld", (long long)size);
     if (!coin || !host_samples || !out_samples || !out_challenges || !work) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: null pointer");
+    if (host_words < VI_SC_HOST_WORDS) return vi::fail(VI_EINVAL, "vi_sumcheck_prove: host_samples holds %zu words, %d are needed", host_words, VI_SC_HOST_WORDS);
     if (!ws || ws_bytes < vi_sumcheck_workspace_bytes()) return vi::fail(VI_ENOMEM, "vi_sumcheck_prove: workspace below %zu bytes", vi_sumcheck_workspace_bytes());
     int deg = 0;
     int rc = check_terms("vi_sumcheck_prove", tables, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
@@ -1032,33 +1052,159 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
     std::atomic_thread_fence(std::memory_order_seq_cst);
     rc = sumcheck_eval_on("vi_sumcheck_prove", tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, host_samples,
                           (u64 *)ws, tag + 1, stream, split ? &groups : nullptr);
-    if (rc) return rc;
+    if (rc) return rc;                       // nothing has been queued
+    // From here on kernels may be in flight that write host_samples, work[] and ws: every error exit waits for
+    // them to retire first, so that the caller may release those buffers as soon as the call has returned.
     const uint64_t *const *src = tables;
     int round = 0;
     for (;;) {
         rc = wait_for_samples(arrived, tag + (u64)round + 1, s);
-        if (rc) return rc;
+        if (rc) break;
         u64 y[NSAMP];
         for (int x = 0; x < ns; ++x) y[x] = out_samples[(size_t)round * ns + x] = ((const volatile u64 *)host_samples)[x];
         uint64_t r = 0;
-        int stop = coin(round, y, ns, &r, user);
-        if (stop) {
-            (void)hipStreamSynchronize(s);     // the last kernel retires before the caller releases its buffers
-            return vi::fail(VI_EINVAL, "vi_sumcheck_prove: coin callback asked to stop in round %d", round);
+        if (coin(round, y, ns, &r, user)) {
+            rc = vi::fail(VI_EINVAL, "vi_sumcheck_prove: coin callback asked to stop in round %d", round);
+            break;
         }
         r %= gl::P;
         out_challenges[round] = r;
         ++round;
         if (half < 2) break;
         const uint64_t claim = interpolate_at(y, winv, ns, r);
+        // only the first fold reads the caller's words; the work buffers hold canonical values
         rc = fold_eval_on(src, work, n_tables, half, r, term_off, factor_idx, coeffs, n_terms, &claim, host_samples, ws,
-                          ws_bytes, tag + (u64)round + 1, stream, split ? &groups : nullptr);
-        if (rc) return rc;
+                          ws_bytes, tag + (u64)round + 1, stream, split ? &groups : nullptr, src == tables ? 1 : 0);
+        if (rc) break;
         src = work;
         half /= 2;
     }
-    // the last round's kernel has stored its samples; wait for it to retire so that the caller may release buffers
-    VI_HIP(hipStreamSynchronize(s));
+    // the last kernel retires before the caller releases its buffers
+    const hipError_t e = hipStreamSynchronize(s);
+    if (rc) return rc;
+    if (e != hipSuccess) return vi::fail(VI_EHIP, "vi_sumcheck_prove: %s", hipGetErrorString(e));
+    return VI_OK;
+}
+
+}  // extern "C"
+
+#include "sumcheck_fast.hpp"
+
+extern "C" {
+
+size_t vi_sumcheck_prove_coins_workspace_bytes(int64_t size) {
+    if (size < 2 || (size & (size - 1))) return 0;
+    return (size_t)(vi::ilog2(size) + 1) * MAX_BLOCKS * NSAMP * sizeof(u64);
+}
+
+int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                            const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                            const uint64_t *challenges, uint64_t *samples, void *ws, size_t ws_bytes, void *stream) {
+    const char *who = "vi_sumcheck_prove_coins";
+    if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "%s: size must be a power of two >= 2, got %lld", who, (long long)size);
+    const int v = vi::ilog2(size);
+    if (v > MAX_ROUNDS) return vi::fail(VI_EINVAL, "%s: %d rounds exceed %d", who, v, MAX_ROUNDS);
+    if (!challenges || !samples || !work) return vi::fail(VI_EINVAL, "%s: null pointer", who);
+    if (!ws || ws_bytes < vi_sumcheck_prove_coins_workspace_bytes(size))
+        return vi::fail(VI_ENOMEM, "%s: workspace below %zu bytes", who, vi_sumcheck_prove_coins_workspace_bytes(size));
+    int deg = 0;
+    int rc = check_terms(who, tables, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
+    if (rc) return rc;
+    for (int t = 0; t < n_tables; ++t)
+        if (!work[t]) return vi::fail(VI_EINVAL, "%s: null work buffer %d", who, t);
+    hipStream_t s = (hipStream_t)stream;
+    u64 *part = (u64 *)ws;
+
+    ChainDesc C;
+    for (int k = 0; k < MAX_ROUNDS; ++k) {
+        C.r[k] = k < v ? challenges[k] % gl::P : 0;
+        C.off[k] = 0;
+        C.nb[k] = 0;
+    }
+    for (int x = 0; x < NSAMP; ++x) C.winv[x] = 0;
+    lagrange_weights(deg + 1, C.winv);
+    C.scale = 1;
+    C.skip_mask = 0;
+    C.n_rounds = v;
+    C.n_prior = v;
+    C.deg = deg;
+
+    const bool split = !fits_one_desc(n_tables, term_off, n_terms);
+    if (!split) {
+        Desc D;
+        rc = fill_desc(D, tables, work, n_tables, term_off, factor_idx, coeffs, n_terms, true, who);
+        if (rc) return rc;
+        // the shapes with a kernel of their own: several rounds per launch
+        if ((D.product && n_tables <= 4) || D.gate) {
+            FastDesc F;
+            for (int t = 0; t < 4; ++t) {
+                F.src[t] = t < n_tables ? D.src[t] : nullptr;
+                F.dst[t] = t < n_tables ? D.dst[t] : nullptr;
+            }
+            F.lin_coeff = D.gate ? D.lin_coeff[0] : 1;
+            C.scale = D.out_scale;
+            if (D.gate) return prove_fast_shape<4, 2>(F, work, size, C, part, samples, s);
+            switch (n_tables) {
+                case 1: return prove_fast_shape<1, 1>(F, work, size, C, part, samples, s);
+                case 2: return prove_fast_shape<2, 1>(F, work, size, C, part, samples, s);
+                case 3: return prove_fast_shape<3, 1>(F, work, size, C, part, samples, s);
+                default: return prove_fast_shape<4, 1>(F, work, size, C, part, samples, s);
+            }
+        }
+        // any other sum of at most one descriptor: one launch per round, queued back to back
+        i64 half = size / 2;
+        unsigned off = 0;
+        const bool regs = n_tables <= REG_TABLES;
+        C.scale = D.out_scale;
+        for (int k = 0; k < v; ++k, half >>= 1) {
+            int nb;
+            if (k == 0) {
+                if (regs) nb = launch_round<0>(D, half, 0, part + off, blocks_for(half), nullptr, 1, 0, 0, s);
+                else nb = launch_eval_mem(D, half, part + off, 0, 1, s);
+                VI_LAUNCH_CHECK("sumcheck eval");
+            } else {
+                // half = pairs of this round; the fold by r_(k-1) halves tables of 4 * half words
+                Desc E = D;
+                E.canon_src = k == 1;
+                if (k > 1) for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+                if (regs) {
+                    E.skip1 = 1;
+                    C.skip_mask |= 1ull << k;
+                    nb = launch_round<2>(E, 2 * half, C.r[k - 1], part + off, blocks_for(half), nullptr, 1, 0, 0, s);
+                    VI_LAUNCH_CHECK("sumcheck fold+eval");
+                } else {
+                    rc = fold_tables(E.src, E.dst, n_tables, 2 * half, C.r[k - 1], s, E.canon_src);
+                    if (rc) return rc;
+                    for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+                    nb = launch_eval_mem(E, half, part + off, 0, 1, s);
+                    VI_LAUNCH_CHECK("sumcheck eval");
+                }
+            }
+            C.off[k] = off;
+            C.nb[k] = (unsigned short)nb;
+            off += (unsigned)nb * NSAMP;
+        }
+    } else {
+        // beyond one descriptor: fold every table, then evaluate group by group, per round
+        std::vector<TermGroup> groups;
+        split_terms(n_tables, term_off, factor_idx, coeffs, n_terms, groups);
+        i64 half = size / 2;
+        unsigned off = 0;
+        for (int k = 0; k < v; ++k, half >>= 1) {
+            int nb = 0;
+            if (k > 0) {
+                rc = fold_tables(k == 1 ? tables : (const uint64_t *const *)work, work, n_tables, 2 * half, C.r[k - 1], s, k == 1);
+                if (rc) return rc;
+            }
+            rc = eval_groups(who, k == 0 ? tables : (const uint64_t *const *)work, groups, deg, half, part + off, nullptr, 0, s, &nb);
+            if (rc) return rc;
+            C.off[k] = off;
+            C.nb[k] = (unsigned short)nb;
+            off += (unsigned)nb * NSAMP;
+        }
+    }
+    hipLaunchKernelGGL(k_finish, dim3(1), dim3(TAIL_THREADS), 0, s, C, (const u64 *)part, samples);
+    VI_LAUNCH_CHECK("sumcheck finish");
     return VI_OK;
 }
 

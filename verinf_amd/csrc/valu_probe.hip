@@ -1,0 +1,103 @@
+// Issue-rate probe for the integer VALU instructions the field arithmetic is made of.
+//
+// Measurement hook, no counterpart in the reference: the transforms and the hashing of this library are bound
+// by how fast a SIMD issues 32-bit integer instructions, so the figure they are put against -- wave-instructions
+// per second of the whole chip, per instruction class -- is measured here rather than assumed.  A kernel of a
+// class runs `iters` times a block of 256 instructions of that class on four independent register chains
+// (dependent instructions are four apart, beyond the pipeline depth), on every SIMD of the chip at eight
+// wavefronts each; thread 0 of every workgroup also reads the shader clock counter and the constant 100 MHz
+// counter before and after, which gives the clock the SIMDs actually ran at during the loop.
+#include "common.hpp"
+
+namespace {
+
+#define VI_REP4(...) __VA_ARGS__ __VA_ARGS__ __VA_ARGS__ __VA_ARGS__
+#define VI_REP16(...) VI_REP4(VI_REP4(__VA_ARGS__))
+#define VI_REP64(...) VI_REP4(VI_REP16(__VA_ARGS__))
+
+// out[0 .. blocks*256): a value that depends on every chain (keeps the loop alive);
+// clocks[4b .. 4b+3]: shader-clock ticks and 100 MHz ticks at the start and the end of workgroup b
+#define VI_PROBE_KERNEL(name, ...)                                                                        \
+    __global__ __launch_bounds__(256) void name(uint64_t *out, uint64_t *clocks, int iters) {             \
+        uint32_t a0 = threadIdx.x, a1 = a0 + 1, a2 = a0 + 2, a3 = a0 + 3;                                  \
+        uint64_t d0 = a0, d1 = a1, d2 = a2, d3 = a3;                                                       \
+        uint64_t c0 = 0, t0 = 0;                                                                           \
+        if (threadIdx.x == 0) { c0 = __builtin_readcyclecounter(); t0 = wall_clock64(); }                  \
+        for (int i = 0; i < iters; ++i) { VI_REP64(__VA_ARGS__) }                                          \
+        if (threadIdx.x == 0) {                                                                            \
+            clocks[4 * blockIdx.x + 0] = c0;                                                               \
+            clocks[4 * blockIdx.x + 1] = __builtin_readcyclecounter();                                     \
+            clocks[4 * blockIdx.x + 2] = t0;                                                               \
+            clocks[4 * blockIdx.x + 3] = wall_clock64();                                                   \
+        }                                                                                                  \
+        out[(size_t)blockIdx.x * 256 + threadIdx.x] = a0 + a1 + a2 + a3 + d0 + d1 + d2 + d3;               \
+    }
+
+#define VI_A32 "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3)
+#define VI_D64 "+v"(d0), "+v"(d1), "+v"(d2), "+v"(d3)
+
+VI_PROBE_KERNEL(k_add_u32, asm volatile("v_add_u32 %0, %0, %1\n v_add_u32 %1, %1, %2\n v_add_u32 %2, %2, %3\n v_add_u32 %3, %3, %0" : VI_A32);)
+VI_PROBE_KERNEL(k_add_co, asm volatile("v_add_co_u32 %0, vcc, %0, %1\n v_add_co_u32 %1, vcc, %1, %2\n v_add_co_u32 %2, vcc, %2, %3\n v_add_co_u32 %3, vcc, %3, %0" : VI_A32 : : "vcc");)
+VI_PROBE_KERNEL(k_addc_co, asm volatile("v_addc_co_u32 %0, vcc, %0, %1, vcc\n v_addc_co_u32 %1, vcc, %1, %2, vcc\n v_addc_co_u32 %2, vcc, %2, %3, vcc\n v_addc_co_u32 %3, vcc, %3, %0, vcc" : VI_A32 : : "vcc");)
+VI_PROBE_KERNEL(k_cndmask, asm volatile("v_cndmask_b32 %0, %0, %1, vcc\n v_cndmask_b32 %1, %1, %2, vcc\n v_cndmask_b32 %2, %2, %3, vcc\n v_cndmask_b32 %3, %3, %0, vcc" : VI_A32 : : "vcc");)
+VI_PROBE_KERNEL(k_alignbit, asm volatile("v_alignbit_b32 %0, %0, %1, 7\n v_alignbit_b32 %1, %1, %2, 9\n v_alignbit_b32 %2, %2, %3, 11\n v_alignbit_b32 %3, %3, %0, 13" : VI_A32);)
+VI_PROBE_KERNEL(k_add3, asm volatile("v_add3_u32 %0, %0, %1, %2\n v_add3_u32 %1, %1, %2, %3\n v_add3_u32 %2, %2, %3, %0\n v_add3_u32 %3, %3, %0, %1" : VI_A32);)
+VI_PROBE_KERNEL(k_xor, asm volatile("v_xor_b32 %0, %0, %1\n v_xor_b32 %1, %1, %2\n v_xor_b32 %2, %2, %3\n v_xor_b32 %3, %3, %0" : VI_A32);)
+VI_PROBE_KERNEL(k_mul_lo, asm volatile("v_mul_lo_u32 %0, %0, %1\n v_mul_lo_u32 %1, %1, %2\n v_mul_lo_u32 %2, %2, %3\n v_mul_lo_u32 %3, %3, %0" : VI_A32);)
+VI_PROBE_KERNEL(k_mul_hi, asm volatile("v_mul_hi_u32 %0, %0, %1\n v_mul_hi_u32 %1, %1, %2\n v_mul_hi_u32 %2, %2, %3\n v_mul_hi_u32 %3, %3, %0" : VI_A32);)
+VI_PROBE_KERNEL(k_mad_u64_u32, asm volatile("v_mad_u64_u32 %0, s[10:11], %4, %5, %0\n v_mad_u64_u32 %1, s[10:11], %5, %6, %1\n v_mad_u64_u32 %2, s[10:11], %6, %7, %2\n v_mad_u64_u32 %3, s[10:11], %7, %4, %3" : VI_D64 : "v"(a0), "v"(a1), "v"(a2), "v"(a3) : "s10", "s11");)
+VI_PROBE_KERNEL(k_lshl_add_u64, asm volatile("v_lshl_add_u64 %0, %0, 0, %1\n v_lshl_add_u64 %1, %1, 0, %2\n v_lshl_add_u64 %2, %2, 0, %3\n v_lshl_add_u64 %3, %3, 0, %0" : VI_D64);)
+VI_PROBE_KERNEL(k_cmp_u64, asm volatile("v_cmp_lt_u64 vcc, %0, %1\n v_cmp_lt_u64 vcc, %1, %2\n v_cmp_lt_u64 vcc, %2, %3\n v_cmp_lt_u64 vcc, %3, %0" : VI_D64 : : "vcc");)
+VI_PROBE_KERNEL(k_mul_u32_u24, asm volatile("v_mul_u32_u24 %0, %0, %1\n v_mul_u32_u24 %1, %1, %2\n v_mul_u32_u24 %2, %2, %3\n v_mul_u32_u24 %3, %3, %0" : VI_A32);)
+VI_PROBE_KERNEL(k_fma_f64, asm volatile("v_fma_f64 %0, %0, %1, %2\n v_fma_f64 %1, %1, %2, %3\n v_fma_f64 %2, %2, %3, %0\n v_fma_f64 %3, %3, %0, %1" : VI_D64);)
+// the canonical modular sum as the kernels issue it (six instructions and two scalar ones per element)
+VI_PROBE_KERNEL(k_mod_add_seq, {
+    uint32_t r0, r1;
+    asm volatile("v_add_co_u32 %0, vcc, %0, %2\n v_add_co_u32 %4, s[10:11], -1, %0\n s_nop 0\n"
+                 "v_addc_co_u32 %1, vcc, %1, %3, vcc\n v_addc_co_u32 %5, s[10:11], 0, %1, s[10:11]\n"
+                 "s_or_b64 vcc, vcc, s[10:11]\n v_cndmask_b32 %0, %0, %4, vcc\n v_cndmask_b32 %1, %1, %5, vcc"
+                 : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "=&v"(r0), "=&v"(r1) : : "vcc", "scc", "s10", "s11");
+})
+
+typedef void (*probe_fn)(uint64_t *, uint64_t *, int);
+struct Probe {
+    const char *name;
+    probe_fn fn;
+    int per_block;          // VALU instructions per unrolled block of the loop body
+};
+const Probe PROBES[] = {
+    {"v_add_u32", k_add_u32, 256},          {"v_add_co_u32", k_add_co, 256},       {"v_addc_co_u32", k_addc_co, 256},
+    {"v_cndmask_b32", k_cndmask, 256},      {"v_alignbit_b32", k_alignbit, 256},   {"v_add3_u32", k_add3, 256},
+    {"v_xor_b32", k_xor, 256},              {"v_mul_lo_u32", k_mul_lo, 256},       {"v_mul_hi_u32", k_mul_hi, 256},
+    {"v_mad_u64_u32", k_mad_u64_u32, 256},  {"v_lshl_add_u64", k_lshl_add_u64, 256}, {"v_cmp_lt_u64", k_cmp_u64, 256},
+    {"v_mul_u32_u24", k_mul_u32_u24, 256},  {"v_fma_f64", k_fma_f64, 256},         {"modular add sequence (6 VALU)", k_mod_add_seq, 384},
+};
+constexpr int N_PROBES = sizeof(PROBES) / sizeof(PROBES[0]);
+
+}  // namespace
+
+extern "C" {
+
+int vi_valu_probe_count(void) { return N_PROBES; }
+
+/* rate of the constant counter the probe reads beside the shader clock, in kHz (0 if unknown) */
+int vi_wall_clock_khz(void) {
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+    return khz;
+}
+
+const char *vi_valu_probe_name(int kind) { return kind >= 0 && kind < N_PROBES ? PROBES[kind].name : ""; }
+
+int vi_valu_probe(int kind, int iters, int blocks, uint64_t *out, uint64_t *clocks, int64_t *wave_instructions,
+                  void *stream) {
+    if (kind < 0 || kind >= N_PROBES) return vi::fail(VI_EINVAL, "vi_valu_probe: kind %d (0..%d)", kind, N_PROBES - 1);
+    if (iters < 1 || blocks < 1 || !out || !clocks) return vi::fail(VI_EINVAL, "vi_valu_probe: bad argument");
+    hipLaunchKernelGGL(PROBES[kind].fn, dim3(blocks), dim3(256), 0, (hipStream_t)stream, out, clocks, iters);
+    VI_LAUNCH_CHECK("valu probe");
+    if (wave_instructions) *wave_instructions = (int64_t)blocks * 4 * iters * PROBES[kind].per_block;
+    return VI_OK;
+}
+
+}  // extern "C"

@@ -295,20 +295,10 @@ def _as_table(v, field_p):
     return torch.from_numpy(np.array([int(x) % field_p for x in v], dtype=np.uint64)).cuda()
 
 
-def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
-    """Sumcheck prover for sum_x sum_k c_k prod_j f_kj(x) with the tables on the device.
-
-    terms  [(coefficient, [factor, ...]), ...]; a factor is a Python sequence or a
-           CUDA uint64 tensor (tensors are used where they are, never copied to the
-           host); a factor object that appears several times is held once.
-    coin   host callback round -> challenge (reduced mod p here).
-    mask   optional callback (deg, mu) -> ascending coefficients of the scalar mask
-           polynomial added to the samples (gpu.py:397-406).
-    Returns (claim, round_polys, challenges, mu) exactly as gpu.py:350-410.
-    The caller's tensors are never modified."""
-    _require_gpu()
+def _sumcheck_problem(terms, field_p, who):
+    """Distinct factor objects as device tables + the terms over their indices."""
     if field_p != P:
-        raise ValueError("prove_terms_gpu: only the Goldilocks field is supported")
+        raise ValueError(f"{who}: only the Goldilocks field is supported")
     if not terms:
         raise ValueError("no terms")
     uniq, tables, tterms = {}, [], []
@@ -323,10 +313,94 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
         tterms.append((int(c) % field_p, ids))
     size = int(tables[0].numel())
     if any(int(t.numel()) != size for t in tables):
-        raise ValueError("prove_terms_gpu: factors of different lengths")
+        raise ValueError(f"{who}: factors of different lengths")
     if size < 1 or size & (size - 1):
-        raise ValueError("prove_terms_gpu: table length must be a power of two")
+        raise ValueError(f"{who}: table length must be a power of two")
+    return tables, tterms, size
+
+
+def _single_point(tables, tterms, mu0, field_p):
+    """No variables: the claim is the term sum at the one point there is."""
+    total = 0
+    vals = [int(t.cpu()[0].item()) for t in tables]
+    for c, ids in tterms:
+        prod = c
+        for i in ids:
+            prod = prod * vals[i] % field_p
+        total += prod
+    mu = mu0 % field_p
+    return (total + mu) % field_p, [], [], mu
+
+
+def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
+    """Sumcheck prover for sum_x sum_k c_k prod_j f_kj(x) with the tables on the device.
+
+    terms  [(coefficient, [factor, ...]), ...]; a factor is a Python sequence or a
+           CUDA uint64 tensor (tensors are used where they are, never copied to the
+           host); a factor object that appears several times is held once.
+    coin   host callback round -> challenge (reduced mod p here).
+    mask   optional callback (deg, mu) -> ascending coefficients of the scalar mask
+           polynomial added to the samples (gpu.py:397-406).
+    Returns (claim, round_polys, challenges, mu) exactly as gpu.py:350-410.
+    The caller's tensors are never modified.
+
+    `coin` is asked by round number only and `mask` by (deg, mu) (gpu.py:398, 403): neither
+    sees a round's samples, so both are called for every round BEFORE the first launch -- in
+    the reference's order mask(deg, mu_k), coin(k), mu_(k+1) = h_k(r_k), so that callbacks
+    sharing state (one random.Random, a tape) draw exactly what they draw there -- and the
+    whole proof is queued on the stream without a host round trip
+    (vi_sumcheck_prove_coins).  prove_terms_gpu_interactive is the variant for a coin that
+    does need the samples."""
+    _require_gpu()
+    tables, tterms, size = _sumcheck_problem(terms, field_p, "prove_terms_gpu")
     n_rounds = size.bit_length() - 1
+    if n_rounds == 0:
+        return _single_point(tables, tterms, mu0, field_p)
+    prob = _Problem(tables, tterms)
+    deg = prob.deg
+    mu = mu0 % field_p
+    challenges, masks = [], []
+    for rnd in range(n_rounds):
+        h = mask(deg, mu) if mask is not None else None
+        r = coin(rnd) % field_p
+        challenges.append(r)
+        masks.append(h)
+        if h is not None:
+            mu = _poly_eval(h, r, field_p)
+    L = _lib.lib()
+    dev = tables[0].device
+    with torch.cuda.device(dev):
+        ws = _lib.workspace(L.vi_sumcheck_prove_coins_workspace_bytes(size), dev, "sumcheck_coins")
+        work = _work_tables(tables, size, dev)
+        samples_host = _pinned_samples(8 * n_rounds)
+        chal = (ctypes.c_uint64 * n_rounds)(*challenges)
+        stream = torch.cuda.current_stream()
+        _lib.check(L.vi_sumcheck_prove_coins(_Problem.ptrs(tables), _Problem.ptrs(work), prob.n_tables, size,
+                                             prob.term_off, prob.factor_idx, prob.coeffs, prob.n_terms, chal,
+                                             samples_host.data_ptr(), ws.data_ptr(), ws.numel(), stream.cuda_stream))
+        stream.synchronize()
+        flat = samples_host[:8 * n_rounds].tolist()
+    round_polys = []
+    for rnd in range(n_rounds):
+        ys = flat[8 * rnd:8 * rnd + deg + 1]
+        h = masks[rnd]
+        if h is not None:
+            ys = [(y + _poly_eval(h, x, field_p)) % field_p for x, y in enumerate(ys)]
+        round_polys.append(list(enumerate(ys)))
+    # S(0) + S(1) of the first round is the sum over the cube
+    claim = (flat[0] + flat[1] + mu0) % field_p
+    return claim, round_polys, challenges, mu
+
+
+def prove_terms_gpu_interactive(terms, coin, field_p: int, mask=None, mu0: int = 0):
+    """prove_terms_gpu for a verifier coin that needs the samples: coin(round, samples) with
+    samples = [(x, S(x))] of that round (mask applied) -> challenge.  One launch and one host
+    wait per round (vi_sumcheck_prove); same return value."""
+    _require_gpu()
+    tables, tterms, size = _sumcheck_problem(terms, field_p, "prove_terms_gpu_interactive")
+    n_rounds = size.bit_length() - 1
+    if n_rounds == 0:
+        return _single_point(tables, tterms, mu0, field_p)
     prob = _Problem(tables, tterms)
     deg = prob.deg
     L = _lib.lib()
@@ -335,23 +409,11 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
 
     with torch.cuda.device(dev):
         ws = _lib.workspace(L.vi_sumcheck_workspace_bytes(), dev, "sumcheck")
-        if n_rounds == 0:
-            # a single point: the claim is the term sum at that point
-            total = 0
-            vals = [int(t.cpu()[0].item()) for t in tables]
-            for c, ids in tterms:
-                prod = c
-                for i in ids:
-                    prod = prod * vals[i] % field_p
-                total += prod
-            return (total + mu) % field_p, [], [], mu
-
-        # The round loop runs inside the library (vi_sumcheck_prove): per round one fused
-        # launch, a wait on a word of pinned host memory that the kernel stores behind its samples, and
-        # this callback -- the only Python left in the loop -- which applies the optional
-        # scalar mask and asks the verifier coin for the challenge.
-        samples_host = _pinned_samples()
-        work = [torch.empty(size // 2, dtype=torch.uint64, device=dev) for _ in tables] if n_rounds > 1 else tables
+        # The round loop runs inside the library: per round one fused launch, a wait on a word of pinned host
+        # memory that the kernel stores behind its samples, and this callback -- the only Python left in the
+        # loop -- which applies the optional scalar mask and asks the verifier coin for the challenge.
+        samples_host = _pinned_samples(16)
+        work = _work_tables(tables, size, dev)
         round_polys, challenges = [], []
         state = {"mu": mu, "error": None}
 
@@ -362,7 +424,7 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
                     h = mask(deg, state["mu"])
                     samples = [(x, (y + _poly_eval(h, x, field_p)) % field_p) for x, y in samples]
                 round_polys.append(samples)
-                r = coin(rnd) % field_p
+                r = coin(rnd, samples) % field_p
                 challenges.append(r)
                 if mask is not None:
                     state["mu"] = _poly_eval(h, r, field_p)
@@ -377,7 +439,7 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
         out_chals = (ctypes.c_uint64 * n_rounds)()
         rc = L.vi_sumcheck_prove(_Problem.ptrs(tables), _Problem.ptrs(work), prob.n_tables, size, prob.term_off,
                                  prob.factor_idx, prob.coeffs, prob.n_terms, cb, None, samples_host.data_ptr(),
-                                 out_samples, out_chals, ws.data_ptr(), ws.numel(),
+                                 samples_host.numel(), out_samples, out_chals, ws.data_ptr(), ws.numel(),
                                  torch.cuda.current_stream().cuda_stream)
         if state["error"] is not None:
             raise state["error"]
@@ -388,21 +450,28 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
     return claim, round_polys, challenges, mu
 
 
+def _work_tables(tables, size, dev):
+    """Half-length buffers the folded tables live in (the caller's tensors are never written)."""
+    if size < 4:
+        return tables                        # one round: nothing is folded
+    return [torch.empty(size // 2, dtype=torch.uint64, device=dev) for _ in tables]
+
+
 _PINNED = threading.local()
 
 
-def _pinned_samples():
-    """16 pinned host words (VI_SC_HOST_WORDS of the library header): the round kernels write their samples
-    into the first 8 and a tag of the round that has arrived into the ninth.  One buffer per host thread and
-    stream: a proof waits for each round's samples before it goes on, so a thread needs one per stream it drives, and
-    two threads (or two streams) never see each other's samples."""
+def _pinned_samples(words: int):
+    """Pinned host words the sumcheck kernels write their samples into (and, for the interactive loop, the tag of
+    the round that has arrived).  One buffer per host thread and stream: a proof is read back before the next one
+    on that stream starts, and two threads (or two streams) never see each other's samples."""
     bufs = getattr(_PINNED, "bufs", None)
     if bufs is None:
         bufs = _PINNED.bufs = {}
     key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
-    if key not in bufs:
-        bufs[key] = torch.zeros(16, dtype=torch.uint64).pin_memory()
-    return bufs[key]
+    buf = bufs.get(key)
+    if buf is None or buf.numel() < words:
+        buf = bufs[key] = torch.zeros(max(words, 512), dtype=torch.uint64).pin_memory()
+    return buf
 
 
 def _poly_eval(coeffs: Sequence[int], x: int, p: int) -> int:
