@@ -57,6 +57,9 @@ int vi_gl_unop(int op, const uint64_t *a, uint64_t arg, uint64_t *out, int64_t n
  * applied elementwise, so that the test-suite can drive it with chosen operands.
  * op 0: modular add of canonical a, b;  1: a - b;  2 / 3: sum / difference of the butterfly (a, b);
  * 4: a mod p of any word;  5: a * b of any words;  6: (hi = b, lo = a) mod p;
+ * 7: the lazily reduced product, made canonical;  8 / 9: a * b + c with c = rotl(a, 17) ^ b, canonical / lazily
+ * reduced then made canonical;  10: the five-word sum a b + b b + a a + ~a ~b + (2^64 - 1)^2 reduced;
+ * 11: forty times a b summed in five words, reduced;
  * 100 + e, 0 <= e < 96: canonical a times 2^e (the compile-time shift twiddle). */
 int vi_gl_probe(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream);
 

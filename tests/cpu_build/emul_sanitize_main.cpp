@@ -12,9 +12,12 @@ static u64 rnd() {
     return rnd_state % gl::P;
 }
 
+// a heap block of exactly `words` words (one byte when there are none, which no index map may touch as a word)
+static u64 *exact(size_t words) { return (u64 *)malloc(words ? words * 8 : 1); }
+
 static int check_ntt(int logn, long m) {
     size_t n = (size_t)m << logn;
-    u64 *a = (u64 *)malloc(n * 8 + 8), *b = (u64 *)malloc(n * 8 + 8);
+    u64 *a = exact(n), *b = exact(n);
     for (size_t i = 0; i < n; ++i) a[i] = b[i] = rnd();
     emu_ntt_batched(a, m, logn, 0);
     emu_ntt_batched(a, m, logn, 1);
@@ -28,8 +31,8 @@ static int check_ntt(int logn, long m) {
 static int check_lde(int logK, int logN, long m, long w, long in_stride) {
     size_t K = (size_t)1 << logK, N = (size_t)1 << logN;
     size_t in_words = m ? (size_t)(m - 1) * in_stride + w : 0;
-    u64 *in = (u64 *)malloc(in_words * 8 + 8), *out = (u64 *)malloc((size_t)m * N * 8 + 8);
-    u64 *co = (u64 *)malloc((size_t)m * K * 8 + 8), *out2 = (u64 *)malloc((size_t)m * N * 8 + 8);
+    u64 *in = exact(in_words), *out = exact((size_t)m * N);
+    u64 *co = exact((size_t)m * K), *out2 = exact((size_t)m * N);
     for (size_t i = 0; i < in_words; ++i) in[i] = rnd();
     int bad = 0;
     if (w > 0) {

@@ -161,6 +161,45 @@ def test_host_verifier_accepts_oracle_proofs_and_rejects_tampering():
         tp.take(2)
 
 
+def test_commit_host_helpers_of_rs():
+    """The host side of layergkr/rs.py: the challenge PRF against the oracle's, distinct column sampling, the
+    Python-integer linear combination, and a host tree whose opening paths verify (odd levels included)."""
+    from verinf_amd.layergkr import rs
+    from verinf_amd.prover import protocol as pr
+    seed = bytes(range(32))
+    want = O.challenge_vec(seed, b"cols", 40)
+    assert [pr.challenge(seed, i, "cols") for i in range(40)] == [int(v) for v in want]
+    assert pr.challenge(5, 3, "lin") == int(O.challenge_vec((5).to_bytes(32, "little"), b"lin", 4)[3])
+    assert pr.challenge(b"ab", 0, "x") == pr.challenge(b"ab" + bytes(30), 0, "x")
+    cols = rs.sample_columns(seed, 12, 16)
+    assert len(cols) == len(set(cols)) == 12 and all(0 <= c < 16 for c in cols)
+    draws = [pr.challenge(seed, i, "cols") % 16 for i in range(200)]
+    assert cols == list(dict.fromkeys(draws))[:12]           # first occurrences, in draw order
+    assert rs.sample_columns(seed, 16, 16) == list(dict.fromkeys(draws))[:16]
+    with pytest.raises(ValueError):
+        rs.sample_columns(seed, 17, 16)
+    cfg = rs.Config(ELL=16, K_DEG=32, N_LIG=64, T_QUERIES=4)
+    r = random.Random(6)
+    cws = [[r.randrange(P) for _ in range(64)] for _ in range(5)]
+    co = [r.randrange(P) for _ in range(4)] + [0]
+    assert rs.linear_combination(cfg, cws, co) == [sum(a * cw[j] for a, cw in zip(co, cws)) % P for j in range(64)]
+    with pytest.raises(ValueError):
+        rs.linear_combination(cfg, cws, co[:3])
+    for n in (1, 2, 5, 8, 11):
+        leaves = [pr.blake3_digest(bytes([i])) for i in range(n)]
+        tree = rs.build_tree(leaves)
+        assert tree[0] == leaves and len(tree[-1]) == 1
+        want_levels = O.merkle_levels(np.frombuffer(b"".join(leaves), dtype=np.uint8).reshape(n, 32))
+        assert [len(l) for l in tree] == [len(l) for l in want_levels]
+        assert tree[-1][0] == want_levels[-1][0].tobytes()
+        for i in range(n):
+            path = rs.merkle_path(tree, i)
+            assert pr.merkle_verify(leaves[i], path, tree[-1][0])
+            if path:
+                sib, side = path[0]
+                assert not pr.merkle_verify(leaves[i], [(sib, 1 - side)] + path[1:], tree[-1][0]) or sib == leaves[i]
+
+
 def test_bench_refuses_more_than_one_gpu():
     """This build runs on one GPU; bench.py says so instead of starting ranks."""
     import subprocess

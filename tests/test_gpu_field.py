@@ -170,7 +170,15 @@ def test_device_field_primitives_one_by_one():
     assert run(5, xa, ya) == [x * y % P for x, y in zip(xa, ya)]
     assert run(6, xa, ya) == [((y << 64) + x) % P for x, y in zip(xa, ya)]
     assert run(4, anyw, anyw) == [x % P for x in anyw]
+    # the sumcheck passes' own forms: lazily reduced product, fused multiply-add, sums of unreduced products
+    M = (1 << 64) - 1
+    cs = [(((x << 17) | (x >> 47)) & M) ^ y for x, y in zip(xa, ya)]
+    assert run(7, xa, ya) == [x * y % P for x, y in zip(xa, ya)]
+    assert run(8, xa, ya) == [(x * y + c) % P for x, y, c in zip(xa, ya, cs)]
+    assert run(9, xa, ya) == [(x * y + c) % P for x, y, c in zip(xa, ya, cs)]
+    assert run(10, xa, ya) == [(x * y + y * y + x * x + (M - x) * (M - y) + M * M) % P for x, y in zip(xa, ya)]
+    assert run(11, xa, ya) == [40 * x * y % P for x, y in zip(xa, ya)]
     for e in range(96):
         assert run(100 + e, canon, canon) == [(x << e) % P for x in canon], e
     with pytest.raises(RuntimeError):
-        _lib.check(L.vi_gl_probe(7, 0, 0, 0, 1, None))
+        _lib.check(L.vi_gl_probe(99, 0, 0, 0, 1, None))

@@ -207,8 +207,7 @@ def test_lde_gates_and_layergkr_entry_points():
     assert gpu.selftest_ntt_spot(big, n_cols=6) is None
     # chunked == unchunked, and a row count past the reference's grid cap completes
     cfg = rs.Config(ELL=64, K_DEG=128, N_LIG=256, T_QUERIES=8)
-    g = torch.Generator(device="cuda").manual_seed(3)
-    msgs = torch.randint(0, 1 << 62, (300, cfg.ELL), generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
+    msgs = rand_field_dev((300, cfg.ELL), 3)                # uniform in [0, p)
     ref = gpu.encode_batch_ntt(cfg, msgs).clone()
     saved = gpu.MAX_GRID_ROWS
     try:
@@ -232,6 +231,28 @@ def test_lde_gates_and_layergkr_entry_points():
     assert c.n_rows == 4 and c.col_values(5) == [int(v) for v in got[:, 5]]
 
 
+def test_dense_backend_gate_of_rs_at_the_reference_geometries():
+    """rs._gpu_ok opens only after gpu.selftest agrees with the definition (layergkr/tests/test_gpu.py:21-23,
+    66-82), and the host and device linear combinations agree."""
+    from verinf_amd.layergkr import gpu, rs
+    configs = [rs.Config(ELL=16, K_DEG=32, N_LIG=64, T_QUERIES=4), rs.Config(ELL=64, K_DEG=128, N_LIG=256, T_QUERIES=8),
+               rs.Config(ELL=256, K_DEG=512, N_LIG=1024, T_QUERIES=8)]
+    cfg = configs[1]
+    rs._GPU_OK.clear()
+    assert rs._gpu_ok(cfg) is True
+    assert (cfg.ELL, cfg.K_DEG, cfg.N_LIG) in rs._GPU_OK
+    assert rs._gpu_ok(configs[0]) is True
+    r = random.Random(5)
+    cw = [rs.encode_row(cfg, [r.randrange(P) for _ in range(cfg.ELL)]) for _ in range(6)]
+    co = [r.randrange(P) for _ in range(6)]
+    assert rs.linear_combination(cfg, cw, co) == gpu.linear_combination(cfg, cw, co)
+    cols = rs.sample_columns(b"seed", cfg.T_QUERIES, cfg.N_LIG)
+    c = rs.Commit.from_messages(cfg, [[r.randrange(P) for _ in range(cfg.ELL)] for _ in range(3)])
+    for col in cols:
+        vals, path = c.open(col)
+        assert c.check_open(col, vals, path)
+
+
 def test_dense_lagrange_encoder_and_its_gate():
     """The reference's dense encoder surface (layergkr/gpu.py:80-122, 256-271, 413-434; rs.py:66-77): the matrix
     against the closed form in Python integers, the matmul encoder against the NTT encoder, the gate green."""
@@ -252,17 +273,17 @@ def test_dense_lagrange_encoder_and_its_gate():
 
 
 def test_lde_full_baseline_shape_properties(cp):
-    """The headline LDE shape (1024 x 2^16 -> 2^18): bit-exact against the oracle on a
-    row sample, codeword property (inverse transform has no coefficient >= K) on all rows."""
+    """The headline LDE shape (1024 x 2^16 -> 2^18): all 1024 rows bit-exact against the oracle, and the codeword
+    property (inverse transform has no coefficient >= K) on all rows."""
     K, N, m = 1 << 16, 1 << 18, 1024
     msgs = rand_field_dev((m, K), 2)                     # uniform in [0, p), words above 2^63 included
     assert int((msgs.view(torch.int64) < 0).sum()) > m * K // 4
     out = cp.coset_lde(msgs, K, N, 7)
-    rows = [0, 1, 511, 1023]
-    sample = to_np(msgs.view(torch.int64)[rows].contiguous().view(torch.uint64))
-    want = O.coset_lde_rows(sample, K, N, 7)
-    got = to_np(out.view(torch.int64)[rows].contiguous().view(torch.uint64))
-    assert np.array_equal(got, want)
+    host = to_np(msgs)
+    for lo in range(0, m, 256):                          # 512 MiB of codewords per slice on the host
+        want = O.coset_lde_rows(host[lo:lo + 256], K, N, 7)
+        assert np.array_equal(to_np(out[lo:lo + 256]), want), lo
+        del want
     for lo in range(0, m, 256):
         blk = out[lo:lo + 256].clone()
         cp.ntt_inverse_batched(blk)

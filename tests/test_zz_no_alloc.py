@@ -57,6 +57,46 @@ def test_static_entry_point_matches_the_workspace_one_on_two_calls_in_a_row():
         assert got == samples[0]
 
 
+def test_static_entry_point_with_tables_in_memory_and_no_device_allocation():
+    """Twenty tables (more than a thread keeps in registers: the kernel that walks the tables in memory, with several
+    rows of partial-sum slots at the small size) through the static scratch, at 2^20 and then 2^11; and a warm
+    call leaves the device's free memory and torch's allocation count where they were."""
+    from verinf_amd import _lib
+    L = _lib.lib()
+    n = 20
+    terms = [(j + 2, [0, j, j + 1]) for j in range(1, n - 1, 2)] + [(P - 7, [0, j]) for j in range(1, n)]
+    for v in (20, 11):
+        tabs = [rand_field(1 << v, 930 + 31 * v + j) for j in range(n)]
+        dev = [to_dev(t) for t in tabs]
+        half = 1 << (v - 1)
+        got = _call(L, True, dev, half, terms)
+        assert got == _call(L, False, dev, half, terms)
+        _, samples, _ = O.sumcheck_prove(tabs, terms, [1] * v)
+        assert got == samples[0]
+        # warm now: nothing may be allocated by a further call
+        ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dev])
+        off, idx = [0], []
+        for _, fs in terms:
+            idx += fs
+            off.append(len(idx))
+        term_off = (ctypes.c_int * len(off))(*off)
+        factor_idx = (ctypes.c_int * len(idx))(*idx)
+        coeffs = (ctypes.c_uint64 * len(terms))(*[c for c, _ in terms])
+        out = torch.zeros(8, dtype=torch.uint64, device="cuda")
+        torch.cuda.synchronize()
+        free0, _ = torch.cuda.mem_get_info()
+        stats0 = torch.cuda.memory_stats()
+        for _ in range(3):
+            _lib.check(L.vi_sumcheck_eval_static(ptrs, n, half, term_off, factor_idx, coeffs, len(terms), out.data_ptr(),
+                                                 _lib.stream_ptr()))
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        stats1 = torch.cuda.memory_stats()
+        assert free1 == free0
+        assert stats1["allocation.all.allocated"] == stats0["allocation.all.allocated"]
+        assert out.cpu().numpy()[:4].tolist() == got
+
+
 def test_static_entry_point_rejects_sizes_beyond_its_limit():
     from verinf_amd import _lib
     L = _lib.lib()

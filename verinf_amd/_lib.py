@@ -147,7 +147,7 @@ def stream_ptr() -> int:
 _ws_cache = {}
 
 
-def workspace(nbytes: int, device=None, tag: str = "ws"):
+def workspace(nbytes: int, device=None, tag: str = "ws", stream_ptr=None):
     """A cached uint8 device buffer of at least nbytes for the CURRENT stream of `device`.
 
     One buffer per (purpose, device, stream): the wrappers launch on torch's current stream, so two streams
@@ -155,7 +155,8 @@ def workspace(nbytes: int, device=None, tag: str = "ws"):
     stream it was allocated on -- when it is outgrown and dropped, the caching allocator may reuse its memory
     in stream order without further bookkeeping.  Buffers grow and are kept; release_workspaces() drops them."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
-    key = (tag, device.index, torch.cuda.current_stream(device).cuda_stream)
+    # stream_ptr: the current stream's handle when the caller has looked it up already
+    key = (tag, device.index, torch.cuda.current_stream(device).cuda_stream if stream_ptr is None else stream_ptr)
     buf = _ws_cache.get(key)
     if buf is None or buf.numel() < nbytes:
         with torch.cuda.device(device):

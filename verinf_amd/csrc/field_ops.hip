@@ -78,6 +78,23 @@ __global__ __launch_bounds__(BLOCK) void k_probe(int op, const u64 *a, const u64
         else if (op == 4) r = gl::canon(x);
         else if (op == 5) r = gl::mul(x, y);
         else if (op == 6) r = gl::reduce128(x, y);
+        else if (op == 7) r = gl::canon(gl::mul_lazy(x, y));
+        else if (op == 8) r = gl::mul_add(x, y, ((x << 17) | (x >> 47)) ^ y);
+        else if (op == 9) r = gl::canon(gl::mul_add_lazy(x, y, ((x << 17) | (x >> 47)) ^ y));
+        else if (op == 10 || op == 11) {
+            gl::Wide A;
+            gl::wide_zero(A);
+            if (op == 10) {
+                gl::wide_mul_acc(A, x, y);
+                gl::wide_mul_acc(A, y, y);
+                gl::wide_mul_acc(A, x, x);
+                gl::wide_mul_acc(A, ~x, ~y);
+                gl::wide_mul_acc(A, ~0ull, ~0ull);
+            } else {
+                for (int k = 0; k < 40; ++k) gl::wide_mul_acc(A, x, y);      // carries into the fifth word
+            }
+            r = gl::wide_reduce(A);
+        }
         else r = shift_by<0>(x, op - 100);
         out[i] = r;
     }
@@ -245,7 +262,7 @@ int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *
 
 int vi_gl_probe(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream) {
     const bool shift = op >= 100 && op < 196;
-    if (!shift && (op < 0 || op > 6)) return vi::fail(VI_EINVAL, "vi_gl_probe: op = %d", op);
+    if (!shift && (op < 0 || op > 11)) return vi::fail(VI_EINVAL, "vi_gl_probe: op = %d", op);
     if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_probe: n = %lld", (long long)n);
     if (n == 0) return VI_OK;
     const bool needs_b = !shift && op != 4;

@@ -192,6 +192,146 @@ __device__ __forceinline__ u64 mul(u64 a, u64 b) {
     return reduce_words((u32)p00, w1, hl, hh, st);
 }
 
+// the reduction of reduce_words() without its last step: a 64-bit word congruent to the value, not necessarily
+// below p (three instructions instead of six after the multiply-add); good as an operand of a further product
+__device__ __forceinline__ u64 reduce_words_lazy(u32 l0, u32 l1, u32 hl, u32 hh, u64 bin) {
+    u32 x0, x1, m;
+    asm("v_subb_co_u32 %[x0], vcc, %[l0], %[hh], %[bin]\n\t"
+        "s_nop 1\n\t"
+        "v_subbrev_co_u32 %[x1], vcc, 0, %[l1], vcc\n\t"
+        "s_nop 1\n\t"
+        "v_subb_co_u32 %[m], vcc, %[x0], %[x0], vcc\n\t"
+        "v_sub_co_u32 %[x0], vcc, %[x0], %[m]\n\t"
+        "s_nop 1\n\t"
+        "v_subbrev_co_u32 %[x1], vcc, 0, %[x1], vcc"
+        : [x0] "=&v"(x0), [x1] "=&v"(x1), [m] "=&v"(m)
+        : [l0] "v"(l0), [l1] "v"(l1), [hh] "v"(hh), [bin] "s"(bin)
+        : "vcc");
+    u64 w, st;
+    asm("v_mad_u64_u32 %[w], %[st], %[hl], -1, %[x]"
+        : [w] "=&v"(w), [st] "=&s"(st)
+        : [hl] "v"(hl), [x] "v"(pack(x0, x1)));
+    // the sum wrapped past 2^64 (st): add 2^64 mod p = 2^32 - 1; it cannot wrap again (w <= 2^64 - 2^33 then)
+    u32 w0 = (u32)w, w1 = (u32)(w >> 32), e;
+    asm("s_nop 1\n\t"
+        "v_cndmask_b32 %[e], 0, -1, %[st]\n\t"
+        "v_add_co_u32 %[w0], vcc, %[w0], %[e]\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[w1], vcc, 0, %[w1], vcc"
+        : [e] "=&v"(e), [w0] "+v"(w0), [w1] "+v"(w1)
+        : [st] "s"(st)
+        : "vcc");
+    return pack(w0, w1);
+}
+
+// the four partial products of a * b (+ c, a 64-bit addend of the lowest one) as the words l0 l1 hl hh of the
+// 128-bit result; *st receives the carry of the cross sum, which weighs 2^96 = -1 and goes into the reduction as a
+// borrow
+template <bool ADD>
+__device__ __forceinline__ void mul_words(u64 a, u64 b, u64 c, u32 &l0, u32 &l1, u32 &hl, u32 &hh, u64 &st) {
+    u32 a0 = (u32)a, a1 = (u32)(a >> 32), b0 = (u32)b, b1 = (u32)(b >> 32);
+    u64 p00, mm, p11, cy = 0;
+    if (ADD) {
+        asm("v_mad_u64_u32 %[p00], %[cy], %[a0], %[b0], %[c]\n\t"
+            "v_mad_u64_u32 %[mm], vcc, %[a1], %[b0], 0\n\t"
+            "v_mad_u64_u32 %[p11], vcc, %[a1], %[b1], 0\n\t"
+            "v_mad_u64_u32 %[mm], %[st], %[a0], %[b1], %[mm]"
+            : [p00] "=&v"(p00), [mm] "=&v"(mm), [p11] "=&v"(p11), [st] "=&s"(st), [cy] "=&s"(cy)
+            : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1), [c] "v"(c)
+            : "vcc");
+    } else {
+        asm("v_mad_u64_u32 %[p00], vcc, %[a0], %[b0], 0\n\t"
+            "v_mad_u64_u32 %[mm], vcc, %[a1], %[b0], 0\n\t"
+            "v_mad_u64_u32 %[p11], vcc, %[a1], %[b1], 0\n\t"
+            "v_mad_u64_u32 %[mm], %[st], %[a0], %[b1], %[mm]"
+            : [p00] "=&v"(p00), [mm] "=&v"(mm), [p11] "=&v"(p11), [st] "=&s"(st)
+            : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1)
+            : "vcc");
+    }
+    u32 q0 = (u32)p11, q1 = (u32)(p11 >> 32);
+    if (ADD) {
+        // the carry of the lowest product plus c weighs 2^64: into a1 b1 <= (2^32 - 1)^2, which cannot overflow
+        asm("v_addc_co_u32 %[q0], vcc, 0, %[q0], %[cy]\n\t"
+            "s_nop 1\n\t"
+            "v_addc_co_u32 %[q1], vcc, 0, %[q1], vcc"
+            : [q0] "+v"(q0), [q1] "+v"(q1)
+            : [cy] "s"(cy)
+            : "vcc");
+    }
+    u32 w1 = (u32)(p00 >> 32);
+    asm("v_add_co_u32 %[w1], vcc, %[w1], %[m0]\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[hl], vcc, %[q0], %[m1], vcc\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[hh], vcc, 0, %[q1], vcc"
+        : [w1] "+v"(w1), [hl] "=&v"(hl), [hh] "=&v"(hh)
+        : [m0] "v"((u32)mm), [m1] "v"((u32)(mm >> 32)), [q0] "v"(q0), [q1] "v"(q1)
+        : "vcc");
+    l0 = (u32)p00;
+    l1 = w1;
+}
+
+// a * b + c -> [0, p): the addend rides on the first partial product (20 instructions against 24 for mul + add)
+__device__ __forceinline__ u64 mul_add(u64 a, u64 b, u64 c) {
+    u32 l0, l1, hl, hh;
+    u64 st;
+    mul_words<true>(a, b, c, l0, l1, hl, hh, st);
+    return reduce_words(l0, l1, hl, hh, st);
+}
+
+// a * b + c as a 64-bit word congruent to it, not necessarily below p
+__device__ __forceinline__ u64 mul_add_lazy(u64 a, u64 b, u64 c) {
+    u32 l0, l1, hl, hh;
+    u64 st;
+    mul_words<true>(a, b, c, l0, l1, hl, hh, st);
+    return reduce_words_lazy(l0, l1, hl, hh, st);
+}
+
+// a * b as a 64-bit word congruent to the product, not necessarily below p
+__device__ __forceinline__ u64 mul_lazy(u64 a, u64 b) {
+    u32 l0, l1, hl, hh;
+    u64 st;
+    mul_words<false>(a, b, 0, l0, l1, hl, hh, st);
+    return reduce_words_lazy(l0, l1, hl, hh, st);
+}
+
+// five words w[0..4] (an integer below 2^160) += a * b, the full 128-bit product, nothing reduced: 13 instructions
+// against the 24 of a product reduced to [0, p) followed by a modular addition.  The two carry chains (the words
+// of the product, the words of the sum) are interleaved so that each carry is read two slots after it was written.
+__device__ __forceinline__ void mul_acc(u32 (&w)[5], u64 a, u64 b) {
+    u32 a0 = (u32)a, a1 = (u32)(a >> 32), b0 = (u32)b, b1 = (u32)(b >> 32);
+    u64 p00, mm, p11, st;
+    asm("v_mad_u64_u32 %[p00], vcc, %[a0], %[b0], 0\n\t"
+        "v_mad_u64_u32 %[mm], vcc, %[a1], %[b0], 0\n\t"
+        "v_mad_u64_u32 %[p11], vcc, %[a1], %[b1], 0\n\t"
+        "v_mad_u64_u32 %[mm], %[st], %[a0], %[b1], %[mm]"
+        : [p00] "=&v"(p00), [mm] "=&v"(mm), [p11] "=&v"(p11), [st] "=&s"(st)
+        : [a0] "v"(a0), [a1] "v"(a1), [b0] "v"(b0), [b1] "v"(b1)
+        : "vcc");
+    // product words: p00.lo | p00.hi + mm.lo | p11.lo + mm.hi + carry | p11.hi + carry + st (st = carry of the cross
+    // sum; the product is below 2^128, so the top word cannot overflow)
+    u32 w1 = (u32)(p00 >> 32), hl, hh;
+    u64 cb;
+    asm("v_add_co_u32 %[w1], vcc, %[w1], %[m0]\n\t"
+        "v_add_co_u32 %[A0], %[cb], %[A0], %[w0]\n\t"
+        "s_nop 0\n\t"
+        "v_addc_co_u32 %[hl], vcc, %[q0], %[m1], vcc\n\t"
+        "v_addc_co_u32 %[A1], %[cb], %[A1], %[w1], %[cb]\n\t"
+        "s_nop 0\n\t"
+        "v_addc_co_u32 %[hh], vcc, 0, %[q1], vcc\n\t"
+        "v_addc_co_u32 %[A2], %[cb], %[A2], %[hl], %[cb]\n\t"
+        "s_nop 0\n\t"
+        "v_addc_co_u32 %[hh], vcc, 0, %[hh], %[st]\n\t"
+        "v_addc_co_u32 %[A3], %[cb], %[A3], %[hh], %[cb]\n\t"
+        "s_nop 1\n\t"
+        "v_addc_co_u32 %[A4], %[cb], 0, %[A4], %[cb]"
+        : [w1] "+v"(w1), [hl] "=&v"(hl), [hh] "=&v"(hh), [cb] "=&s"(cb), [A0] "+v"(w[0]), [A1] "+v"(w[1]),
+          [A2] "+v"(w[2]), [A3] "+v"(w[3]), [A4] "+v"(w[4])
+        : [w0] "v"((u32)p00), [m0] "v"((u32)mm), [m1] "v"((u32)(mm >> 32)), [q0] "v"((u32)p11),
+          [q1] "v"((u32)(p11 >> 32)), [st] "s"(st)
+        : "vcc");
+}
+
 // canonical v times 2^E, 0 <= E < 96, canonical result; s = 32 q + r moves v into limbs m0 m1 m2 at phi^q
 template <int E>
 __device__ __forceinline__ u64 mul_pow2(u64 v) {
@@ -330,14 +470,59 @@ VI_HD u64 mul(u64 a, u64 b) {
     return reduce128(lo, hi);
 }
 
+// a * b + c in [0, p) for any words a, b, c
+VI_HD u64 mul_add(u64 a, u64 b, u64 c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::mul_add(a, b, c);
+#endif
+    return add(mul(a, b), canon(c));
+}
+
+// a * b + c as a word congruent to it, not necessarily below p
+VI_HD u64 mul_add_lazy(u64 a, u64 b, u64 c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return dev::mul_add_lazy(a, b, c);
+#endif
+    return mul_add(a, b, c);
+}
+
 // product as a non-canonical word (see reduce128_lazy): for chains of multiplications
 VI_HD u64 mul_lazy(u64 a, u64 b) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    return dev::mul(a, b);           // the scheduled canonical product is shorter than a lazy one written in C++
+    return dev::mul_lazy(a, b);
 #endif
     u64 lo, hi;
     mul_wide(a, b, lo, hi);
     return reduce128_lazy(lo, hi);
+}
+
+// Sums of products kept as plain integers: five 32-bit words, reduced once at the end.
+struct Wide {
+    u32 w[5];
+};
+VI_HD void wide_zero(Wide &A) {
+    for (int i = 0; i < 5; ++i) A.w[i] = 0;
+}
+// A += a * b (any 64-bit words); the caller keeps the number of products below 2^32
+VI_HD void wide_mul_acc(Wide &A, u64 a, u64 b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    dev::mul_acc(A.w, a, b);
+#else
+    u64 lo, hi;
+    mul_wide(a, b, lo, hi);
+    const u64 add[4] = {(u32)lo, lo >> 32, (u32)hi, hi >> 32};
+    u64 carry = 0;
+    for (int i = 0; i < 5; ++i) {
+        const u64 t = (u64)A.w[i] + (i < 4 ? add[i] : 0) + carry;
+        A.w[i] = (u32)t;
+        carry = t >> 32;
+    }
+#endif
+}
+// the integer mod p: words 0..3 as a 128-bit value, word 4 weighs 2^128 = -2^32
+VI_HD u64 wide_reduce(const Wide &A) {
+    const u64 x = reduce128(((u64)A.w[1] << 32) | A.w[0], ((u64)A.w[3] << 32) | A.w[2]);
+    return sub(x, (u64)A.w[4] << 32);
 }
 
 VI_HD u64 pow(u64 base, u64 e) {

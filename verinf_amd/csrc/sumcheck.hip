@@ -1094,7 +1094,7 @@ extern "C" {
 
 size_t vi_sumcheck_prove_coins_workspace_bytes(int64_t size) {
     if (size < 2 || (size & (size - 1))) return 0;
-    return (size_t)(vi::ilog2(size) + 1) * MAX_BLOCKS * NSAMP * sizeof(u64);
+    return (size_t)(vi::ilog2(size) + 1) * MAX_BLOCKS * NSAMP * sizeof(u64);     // a region per round + one of single rows
 }
 
 int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
@@ -1125,6 +1125,9 @@ int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work
     lagrange_weights(deg + 1, C.winv);
     C.scale = 1;
     C.skip_mask = 0;
+    C.inf_node = 0;
+    C.dfact = 1;
+    for (int x = 0; x < NSAMP; ++x) C.cinf[x] = 0;
     C.n_rounds = v;
     C.n_prior = v;
     C.deg = deg;
@@ -1143,12 +1146,12 @@ int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work
             }
             F.lin_coeff = D.gate ? D.lin_coeff[0] : 1;
             C.scale = D.out_scale;
-            if (D.gate) return prove_fast_shape<4, 2>(F, work, size, C, part, samples, s);
+            if (D.gate) return prove_fast_shape<4, 2>(F, size, C, part, samples, s);
             switch (n_tables) {
-                case 1: return prove_fast_shape<1, 1>(F, work, size, C, part, samples, s);
-                case 2: return prove_fast_shape<2, 1>(F, work, size, C, part, samples, s);
-                case 3: return prove_fast_shape<3, 1>(F, work, size, C, part, samples, s);
-                default: return prove_fast_shape<4, 1>(F, work, size, C, part, samples, s);
+                case 1: return prove_fast_shape<1, 1>(F, size, C, part, samples, s);
+                case 2: return prove_fast_shape<2, 1>(F, size, C, part, samples, s);
+                case 3: return prove_fast_shape<3, 1>(F, size, C, part, samples, s);
+                default: return prove_fast_shape<4, 1>(F, size, C, part, samples, s);
             }
         }
         // any other sum of at most one descriptor: one launch per round, queued back to back

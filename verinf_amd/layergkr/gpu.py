@@ -21,6 +21,7 @@ mle_eval work on Python lists).  The dense Lagrange-matrix encoders
 (`encode_batch[_t]`) of the reference module are not provided: the NTT encoder is
 the one encoder here.
 """
+import contextlib
 import ctypes
 import threading
 from typing import Optional, Sequence
@@ -290,7 +291,7 @@ def _as_table(v, field_p):
     if hasattr(v, "shape"):
         if v.dtype != torch.uint64 or not v.is_cuda:
             raise RuntimeError("prove_terms_gpu: tensor factors must be CUDA uint64")
-        return v.reshape(-1).contiguous()
+        return v if v.dim() == 1 and v.is_contiguous() else v.reshape(-1).contiguous()
     import numpy as np
     return torch.from_numpy(np.array([int(x) % field_p for x in v], dtype=np.uint64)).cuda()
 
@@ -369,26 +370,29 @@ def prove_terms_gpu(terms, coin, field_p: int, mask=None, mu0: int = 0):
             mu = _poly_eval(h, r, field_p)
     L = _lib.lib()
     dev = tables[0].device
-    with torch.cuda.device(dev):
-        ws = _lib.workspace(L.vi_sumcheck_prove_coins_workspace_bytes(size), dev, "sumcheck_coins")
-        work = _work_tables(tables, size, dev)
-        samples_host = _pinned_samples(8 * n_rounds)
-        chal = (ctypes.c_uint64 * n_rounds)(*challenges)
+    with _on_device(dev):
         stream = torch.cuda.current_stream()
-        _lib.check(L.vi_sumcheck_prove_coins(_Problem.ptrs(tables), _Problem.ptrs(work), prob.n_tables, size,
+        sp = stream.cuda_stream
+        ws = _lib.workspace(L.vi_sumcheck_prove_coins_workspace_bytes(size), dev, "sumcheck_coins", sp)
+        # the folded tables live in one cached scratch buffer, a half-length slice per table (the caller's
+        # tensors are never written)
+        half_bytes = (size // 2) * 8
+        work = _lib.workspace(max(prob.n_tables * half_bytes, 256), dev, "sumcheck_work", sp)
+        work_p = (ctypes.c_void_p * prob.n_tables)(*[work.data_ptr() + t * half_bytes for t in range(prob.n_tables)])
+        samples_host, samples_np = _pinned_samples(8 * n_rounds, sp)
+        chal = (ctypes.c_uint64 * n_rounds)(*challenges)
+        _lib.check(L.vi_sumcheck_prove_coins(_Problem.ptrs(tables), work_p, prob.n_tables, size,
                                              prob.term_off, prob.factor_idx, prob.coeffs, prob.n_terms, chal,
-                                             samples_host.data_ptr(), ws.data_ptr(), ws.numel(), stream.cuda_stream))
+                                             samples_host.data_ptr(), ws.data_ptr(), ws.numel(), sp))
         stream.synchronize()
-        flat = samples_host[:8 * n_rounds].tolist()
-    round_polys = []
-    for rnd in range(n_rounds):
-        ys = flat[8 * rnd:8 * rnd + deg + 1]
-        h = masks[rnd]
-        if h is not None:
-            ys = [(y + _poly_eval(h, x, field_p)) % field_p for x, y in enumerate(ys)]
-        round_polys.append(list(enumerate(ys)))
+        rows = samples_np[:8 * n_rounds].reshape(n_rounds, 8)[:, :deg + 1].tolist()
+    if mask is None:
+        round_polys = [list(enumerate(ys)) for ys in rows]
+    else:
+        round_polys = [[(x, (y + _poly_eval(h, x, field_p)) % field_p) for x, y in enumerate(ys)]
+                       for ys, h in zip(rows, masks)]
     # S(0) + S(1) of the first round is the sum over the cube
-    claim = (flat[0] + flat[1] + mu0) % field_p
+    claim = (rows[0][0] + rows[0][1] + mu0) % field_p
     return claim, round_polys, challenges, mu
 
 
@@ -412,7 +416,7 @@ def prove_terms_gpu_interactive(terms, coin, field_p: int, mask=None, mu0: int =
         # The round loop runs inside the library: per round one fused launch, a wait on a word of pinned host
         # memory that the kernel stores behind its samples, and this callback -- the only Python left in the
         # loop -- which applies the optional scalar mask and asks the verifier coin for the challenge.
-        samples_host = _pinned_samples(16)
+        samples_host, _ = _pinned_samples(16, torch.cuda.current_stream().cuda_stream)
         work = _work_tables(tables, size, dev)
         round_polys, challenges = [], []
         state = {"mu": mu, "error": None}
@@ -458,19 +462,27 @@ def _work_tables(tables, size, dev):
 
 
 _PINNED = threading.local()
+_NO_GUARD = contextlib.nullcontext()
 
 
-def _pinned_samples(words: int):
+def _on_device(dev):
+    """Context that makes `dev` current; nothing to do (and nothing paid) when it already is."""
+    return _NO_GUARD if dev.index is None or dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
+
+
+def _pinned_samples(words: int, stream_ptr: int):
     """Pinned host words the sumcheck kernels write their samples into (and, for the interactive loop, the tag of
-    the round that has arrived).  One buffer per host thread and stream: a proof is read back before the next one
-    on that stream starts, and two threads (or two streams) never see each other's samples."""
+    the round that has arrived), with a numpy view of the same memory.  One buffer per host thread and stream: a
+    proof is read back before the next one on that stream starts, and two threads (or two streams) never see each
+    other's samples."""
     bufs = getattr(_PINNED, "bufs", None)
     if bufs is None:
         bufs = _PINNED.bufs = {}
-    key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
+    key = (torch.cuda.current_device(), stream_ptr)
     buf = bufs.get(key)
-    if buf is None or buf.numel() < words:
-        buf = bufs[key] = torch.zeros(max(words, 512), dtype=torch.uint64).pin_memory()
+    if buf is None or buf[0].numel() < words:
+        t = torch.zeros(max(words, 512), dtype=torch.uint64).pin_memory()
+        buf = bufs[key] = (t, t.numpy())
     return buf
 
 
@@ -542,7 +554,7 @@ def selftest(cfg: Config, n_rows: int = 4, seed: int = 1) -> Optional[str]:
             j = next(k for k in range(cfg.N_LIG) if want[i][k] != got[i][k])
             return f"row {i} column {j}: definition {want[i][j]} != dense {got[i][j]}"
     co = [r.randrange(P) for _ in range(n_rows)]
-    comb = [sum(c * row[j] for c, row in zip(co, want)) % P for j in range(cfg.N_LIG)]
-    if comb != [int(v) for v in linear_combination(cfg, want, co)]:
+    from . import rs
+    if rs.linear_combination(cfg, want, co) != [int(v) for v in linear_combination(cfg, want, co)]:
         return "linear_combination disagrees"
     return None

@@ -15,40 +15,52 @@ from typing import List, Sequence, Tuple
 import torch
 
 from ..prover.protocol import (  # noqa: F401  (re-exported like the reference)
-    Config, P, blake3_digest, eval_zeta_form, merkle_leaf, merkle_verify)
+    Config, P, blake3_digest, challenge, eval_zeta_form, merkle_leaf, merkle_verify)
 
 Codeword = List[int]
 Path = List[Tuple[bytes, int]]
 
 
-def _b3(a: bytes, b: bytes) -> bytes:
-    return blake3_digest(a + b)
-
-
 def build_tree(leaves: List[bytes]) -> List[List[bytes]]:
-    """Host-side tree over a few leaves (rs.py:135-144): levels[0] = leaves, last level =
-    [root]; an odd node is paired with itself.  The device builds the same tree in
-    cuda_primitives.merkle_build_blake3."""
-    levels = [list(leaves)]
-    while len(levels[-1]) > 1:
-        cur = levels[-1]
-        levels.append([_b3(cur[i], cur[i + 1] if i + 1 < len(cur) else cur[i]) for i in range(0, len(cur), 2)])
-    return levels
+    """The Merkle tree over `leaves` on the host, bottom level first and the root alone in the last level
+    (rs.py:135-144).  A level of odd length hashes its last node with itself.  The device builds the same tree
+    in cuda_primitives.merkle_build_blake3; this one serves the few-leaf trees of tests and openings."""
+    tree = [list(leaves)]
+    nodes = tree[0]
+    while len(nodes) > 1:
+        if len(nodes) % 2:
+            nodes = nodes + nodes[-1:]
+        nodes = [blake3_digest(left + right) for left, right in zip(nodes[0::2], nodes[1::2])]
+        tree.append(nodes)
+    return tree
 
 
 def merkle_path(levels: List[List[bytes]], idx: int) -> Path:
-    """Opening path of leaf `idx` as (sibling, side) pairs, side 1 = sibling on the right
-    (rs.py:147-157); a missing sibling is the node itself."""
-    path: Path = []
-    for level in levels[:-1]:
-        sib = idx ^ 1
-        if sib >= len(level):
-            sib = idx
-        path.append((level[sib], 1 if (idx & 1) == 0 else 0))
-        idx //= 2
-    return path
+    """What a verifier needs to walk from leaf `idx` to the root: per level below the root the sibling's digest and
+    on which side it stands, 1 = to the right of the running node (rs.py:147-157; merkle_verify reads it).  The
+    last node of an odd level is its own sibling."""
+    steps: Path = []
+    position = idx
+    for nodes in levels[:-1]:
+        is_left = position % 2 == 0
+        neighbour = position + 1 if is_left else position - 1
+        steps.append((nodes[min(neighbour, len(nodes) - 1)], 1 if is_left else 0))
+        position >>= 1
+    return steps
 
+
+_GPU_OK: dict = {}
 _NTT_OK: dict = {}
+
+
+def _gpu_ok(cfg: Config) -> bool:
+    """Gate of the dense device encoder and the device linear combination (rs.py:38-47): open for a geometry only
+    after gpu.selftest has found them bit-identical to the definition on the host; cached per geometry."""
+    key = (cfg.ELL, cfg.K_DEG, cfg.N_LIG)
+    if key not in _GPU_OK:
+        from . import gpu
+        _GPU_OK[key] = gpu.available() and gpu.selftest(cfg) is None
+    return _GPU_OK[key]
 
 
 def _ntt_ok(cfg: Config) -> bool:
@@ -62,6 +74,37 @@ def _ntt_ok(cfg: Config) -> bool:
         else:
             _NTT_OK[key] = gpu.selftest_ntt_spot(cfg) is None
     return _NTT_OK[key]
+
+
+def linear_combination(cfg: Config, codewords: List[Codeword], coeffs: Sequence[int]) -> Codeword:
+    """sum_i coeffs[i] * codewords[i] in Python integers on the host (rs.py:262-281): the second side of the
+    cross-check in gpu.selftest and of the reference's own test; gpu.linear_combination / Commit.combine are the
+    device forms."""
+    if len(codewords) != len(coeffs):
+        raise ValueError("coeffs/codewords length mismatch")
+    totals = [0] * cfg.N_LIG
+    for row, a in zip(codewords, coeffs):
+        a %= P
+        if a:
+            totals = [t + a * int(v) for t, v in zip(totals, row)]
+    return [t % P for t in totals]
+
+
+def sample_columns(seed: bytes, count: int, n_lig: int) -> List[int]:
+    """`count` distinct column indices below n_lig drawn from the verifier coin `seed`, in draw order
+    (rs.py:282-294): challenge(seed, i, "cols") mod n_lig for i = 0, 1, ..., repeats dropped."""
+    if count > n_lig:
+        raise ValueError(f"cannot draw {count} distinct columns out of {n_lig}")
+    picked: List[int] = []
+    taken = set()
+    i = 0
+    while len(picked) < count:
+        col = challenge(seed, i, "cols") % n_lig
+        i += 1
+        if col not in taken:
+            taken.add(col)
+            picked.append(col)
+    return picked
 
 
 def lagrange_matrix(cfg: Config) -> List[List[int]]:

@@ -148,6 +148,16 @@ def blake3_digest(data: bytes) -> bytes:
     return b"".join(w.to_bytes(4, "little") for w in nodes[0])
 
 
+def challenge(seed, index: int, label: str = "") -> int:
+    """The (label, index)-th field challenge of `seed` on the host (prover/protocol.py:127-135): the low 128 bits of
+    BLAKE3(seed32 || label || index_le8), little-endian, mod p.  `seed` is bytes (padded / cut to 32) or an int
+    (its 32-byte little-endian form).  cuda_primitives.challenge_vec / challenge_at give the same values on the
+    device."""
+    key = bytes(seed).ljust(32, b"\x00")[:32] if isinstance(seed, (bytes, bytearray)) else int(seed).to_bytes(32, "little")
+    digest = blake3_digest(key + label.encode() + int(index).to_bytes(8, "little"))
+    return int.from_bytes(digest[:16], "little") % P
+
+
 EMPTY_COMMIT_ROOT = b"\x00" * 32        # sentinel for a commit with no rows
 
 
