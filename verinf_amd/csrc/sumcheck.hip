@@ -299,27 +299,36 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
 // Small rounds are bound by the latency of one thread's chain of loads (two per factor slot), so the grid's y dimension
 // deals the terms out: workgroup row ty takes the terms k = ty (mod gridDim.y) of the bracket -- the constant c0 goes
 // to row 0 -- and multiplies its share by the common factor; the shares add up in k_final like any other partials.
+// NS: evaluation points kept per pair (4 when the degree is at most 3, else NSAMP).
+// Sums of products are kept as plain five-word integers and reduced once (gl::wide_mul_acc): the linear part as
+// L = sum_k c_k lo_k and H = sum_k c_k hi_k over the raw table words (its value is c0 + L at x = 0, c0 + H at x = 1 and
+// moves by H - L per step: two multiply-accumulates per term and pair, no subtraction, no reduction of the words),
+// a product term's last factor into the bracket of its point, the bracket times the common factor into the
+// thread's sample.  D.skip1: S(1) is not summed (the proof's finishing kernel takes it from the claim).
+template <int NS>
 __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 *partial, int accumulate, u64 scale) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const int ty = blockIdx.y, ny = gridDim.y;
     const i64 stride = (i64)gridDim.x * BLOCK;
-    u64 acc[NSAMP];
+    gl::Wide acc[NS];
 #pragma unroll
-    for (int x = 0; x < NSAMP; ++x) acc[x] = 0;
+    for (int x = 0; x < NS; ++x) gl::wide_zero(acc[x]);
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride) {
         // the factored form described at Desc, every factor fetched from its table.  Loads go out in batches ahead
         // of the arithmetic that uses them (the common factor first, used last; four linear terms; two factor slots
         // of a product): one thread's loads are otherwise a chain of round trips to memory.  A slot past the end of
         // its list repeats a valid load (a cache hit) with coefficient 0 or is skipped by a wavefront-uniform test.
-        u64 sx[NSAMP];
         u64 com_lo = 0, com_hi = 0;
         if (D.common >= 0) {
             const u64 *f = D.src[D.common];
             com_lo = f[i];
             com_hi = f[half + i];
         }
+        u64 lin[NS];
         {
-            u64 lc = ty == 0 ? D.c0 : 0, ld = 0;
+            gl::Wide L, H;
+            gl::wide_zero(L);
+            gl::wide_zero(H);
             for (int k0 = ty; k0 < D.n_lin; k0 += 4 * ny) {
                 u64 a[4], b[4], c[4];
 #pragma unroll
@@ -333,69 +342,88 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const u64 cur = gl::canon(a[u]), dif = gl::sub(gl::canon(b[u]), cur);
-                    lc = gl::add(lc, gl::mul(c[u], cur));
-                    ld = gl::add(ld, gl::mul(c[u], dif));
+                    gl::wide_mul_acc(L, c[u], a[u]);
+                    gl::wide_mul_acc(H, c[u], b[u]);
                 }
             }
+            const u64 c0 = ty == 0 ? D.c0 : 0;
+            const u64 l0 = gl::wide_reduce(L), l1 = gl::wide_reduce(H);
+            const u64 ld = gl::sub(l1, l0);
+            u64 lc = gl::addc(l0, c0);
 #pragma unroll
-            for (int x = 0; x < NSAMP; ++x) {
-                sx[x] = lc;
-                if (D.n_lin) lc = gl::add(lc, ld);
+            for (int x = 0; x < NS; ++x) {
+                lin[x] = lc;
+                if (D.n_lin && x + 1 < NS) lc = gl::addc(lc, ld);
             }
         }
-        for (int k = ty; k < D.n_terms; k += ny) {
-            u64 prod[NSAMP];
+        gl::Wide br[NS];                     // the product terms of the bracket, per point
 #pragma unroll
-            for (int x = 0; x < NSAMP; ++x) prod[x] = D.coeff[k];
+        for (int x = 0; x < NS; ++x) gl::wide_zero(br[x]);
+        for (int k = ty; k < D.n_terms; k += ny) {
+            u64 prod[NS];
+#pragma unroll
+            for (int x = 0; x < NS; ++x) prod[x] = D.coeff[k];
             const int j1 = D.term_off[k + 1];
             for (int j = D.term_off[k]; j < j1; j += 2) {
                 const bool two = j + 1 < j1;
                 const u64 *f0 = D.src[D.fidx[j]], *f1 = D.src[D.fidx[two ? j + 1 : j]];
                 const u64 a0 = f0[i], b0 = f0[half + i], a1 = f1[i], b1 = f1[half + i];
-                u64 cur = gl::canon(a0), dif = gl::sub(gl::canon(b0), cur);
+                // the value of a factor at x = 0, 1, 2, ...: lo, hi, then steps of hi - lo
+                u64 cur = gl::canon(a0), nxt = gl::canon(b0);
+                u64 dif = gl::sub(nxt, cur);
+                const bool last0 = !two && j + 1 == j1;
 #pragma unroll
-                for (int x = 0; x < NSAMP; ++x) {
-                    if (x <= D.deg) prod[x] = gl::mul(prod[x], cur);
-                    cur = gl::add(cur, dif);
+                for (int x = 0; x < NS; ++x) {
+                    if (x <= D.deg && !(D.skip1 && x == 1)) {
+                        if (last0) gl::wide_mul_acc(br[x], prod[x], cur);
+                        else prod[x] = gl::mul_lazy(prod[x], cur);
+                    }
+                    if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
                 }
                 if (two) {
                     cur = gl::canon(a1);
-                    dif = gl::sub(gl::canon(b1), cur);
+                    nxt = gl::canon(b1);
+                    dif = gl::sub(nxt, cur);
+                    const bool last1 = j + 2 == j1;
 #pragma unroll
-                    for (int x = 0; x < NSAMP; ++x) {
-                        if (x <= D.deg) prod[x] = gl::mul(prod[x], cur);
-                        cur = gl::add(cur, dif);
+                    for (int x = 0; x < NS; ++x) {
+                        if (x <= D.deg && !(D.skip1 && x == 1)) {
+                            if (last1) gl::wide_mul_acc(br[x], prod[x], cur);
+                            else prod[x] = gl::mul_lazy(prod[x], cur);
+                        }
+                        if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
                     }
                 }
             }
-#pragma unroll
-            for (int x = 0; x < NSAMP; ++x)
-                if (x <= D.deg) sx[x] = gl::add(sx[x], prod[x]);
         }
-        if (D.common >= 0) {
-            u64 cur = gl::canon(com_lo), dif = gl::sub(gl::canon(com_hi), cur);
+        {
+            u64 cur = 1, nxt = 1, dif = 0;
+            if (D.common >= 0) {
+                cur = gl::canon(com_lo);
+                nxt = gl::canon(com_hi);
+                dif = gl::sub(nxt, cur);
+            }
 #pragma unroll
-            for (int x = 0; x < NSAMP; ++x) {
-                if (x <= D.deg) sx[x] = gl::mul(sx[x], cur);
-                cur = gl::add(cur, dif);
+            for (int x = 0; x < NS; ++x) {
+                if (x <= D.deg && !(D.skip1 && x == 1)) gl::wide_mul_acc(acc[x], gl::addc(lin[x], gl::wide_reduce(br[x])), cur);
+                if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
             }
         }
-#pragma unroll
-        for (int x = 0; x < NSAMP; ++x)
-            if (x <= D.deg) acc[x] = gl::add(acc[x], sx[x]);
     }
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-    for (int x = 0; x < NSAMP; ++x) {
-        u64 v = wave_sum(acc[x]);
+    for (int x = 0; x < NS; ++x) {
+        u64 v = wave_sum(gl::wide_reduce(acc[x]));
         if (lane == 0) red[w][x] = v;
     }
     __syncthreads();
     if (threadIdx.x < NSAMP) {
-        u64 v = red[0][threadIdx.x];
-        for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
-        if (scale != 1) v = gl::mul(v, scale);
+        u64 v = 0;
+        if (threadIdx.x < NS) {
+            v = red[0][threadIdx.x];
+            for (int i = 1; i < BLOCK / 64; ++i) v = gl::add(v, red[i][threadIdx.x]);
+            if (scale != 1) v = gl::mul(v, scale);
+        }
         u64 *slot = partial + ((i64)blockIdx.y * gridDim.x + blockIdx.x) * NSAMP + threadIdx.x;
         *slot = accumulate ? gl::add(v, *slot) : v;
     }
@@ -660,14 +688,15 @@ int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 s
     int cap;
     {
         std::lock_guard<std::mutex> lock(mu);
-        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem, 64);
+        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem<4>, 64);
         cap = caps[dev];
     }
     int nbx = blocks_for(half);
     if (nbx > cap) nbx = cap;
     int ny = 1;
     while (ny < 16 && nbx * ny * 2 <= 1024) ny *= 2;     // deal the terms out while the grid is below ~4 workgroups per CU
-    hipLaunchKernelGGL(k_eval_mem, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
+    if (D.deg <= 3) hipLaunchKernelGGL(k_eval_mem<4>, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
+    else hipLaunchKernelGGL(k_eval_mem<NSAMP>, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
     return nbx * ny;
 }
 
@@ -770,7 +799,7 @@ void split_terms(int n_tables, const int *term_off, const int *factor_idx, const
 // samples of sum over all groups at x = 0..deg from `tables` (pairs (i, half + i)); partial: MAX_BLOCKS * NSAMP words.
 // nb_out != NULL: the per-workgroup sums are left in `partial` (*nb_out rows) for a later kernel to add up.
 int eval_groups(const char *who, const uint64_t *const *tables, const std::vector<TermGroup> &groups, int deg, i64 half,
-                u64 *partial, u64 *out_samples, u64 flag, hipStream_t s, int *nb_out = nullptr) {
+                u64 *partial, u64 *out_samples, u64 flag, hipStream_t s, int *nb_out = nullptr, int skip1 = 0) {
     int nb = 0;
     for (size_t g = 0; g < groups.size(); ++g) {
         const TermGroup &G = groups[g];
@@ -781,6 +810,7 @@ int eval_groups(const char *who, const uint64_t *const *tables, const std::vecto
                            (int)G.coeffs.size(), true, who, true);
         if (rc) return rc;
         D.deg = deg;                        // every group yields all the samples of the whole sum
+        D.skip1 = skip1;
         nb = launch_eval_mem(D, half, partial, g > 0 ? 1 : 0, D.out_scale, s);    // the same grid for every group
         VI_LAUNCH_CHECK("sumcheck eval (term group)");
     }
@@ -1170,9 +1200,9 @@ int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work
                 Desc E = D;
                 E.canon_src = k == 1;
                 if (k > 1) for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+                E.skip1 = 1;                 // S(1) of a later round is the claim minus S(0): not summed
+                C.skip_mask |= 1ull << k;
                 if (regs) {
-                    E.skip1 = 1;
-                    C.skip_mask |= 1ull << k;
                     nb = launch_round<2>(E, 2 * half, C.r[k - 1], part + off, blocks_for(half), nullptr, 1, 0, 0, s);
                     VI_LAUNCH_CHECK("sumcheck fold+eval");
                 } else {
@@ -1199,8 +1229,10 @@ int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work
                 rc = fold_tables(k == 1 ? tables : (const uint64_t *const *)work, work, n_tables, 2 * half, C.r[k - 1], s, k == 1);
                 if (rc) return rc;
             }
-            rc = eval_groups(who, k == 0 ? tables : (const uint64_t *const *)work, groups, deg, half, part + off, nullptr, 0, s, &nb);
+            rc = eval_groups(who, k == 0 ? tables : (const uint64_t *const *)work, groups, deg, half, part + off, nullptr, 0, s, &nb,
+                             k > 0 ? 1 : 0);
             if (rc) return rc;
+            if (k > 0) C.skip_mask |= 1ull << k;
             C.off[k] = off;
             C.nb[k] = (unsigned short)nb;
             off += (unsigned)nb * NSAMP;
