@@ -18,6 +18,7 @@
 //
 // Variable order is most-significant first, pairs are (i, half + i)
 // (layergkr/sumcheck.py:51-54).
+#include <algorithm>
 #include <atomic>
 #include <mutex>
 #include <vector>
@@ -1127,24 +1128,173 @@ size_t vi_sumcheck_prove_coins_workspace_bytes(int64_t size) {
     return (size_t)(vi::ilog2(size) + 1) * MAX_BLOCKS * NSAMP * sizeof(u64);     // a region per round + one of single rows
 }
 
-int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
-                            const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
-                            const uint64_t *challenges, uint64_t *samples, void *ws, size_t ws_bytes, void *stream) {
-    const char *who = "vi_sumcheck_prove_coins";
-    if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "%s: size must be a power of two >= 2, got %lld", who, (long long)size);
-    const int v = vi::ilog2(size);
-    if (v > MAX_ROUNDS) return vi::fail(VI_EINVAL, "%s: %d rounds exceed %d", who, v, MAX_ROUNDS);
-    if (!challenges || !samples || !work) return vi::fail(VI_EINVAL, "%s: null pointer", who);
-    if (!ws || ws_bytes < vi_sumcheck_prove_coins_workspace_bytes(size))
-        return vi::fail(VI_ENOMEM, "%s: workspace below %zu bytes", who, vi_sumcheck_prove_coins_workspace_bytes(size));
-    int deg = 0;
-    int rc = check_terms(who, tables, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
-    if (rc) return rc;
-    for (int t = 0; t < n_tables; ++t)
-        if (!work[t]) return vi::fail(VI_EINVAL, "%s: null work buffer %d", who, t);
-    hipStream_t s = (hipStream_t)stream;
-    u64 *part = (u64 *)ws;
+namespace {
 
+// ---- the terms that are linear once a common factor is taken out, as ONE table --------------------------------
+// In a batched gate check (layergkr/relations.py:104-124) most terms are eq(z, .) times a single table (the c of a
+// hadamard gate, the three tables of a rescale or affine gate, the b of a booleanity gate).  Folding is linear, so
+// after round 0 all of them together are the one table lambda = sum_k c_k T_k, folded like any other: the tables
+// that occur in no product are never read again, and every later round walks the product tables and lambda only.
+// lambda is built already folded by the first challenge (half the size: it fits the work buffer of a table that
+// has dropped out), from the raw words of its tables through five-word sums.
+struct LinFoldDesc {
+    const u64 *src[VI_SC_MAX_TABLES];
+    u64 coeff[VI_SC_MAX_TABLES];
+    int n;
+};
+
+__global__ __launch_bounds__(BLOCK) void k_lin_fold(const LinFoldDesc F, i64 half, u64 r, u64 *dst, int accumulate) {
+    const i64 stride = (i64)gridDim.x * BLOCK;
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride) {
+        gl::Wide L, H;
+        gl::wide_zero(L);
+        gl::wide_zero(H);
+        for (int k0 = 0; k0 < F.n; k0 += 4) {            // four tables' loads in flight
+            u64 a[4], b[4], c[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const bool on = k0 + u < F.n;
+                const u64 *f = F.src[on ? k0 + u : k0];
+                a[u] = f[i];
+                b[u] = f[half + i];
+                c[u] = on ? F.coeff[k0 + u] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                gl::wide_mul_acc(L, c[u], a[u]);
+                gl::wide_mul_acc(H, c[u], b[u]);
+            }
+        }
+        const u64 lo = gl::wide_reduce(L), hi = gl::wide_reduce(H);
+        u64 v = gl::mul_add(r, gl::sub(hi, lo), lo);
+        if (accumulate) v = gl::addc(v, dst[i]);
+        dst[i] = v;
+    }
+}
+
+// the rewritten problem: the tables that stay (indices into the caller's list) and lambda as the last table
+struct LinearReduction {
+    std::vector<int> keep;                   // tables folded one by one, ascending
+    std::vector<int> lin_tab;                // tables of lambda
+    std::vector<u64> lin_c;                  // and their coefficients
+    int lambda_buf;                          // the table whose work buffer receives lambda
+    std::vector<int> term_off, fidx;         // terms over positions in keep + [lambda]
+    std::vector<u64> coeffs;
+};
+
+// false: nothing to gain (fewer than two linear tables, no table has dropped out, or the degree would change)
+bool reduce_linear_terms(int n_tables, const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, int deg,
+                         LinearReduction &R) {
+    if (n_terms < 2) return false;
+    // a table every term holds
+    int common = -1;
+    for (int j = term_off[0]; j < term_off[1] && common < 0; ++j) {
+        bool everywhere = true;
+        for (int k = 1; k < n_terms && everywhere; ++k) {
+            bool found = false;
+            for (int q = term_off[k]; q < term_off[k + 1]; ++q) found = found || factor_idx[q] == factor_idx[j];
+            everywhere = found;
+        }
+        if (everywhere) common = factor_idx[j];
+    }
+    std::vector<u64> lin_coeff(n_tables, 0);
+    std::vector<char> is_lin(n_tables, 0), in_kept(n_tables, 0);
+    std::vector<int> kept_terms;
+    for (int k = 0; k < n_terms; ++k) {
+        int rest = -1, n_rest = 0;
+        bool dropped = common < 0;
+        for (int q = term_off[k]; q < term_off[k + 1]; ++q) {
+            if (!dropped && factor_idx[q] == common) { dropped = true; continue; }
+            rest = factor_idx[q];
+            ++n_rest;
+        }
+        if (n_rest == 1) {
+            lin_coeff[rest] = gl::add(lin_coeff[rest], coeffs[k] % gl::P);
+            is_lin[rest] = 1;
+        } else {
+            kept_terms.push_back(k);
+            for (int q = term_off[k]; q < term_off[k + 1]; ++q) in_kept[factor_idx[q]] = 1;
+        }
+    }
+    if (common >= 0) in_kept[common] = 1;
+    R.lin_tab.clear();
+    R.lin_c.clear();
+    R.lambda_buf = -1;
+    for (int t = 0; t < n_tables; ++t) {
+        if (!is_lin[t]) continue;
+        R.lin_tab.push_back(t);
+        R.lin_c.push_back(lin_coeff[t]);
+        if (!in_kept[t] && R.lambda_buf < 0) R.lambda_buf = t;
+    }
+    if (R.lin_tab.size() < 2 || R.lambda_buf < 0) return false;
+    const int lam_deg = common >= 0 ? 2 : 1;
+    int new_deg = lam_deg;
+    for (int k : kept_terms) new_deg = std::max(new_deg, term_off[k + 1] - term_off[k]);
+    if (new_deg != deg) return false;
+    std::vector<int> pos(n_tables, -1);
+    R.keep.clear();
+    for (int t = 0; t < n_tables; ++t)
+        if (in_kept[t]) { pos[t] = (int)R.keep.size(); R.keep.push_back(t); }
+    const int lambda_pos = (int)R.keep.size();
+    R.term_off.assign(1, 0);
+    R.fidx.clear();
+    R.coeffs.clear();
+    for (int k : kept_terms) {
+        for (int q = term_off[k]; q < term_off[k + 1]; ++q) R.fidx.push_back(pos[factor_idx[q]]);
+        R.term_off.push_back((int)R.fidx.size());
+        R.coeffs.push_back(coeffs[k]);
+    }
+    if (common >= 0) R.fidx.push_back(pos[common]);
+    R.fidx.push_back(lambda_pos);
+    R.term_off.push_back((int)R.fidx.size());
+    R.coeffs.push_back(1);
+    return true;
+}
+
+int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                     const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, int deg,
+                     const uint64_t *challenges, uint64_t *samples, u64 *part, hipStream_t s, bool may_reduce);
+
+// round 0 on the problem as given, then every later round on the rewritten one
+int prove_coins_reduced(const char *who, const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                        const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, int deg,
+                        const uint64_t *challenges, uint64_t *samples, u64 *part, hipStream_t s, const LinearReduction &R) {
+    const i64 half = size / 2;
+    int rc = sumcheck_eval_on(who, tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, samples, part, 0, (void *)s);
+    if (rc) return rc;
+    const u64 r0 = challenges[0] % gl::P;
+    std::vector<const uint64_t *> src;
+    std::vector<uint64_t *> dst;
+    for (int t : R.keep) { src.push_back(tables[t]); dst.push_back(work[t]); }
+    rc = fold_tables(src.data(), dst.data(), (int)src.size(), half, r0, s, 1);
+    if (rc) return rc;
+    u64 *lambda = work[R.lambda_buf];
+    for (size_t k0 = 0; k0 < R.lin_tab.size(); k0 += VI_SC_MAX_TABLES) {
+        LinFoldDesc F;
+        F.n = (int)std::min<size_t>(VI_SC_MAX_TABLES, R.lin_tab.size() - k0);
+        for (int k = 0; k < VI_SC_MAX_TABLES; ++k) {
+            F.src[k] = k < F.n ? tables[R.lin_tab[k0 + k]] : nullptr;
+            F.coeff[k] = k < F.n ? R.lin_c[k0 + k] : 0;
+        }
+        hipLaunchKernelGGL(k_lin_fold, dim3(blocks_for(half)), dim3(BLOCK), 0, s, F, half, r0, lambda, k0 > 0 ? 1 : 0);
+        VI_LAUNCH_CHECK("sumcheck linear combination");
+    }
+    // the rewritten problem lives in the work buffers and is folded in place from here on
+    std::vector<const uint64_t *> rt;
+    std::vector<uint64_t *> rw;
+    for (int t : R.keep) { rt.push_back(work[t]); rw.push_back(work[t]); }
+    rt.push_back(lambda);
+    rw.push_back(lambda);
+    return prove_coins_impl(who, rt.data(), rw.data(), (int)rt.size(), half, R.term_off.data(), R.fidx.data(), R.coeffs.data(),
+                            (int)R.coeffs.size(), deg, challenges + 1, samples + NSAMP, part, s, false);
+}
+
+// all rounds of the sum over tables of `size` words; samples: log2(size) rows of NSAMP words
+int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                     const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, int deg,
+                     const uint64_t *challenges, uint64_t *samples, u64 *part, hipStream_t s, bool may_reduce) {
+    const int v = vi::ilog2(size);
+    int rc = VI_OK;
     ChainDesc C;
     for (int k = 0; k < MAX_ROUNDS; ++k) {
         C.r[k] = k < v ? challenges[k] % gl::P : 0;
@@ -1162,6 +1312,14 @@ int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work
     C.n_prior = v;
     C.deg = deg;
 
+    // many terms that are a single table under the common factor: from round 1 on they are one table (needs a round
+    // to fold into, so at least two rounds)
+    if (may_reduce && v >= 2) {
+        LinearReduction R;
+        if (reduce_linear_terms(n_tables, term_off, factor_idx, coeffs, n_terms, deg, R))
+            return prove_coins_reduced(who, tables, work, n_tables, size, term_off, factor_idx, coeffs, n_terms, deg, challenges,
+                                       samples, part, s, R);
+    }
     const bool split = !fits_one_desc(n_tables, term_off, n_terms);
     if (!split) {
         Desc D;
@@ -1241,6 +1399,27 @@ int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(TAIL_THREADS), 0, s, C, (const u64 *)part, samples);
     VI_LAUNCH_CHECK("sumcheck finish");
     return VI_OK;
+}
+
+}  // namespace
+
+int vi_sumcheck_prove_coins(const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
+                            const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms,
+                            const uint64_t *challenges, uint64_t *samples, void *ws, size_t ws_bytes, void *stream) {
+    const char *who = "vi_sumcheck_prove_coins";
+    if (size < 2 || (size & (size - 1))) return vi::fail(VI_EINVAL, "%s: size must be a power of two >= 2, got %lld", who, (long long)size);
+    const int v = vi::ilog2(size);
+    if (v > MAX_ROUNDS) return vi::fail(VI_EINVAL, "%s: %d rounds exceed %d", who, v, MAX_ROUNDS);
+    if (!challenges || !samples || !work) return vi::fail(VI_EINVAL, "%s: null pointer", who);
+    if (!ws || ws_bytes < vi_sumcheck_prove_coins_workspace_bytes(size))
+        return vi::fail(VI_ENOMEM, "%s: workspace below %zu bytes", who, vi_sumcheck_prove_coins_workspace_bytes(size));
+    int deg = 0;
+    int rc = check_terms(who, tables, n_tables, term_off, factor_idx, coeffs, n_terms, &deg);
+    if (rc) return rc;
+    for (int t = 0; t < n_tables; ++t)
+        if (!work[t]) return vi::fail(VI_EINVAL, "%s: null work buffer %d", who, t);
+    return prove_coins_impl(who, tables, work, n_tables, size, term_off, factor_idx, coeffs, n_terms, deg, challenges, samples,
+                            (u64 *)ws, (hipStream_t)stream, true);
 }
 
 }  // extern "C"
