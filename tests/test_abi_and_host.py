@@ -79,6 +79,36 @@ def test_size_queries_and_argument_validation_without_a_device(L):
     assert sc_eval(good_off, good_idx, tables=holed) == -1 and b"null table 57" in L.vi_last_error()
     assert L.vi_sumcheck_eval_static(fake, n, 8, (ctypes.c_int * (n + 1))(*good_off), (ctypes.c_int * (2 * n))(*good_idx),
                                      (ctypes.c_uint64 * n)(*([1] * n)), n, out, None) != 0
+    # the proof with all challenges up front: sizes, workspace, pointers and terms are checked before any launch
+    assert L.vi_sumcheck_prove_coins_workspace_bytes(1 << 26) == 27 * 2048 * 8 * 8
+    assert L.vi_sumcheck_prove_coins_workspace_bytes(24) == 0
+
+    def prove(size, ws_bytes=None, work=fake, chal=True, offsets=good_off, indices=good_idx):
+        off = (ctypes.c_int * len(offsets))(*offsets)
+        idx = (ctypes.c_int * len(indices))(*indices)
+        co = (ctypes.c_uint64 * (len(offsets) - 1))(*([1] * (len(offsets) - 1)))
+        ch = (ctypes.c_uint64 * 64)(*([5] * 64)) if chal else None
+        need = L.vi_sumcheck_prove_coins_workspace_bytes(size) if ws_bytes is None else ws_bytes
+        return L.vi_sumcheck_prove_coins(fake, work, n, size, off, idx, co, len(offsets) - 1, ch, out, ws, need, None)
+
+    assert prove(24) == -1 and b"power of two" in L.vi_last_error()
+    assert prove(1) == -1
+    assert prove(1 << 41) == -1 and b"rounds" in L.vi_last_error()
+    assert prove(1 << 10, ws_bytes=1024) == -3 and b"workspace" in L.vi_last_error()
+    assert prove(1 << 10, chal=False) == -1 and b"null" in L.vi_last_error()
+    assert prove(1 << 10, work=holed) == -1 and b"null work buffer 57" in L.vi_last_error()
+    assert prove(1 << 10, indices=good_idx[:-1] + [n]) == -1 and b"factor index" in L.vi_last_error()
+    # vi_sumcheck_prove states the size of its pinned buffer
+    coin = _lib_coin()
+    assert L.vi_sumcheck_prove(fake, fake, n, 1 << 10, (ctypes.c_int * (n + 1))(*good_off), (ctypes.c_int * (2 * n))(*good_idx),
+                               (ctypes.c_uint64 * n)(*([1] * n)), n, coin, None, out, 8, (ctypes.c_uint64 * 64)(),
+                               (ctypes.c_uint64 * 16)(), ws, ws_bytes, None) == -1
+    assert b"host_samples holds 8 words" in L.vi_last_error()
+
+
+def _lib_coin():
+    from verinf_amd import _lib
+    return _lib.COIN_FN(lambda rnd, samples, n, r_out, user: 1)
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -525,6 +525,47 @@ def test_baseline_shape_three_tables_of_2p26(mods):
     assert not ok and "terminal" in why
 
 
+def test_prove_coins_c_abi_with_samples_in_device_memory(mods):
+    """vi_sumcheck_prove_coins called directly: samples land in DEVICE memory (rows of 8 words), the call returns
+    without waiting, the tables are odd-offset views; a shape with its own multi-round kernels, the gate shape,
+    a sum that is rewritten after round 0 (two tables under a common factor become one) and a general one."""
+    import ctypes
+    from verinf_amd import _lib
+    L = _lib.lib()
+    cases = [(15, 3, [(9, [0, 1, 2])]),
+             (13, 4, [(3, [0, 1, 2]), (P - 5, [0, 3])]),
+             (12, 5, [(3, [0, 1, 2]), (P - 5, [0, 3]), (7, [0, 4])]),
+             (10, 6, [(3, [0, 1]), (P - 5, [2, 3, 4]), (7, [5, 0, 1])])]
+    for v, nt, terms in cases:
+        size = 1 << v
+        tabs = [rand_field(size, 1500 + 10 * v + j) for j in range(nt)]
+        dev = []
+        for t in tabs:
+            buf = to_dev(np.concatenate([np.zeros(1, dtype=np.uint64), t]))
+            dev.append(buf[1:])
+        work = [torch.empty(size // 2, dtype=torch.uint64, device="cuda") for _ in tabs]
+        coins, _ = _coins(v, 50 + v)
+        off, idx = [0], []
+        for _, fs in terms:
+            idx += fs
+            off.append(len(idx))
+        samples = torch.zeros(8 * v, dtype=torch.uint64, device="cuda")
+        ws = torch.empty(L.vi_sumcheck_prove_coins_workspace_bytes(size), dtype=torch.uint8, device="cuda")
+        _lib.check(L.vi_sumcheck_prove_coins((ctypes.c_void_p * nt)(*[t.data_ptr() for t in dev]),
+                                             (ctypes.c_void_p * nt)(*[t.data_ptr() for t in work]), nt, size,
+                                             (ctypes.c_int * len(off))(*off), (ctypes.c_int * len(idx))(*idx),
+                                             (ctypes.c_uint64 * len(terms))(*[c for c, _ in terms]), len(terms),
+                                             (ctypes.c_uint64 * v)(*coins), samples.data_ptr(), ws.data_ptr(), ws.numel(),
+                                             _lib.stream_ptr()))
+        deg = max(len(fs) for _, fs in terms)
+        got = to_np(samples).reshape(v, 8)[:, :deg + 1].tolist()
+        want_claim, want_samples, _ = O.sumcheck_prove(tabs, terms, coins)
+        assert got == want_samples, (v, nt)
+        assert (got[0][0] + got[0][1]) % P == want_claim
+        for t, d in zip(tabs, dev):
+            assert np.array_equal(to_np(d), t), "caller's table was modified"
+
+
 def test_coins_and_masks_drawn_up_front_match_the_interactive_loop(mods):
     """prove_terms_gpu calls mask and coin for all rounds before the first launch, in the reference's order
     (mask, coin, mask, coin, ...): with a coin and a mask tape that share one random.Random -- so that any other
