@@ -300,14 +300,39 @@ __global__ __launch_bounds__(BLOCK) void k_round(const Desc D, i64 half, u64 r, 
 // Small rounds are bound by the latency of one thread's chain of loads (two per factor slot), so the grid's y dimension
 // deals the terms out: workgroup row ty takes the terms k = ty (mod gridDim.y) of the bracket -- the constant c0 goes
 // to row 0 -- and multiplies its share by the common factor; the shares add up in k_final like any other partials.
+// a linear combination of tables: sum_k coeff[k] src[k]
+constexpr int LIN_MAX = 128;
+struct LinFoldDesc {
+    const u64 *src[LIN_MAX];
+    u64 coeff[LIN_MAX];
+    int n;
+};
+
+// What k_eval_mem<*, true> does besides evaluating: it writes every table folded by the round's challenge, so
+// that a round is one pass over the tables (read both halves, write the folded half) instead of an evaluation pass
+// and a fold pass.  A table may be fetched several times on the walk over the terms; its fold is written where it is
+// fetched LAST (wb_*), so that folding in place never shows a later fetch the folded value.  `virt`: one table of
+// the descriptor that does not exist yet -- its two values of a pair are the linear combination V of other tables,
+// formed on the spot (the single table that stands for all the terms linear under the common factor, see
+// reduce_linear_terms), and its fold is written like any other.
+struct FoldOut {
+    u64 r;
+    int virt;
+    int wb_common;
+    unsigned char wb_lin[VI_SC_MAX_TERMS];
+    unsigned char wb_fac[VI_SC_MAX_FACTORS];
+};
+
 // NS: evaluation points kept per pair (4 when the degree is at most 3, else NSAMP).
 // Sums of products are kept as plain five-word integers and reduced once (gl::wide_mul_acc): the linear part as
 // L = sum_k c_k lo_k and H = sum_k c_k hi_k over the raw table words (its value is c0 + L at x = 0, c0 + H at x = 1 and
 // moves by H - L per step: two multiply-accumulates per term and pair, no subtraction, no reduction of the words),
 // a product term's last factor into the bracket of its point, the bracket times the common factor into the
 // thread's sample.  D.skip1: S(1) is not summed (the proof's finishing kernel takes it from the claim).
-template <int NS>
-__global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 *partial, int accumulate, u64 scale) {
+// FOLD: see FoldOut (one row of workgroups only: a table's last fetch must belong to the thread that fetched it first).
+template <int NS, bool FOLD>
+__global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, const FoldOut W, const LinFoldDesc V, i64 half, u64 *partial,
+                                                    int accumulate, u64 scale) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const int ty = blockIdx.y, ny = gridDim.y;
     const i64 stride = (i64)gridDim.x * BLOCK;
@@ -319,11 +344,41 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
         // of the arithmetic that uses them (the common factor first, used last; four linear terms; two factor slots
         // of a product): one thread's loads are otherwise a chain of round trips to memory.  A slot past the end of
         // its list repeats a valid load (a cache hit) with coefficient 0 or is skipped by a wavefront-uniform test.
+        u64 v_lo = 0, v_hi = 0;              // the virtual table's pair
+        if (FOLD && W.virt >= 0) {
+            gl::Wide L, H;
+            gl::wide_zero(L);
+            gl::wide_zero(H);
+            for (int k0 = 0; k0 < V.n; k0 += 4) {
+                u64 a[4], b[4], c[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const bool on = k0 + u < V.n;
+                    const u64 *f = V.src[on ? k0 + u : k0];
+                    a[u] = f[i];
+                    b[u] = f[half + i];
+                    c[u] = on ? V.coeff[k0 + u] : 0;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    gl::wide_mul_acc(L, c[u], a[u]);
+                    gl::wide_mul_acc(H, c[u], b[u]);
+                }
+            }
+            v_lo = gl::wide_reduce(L);
+            v_hi = gl::wide_reduce(H);
+            D.dst[W.virt][i] = gl::mul_add(W.r, gl::sub(v_hi, v_lo), v_lo);
+        }
         u64 com_lo = 0, com_hi = 0;
         if (D.common >= 0) {
-            const u64 *f = D.src[D.common];
-            com_lo = f[i];
-            com_hi = f[half + i];
+            if (FOLD && D.common == W.virt) {
+                com_lo = v_lo;
+                com_hi = v_hi;
+            } else {
+                const u64 *f = D.src[D.common];
+                com_lo = f[i];
+                com_hi = f[half + i];
+            }
         }
         u64 lin[NS];
         {
@@ -336,15 +391,28 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
                 for (int u = 0; u < 4; ++u) {
                     const int k = k0 + u * ny;
                     const bool on = k < D.n_lin;
-                    const u64 *f = D.src[D.lin_idx[on ? k : k0]];
-                    a[u] = f[i];
-                    b[u] = f[half + i];
+                    const int t = D.lin_idx[on ? k : k0];
+                    if (FOLD && t == W.virt) {
+                        a[u] = v_lo;
+                        b[u] = v_hi;
+                    } else {
+                        const u64 *f = D.src[t];
+                        a[u] = f[i];
+                        b[u] = f[half + i];
+                    }
                     c[u] = on ? D.lin_coeff[k] : 0;
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     gl::wide_mul_acc(L, c[u], a[u]);
                     gl::wide_mul_acc(H, c[u], b[u]);
+                    if (FOLD) {
+                        const int k = k0 + u * ny;
+                        if (k < D.n_lin && W.wb_lin[k]) {
+                            const u64 lo = gl::canon(a[u]), hi = gl::canon(b[u]);
+                            D.dst[D.lin_idx[k]][i] = gl::mul_add(W.r, gl::sub(hi, lo), lo);
+                        }
+                    }
                 }
             }
             const u64 c0 = ty == 0 ? D.c0 : 0;
@@ -367,11 +435,16 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
             const int j1 = D.term_off[k + 1];
             for (int j = D.term_off[k]; j < j1; j += 2) {
                 const bool two = j + 1 < j1;
-                const u64 *f0 = D.src[D.fidx[j]], *f1 = D.src[D.fidx[two ? j + 1 : j]];
-                const u64 a0 = f0[i], b0 = f0[half + i], a1 = f1[i], b1 = f1[half + i];
+                const int t0 = D.fidx[j], t1 = D.fidx[two ? j + 1 : j];
+                u64 a0, b0, a1, b1;
+                if (FOLD && t0 == W.virt) { a0 = v_lo; b0 = v_hi; }
+                else { const u64 *f0 = D.src[t0]; a0 = f0[i]; b0 = f0[half + i]; }
+                if (FOLD && t1 == W.virt) { a1 = v_lo; b1 = v_hi; }
+                else { const u64 *f1 = D.src[t1]; a1 = f1[i]; b1 = f1[half + i]; }
                 // the value of a factor at x = 0, 1, 2, ...: lo, hi, then steps of hi - lo
                 u64 cur = gl::canon(a0), nxt = gl::canon(b0);
                 u64 dif = gl::sub(nxt, cur);
+                if (FOLD && W.wb_fac[j]) D.dst[t0][i] = gl::mul_add(W.r, dif, cur);
                 const bool last0 = !two && j + 1 == j1;
 #pragma unroll
                 for (int x = 0; x < NS; ++x) {
@@ -385,6 +458,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
                     cur = gl::canon(a1);
                     nxt = gl::canon(b1);
                     dif = gl::sub(nxt, cur);
+                    if (FOLD && W.wb_fac[j + 1]) D.dst[t1][i] = gl::mul_add(W.r, dif, cur);
                     const bool last1 = j + 2 == j1;
 #pragma unroll
                     for (int x = 0; x < NS; ++x) {
@@ -403,6 +477,7 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, i64 half, u64 
                 cur = gl::canon(com_lo);
                 nxt = gl::canon(com_hi);
                 dif = gl::sub(nxt, cur);
+                if (FOLD && W.wb_common) D.dst[D.common][i] = gl::mul_add(W.r, dif, cur);
             }
 #pragma unroll
             for (int x = 0; x < NS; ++x) {
@@ -679,8 +754,31 @@ int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out,
     return launch_round_u<MODE, 1>(D, half, r, partial, nb, out, scale, direct, flag, s);
 }
 
-// k_eval_mem over `half` pairs: returns the number of partial slots written (x workgroups times term rows)
-int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 scale, hipStream_t s) {
+// Where each table of D is fetched last on k_eval_mem's walk (linear terms, then the factor slots of the product terms,
+// the common factor's values being used at the very end): W.wb_*.  Tables of D that no term fetches are returned in
+// `unused` (they are folded by a launch of their own).
+void fill_fold_flags(const Desc &D, FoldOut &W, std::vector<int> &unused) {
+    for (int k = 0; k < VI_SC_MAX_TERMS; ++k) W.wb_lin[k] = 0;
+    for (int j = 0; j < VI_SC_MAX_FACTORS; ++j) W.wb_fac[j] = 0;
+    W.wb_common = 0;
+    std::vector<int> last_lin(D.n_tables, -1), last_fac(D.n_tables, -1);
+    for (int k = 0; k < D.n_lin; ++k) last_lin[D.lin_idx[k]] = k;
+    const int nf = D.n_terms > 0 ? D.term_off[D.n_terms] : 0;
+    for (int j = 0; j < nf; ++j) last_fac[D.fidx[j]] = j;
+    unused.clear();
+    for (int t = 0; t < D.n_tables; ++t) {
+        if (t == W.virt) continue;                       // written where it is formed
+        if (t == D.common) W.wb_common = 1;
+        else if (last_fac[t] >= 0) W.wb_fac[last_fac[t]] = 1;
+        else if (last_lin[t] >= 0) W.wb_lin[last_lin[t]] = 1;
+        else unused.push_back(t);
+    }
+}
+
+// k_eval_mem over `half` pairs: returns the number of partial slots written (x workgroups times term rows).
+// W != NULL: the launch also writes every table folded by W->r (D.dst), see FoldOut.
+int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 scale, hipStream_t s,
+                    const FoldOut *W = nullptr, const LinFoldDesc *V = nullptr) {
     // a grid-stride loop: no more workgroups than are resident at once (see resident_blocks), looked up per device
     static std::mutex mu;
     static int caps[64] = {0};
@@ -689,15 +787,26 @@ int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 s
     int cap;
     {
         std::lock_guard<std::mutex> lock(mu);
-        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem<4>, 64);
+        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem<4, true>, 64);
         cap = caps[dev];
     }
     int nbx = blocks_for(half);
     if (nbx > cap) nbx = cap;
     int ny = 1;
-    while (ny < 16 && nbx * ny * 2 <= 1024) ny *= 2;     // deal the terms out while the grid is below ~4 workgroups per CU
-    if (D.deg <= 3) hipLaunchKernelGGL(k_eval_mem<4>, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
-    else hipLaunchKernelGGL(k_eval_mem<NSAMP>, dim3(nbx, ny), dim3(BLOCK), 0, s, D, half, partial, accumulate, scale);
+    if (!W)
+        while (ny < 16 && nbx * ny * 2 <= 1024) ny *= 2;     // deal the terms out while the grid is below ~4 workgroups per CU
+    static const FoldOut no_fold = {};
+    static const LinFoldDesc no_virt = {};
+    const FoldOut &w = W ? *W : no_fold;
+    const LinFoldDesc &v = V ? *V : no_virt;
+    const dim3 grid(nbx, ny), block(BLOCK);
+    if (W) {
+        if (D.deg <= 3) hipLaunchKernelGGL((k_eval_mem<4, true>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
+        else hipLaunchKernelGGL((k_eval_mem<NSAMP, true>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
+    } else {
+        if (D.deg <= 3) hipLaunchKernelGGL((k_eval_mem<4, false>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
+        else hipLaunchKernelGGL((k_eval_mem<NSAMP, false>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
+    }
     return nbx * ny;
 }
 
@@ -1137,11 +1246,6 @@ namespace {
 // that occur in no product are never read again, and every later round walks the product tables and lambda only.
 // lambda is built already folded by the first challenge (half the size: it fits the work buffer of a table that
 // has dropped out), from the raw words of its tables through five-word sums.
-struct LinFoldDesc {
-    const u64 *src[VI_SC_MAX_TABLES];
-    u64 coeff[VI_SC_MAX_TABLES];
-    int n;
-};
 
 __global__ __launch_bounds__(BLOCK) void k_lin_fold(const LinFoldDesc F, i64 half, u64 r, u64 *dst, int accumulate) {
     const i64 stride = (i64)gridDim.x * BLOCK;
@@ -1255,29 +1359,69 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
                      const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, int deg,
                      const uint64_t *challenges, uint64_t *samples, u64 *part, hipStream_t s, bool may_reduce);
 
+// rounds of at least this many pairs evaluate and fold in one launch (k_eval_mem<*, true>, one row of workgroups);
+// smaller ones are bound by the latency of a thread's walk and deal the terms over rows of workgroups instead
+constexpr i64 FUSE_MIN_PAIRS = (i64)1 << 18;
+
 // round 0 on the problem as given, then every later round on the rewritten one
 int prove_coins_reduced(const char *who, const uint64_t *const *tables, uint64_t *const *work, int n_tables, int64_t size,
                         const int *term_off, const int *factor_idx, const uint64_t *coeffs, int n_terms, int deg,
                         const uint64_t *challenges, uint64_t *samples, u64 *part, hipStream_t s, const LinearReduction &R) {
     const i64 half = size / 2;
-    int rc = sumcheck_eval_on(who, tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, samples, part, 0, (void *)s);
-    if (rc) return rc;
     const u64 r0 = challenges[0] % gl::P;
-    std::vector<const uint64_t *> src;
-    std::vector<uint64_t *> dst;
-    for (int t : R.keep) { src.push_back(tables[t]); dst.push_back(work[t]); }
-    rc = fold_tables(src.data(), dst.data(), (int)src.size(), half, r0, s, 1);
-    if (rc) return rc;
     u64 *lambda = work[R.lambda_buf];
-    for (size_t k0 = 0; k0 < R.lin_tab.size(); k0 += VI_SC_MAX_TABLES) {
-        LinFoldDesc F;
-        F.n = (int)std::min<size_t>(VI_SC_MAX_TABLES, R.lin_tab.size() - k0);
-        for (int k = 0; k < VI_SC_MAX_TABLES; ++k) {
-            F.src[k] = k < F.n ? tables[R.lin_tab[k0 + k]] : nullptr;
-            F.coeff[k] = k < F.n ? R.lin_c[k0 + k] : 0;
+    const int n_red = (int)R.keep.size() + 1;
+    int rc = VI_OK;
+    bool done = false;
+    if (half >= FUSE_MIN_PAIRS && R.lin_tab.size() <= (size_t)LIN_MAX &&
+        fits_one_desc(n_red, R.term_off.data(), (int)R.coeffs.size())) {
+        // ONE pass over the caller's tables: round 0 of the rewritten sum -- lambda's two values of a pair are formed
+        // from its tables on the spot -- and every table that stays, lambda included, written folded by r_0
+        const uint64_t *src[VI_SC_MAX_TABLES];
+        uint64_t *dst[VI_SC_MAX_TABLES];
+        for (int q = 0; q + 1 < n_red; ++q) { src[q] = tables[R.keep[q]]; dst[q] = work[R.keep[q]]; }
+        src[n_red - 1] = lambda;                           // never read: the table does not exist yet
+        dst[n_red - 1] = lambda;
+        Desc D;
+        rc = fill_desc(D, src, dst, n_red, R.term_off.data(), R.fidx.data(), R.coeffs.data(), (int)R.coeffs.size(), true, who, true);
+        if (rc) return rc;
+        FoldOut W;
+        W.r = r0;
+        W.virt = n_red - 1;
+        std::vector<int> unused;
+        fill_fold_flags(D, W, unused);
+        if (unused.empty()) {
+            LinFoldDesc V;
+            V.n = (int)R.lin_tab.size();
+            for (int k = 0; k < LIN_MAX; ++k) {
+                V.src[k] = k < V.n ? tables[R.lin_tab[k]] : nullptr;
+                V.coeff[k] = k < V.n ? R.lin_c[k] : 0;
+            }
+            const int nb = launch_eval_mem(D, half, part, 0, 1, s, &W, &V);
+            VI_LAUNCH_CHECK("sumcheck eval + fold (round 0)");
+            hipLaunchKernelGGL(k_final, dim3(1), dim3(BLOCK), 0, s, (const u64 *)part, nb, deg, D.out_scale, 0, (u64)0, samples, (u64)0);
+            VI_LAUNCH_CHECK("sumcheck final");
+            done = true;
         }
-        hipLaunchKernelGGL(k_lin_fold, dim3(blocks_for(half)), dim3(BLOCK), 0, s, F, half, r0, lambda, k0 > 0 ? 1 : 0);
-        VI_LAUNCH_CHECK("sumcheck linear combination");
+    }
+    if (!done) {
+        rc = sumcheck_eval_on(who, tables, n_tables, half, term_off, factor_idx, coeffs, n_terms, samples, part, 0, (void *)s);
+        if (rc) return rc;
+        std::vector<const uint64_t *> src;
+        std::vector<uint64_t *> dst;
+        for (int t : R.keep) { src.push_back(tables[t]); dst.push_back(work[t]); }
+        rc = fold_tables(src.data(), dst.data(), (int)src.size(), half, r0, s, 1);
+        if (rc) return rc;
+        for (size_t k0 = 0; k0 < R.lin_tab.size(); k0 += LIN_MAX) {
+            LinFoldDesc F;
+            F.n = (int)std::min<size_t>(LIN_MAX, R.lin_tab.size() - k0);
+            for (int k = 0; k < LIN_MAX; ++k) {
+                F.src[k] = k < F.n ? tables[R.lin_tab[k0 + k]] : nullptr;
+                F.coeff[k] = k < F.n ? R.lin_c[k0 + k] : 0;
+            }
+            hipLaunchKernelGGL(k_lin_fold, dim3(blocks_for(half)), dim3(BLOCK), 0, s, F, half, r0, lambda, k0 > 0 ? 1 : 0);
+            VI_LAUNCH_CHECK("sumcheck linear combination");
+        }
     }
     // the rewritten problem lives in the work buffers and is folded in place from here on
     std::vector<const uint64_t *> rt;
@@ -1347,33 +1491,68 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
         unsigned off = 0;
         const bool regs = n_tables <= REG_TABLES;
         C.scale = D.out_scale;
-        for (int k = 0; k < v; ++k, half >>= 1) {
-            int nb;
-            if (k == 0) {
-                if (regs) nb = launch_round<0>(D, half, 0, part + off, blocks_for(half), nullptr, 1, 0, 0, s);
-                else nb = launch_eval_mem(D, half, part + off, 0, 1, s);
-                VI_LAUNCH_CHECK("sumcheck eval");
-            } else {
-                // half = pairs of this round; the fold by r_(k-1) halves tables of 4 * half words
-                Desc E = D;
-                E.canon_src = k == 1;
-                if (k > 1) for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
-                E.skip1 = 1;                 // S(1) of a later round is the claim minus S(0): not summed
-                C.skip_mask |= 1ull << k;
-                if (regs) {
+        if (regs) {
+            for (int k = 0; k < v; ++k, half >>= 1) {
+                int nb;
+                if (k == 0) {
+                    nb = launch_round<0>(D, half, 0, part + off, blocks_for(half), nullptr, 1, 0, 0, s);
+                    VI_LAUNCH_CHECK("sumcheck eval");
+                } else {
+                    // half = pairs of this round; the fold by r_(k-1) halves tables of 4 * half words
+                    Desc E = D;
+                    E.canon_src = k == 1;
+                    if (k > 1) for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+                    E.skip1 = 1;             // S(1) of a later round is the claim minus S(0): not summed
+                    C.skip_mask |= 1ull << k;
                     nb = launch_round<2>(E, 2 * half, C.r[k - 1], part + off, blocks_for(half), nullptr, 1, 0, 0, s);
                     VI_LAUNCH_CHECK("sumcheck fold+eval");
-                } else {
-                    rc = fold_tables(E.src, E.dst, n_tables, 2 * half, C.r[k - 1], s, E.canon_src);
+                }
+                C.off[k] = off;
+                C.nb[k] = (unsigned short)nb;
+                off += (unsigned)nb * NSAMP;
+            }
+        } else {
+            // tables in memory: a round of many pairs evaluates and writes the folded tables in one launch; a
+            // round of few folds first (one launch) and deals its terms over rows of workgroups
+            bool folded = true;              // the tables of round k are in place (false: still to be folded by r_(k-1))
+            for (int k = 0; k < v; ++k, half >>= 1) {
+                Desc E = D;
+                if (k > 0) for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+                if (!folded) {
+                    // tables of round k - 1 (2 * half pairs) -> tables of round k
+                    rc = fold_tables(k == 1 ? D.src : (const uint64_t *const *)D.dst, D.dst, n_tables, 2 * half, C.r[k - 1], s, k == 1);
                     if (rc) return rc;
-                    for (int t = 0; t < n_tables; ++t) E.src[t] = D.dst[t];
+                    folded = true;
+                }
+                if (k > 0) {
+                    E.skip1 = 1;
+                    C.skip_mask |= 1ull << k;
+                }
+                int nb;
+                if (k + 1 < v && half >= FUSE_MIN_PAIRS) {
+                    FoldOut W;
+                    W.r = C.r[k];
+                    W.virt = -1;
+                    std::vector<int> unused;
+                    fill_fold_flags(E, W, unused);
+                    if (!unused.empty()) {
+                        std::vector<const uint64_t *> us;
+                        std::vector<uint64_t *> ud;
+                        for (int t : unused) { us.push_back(E.src[t]); ud.push_back(E.dst[t]); }
+                        rc = fold_tables(us.data(), ud.data(), (int)us.size(), half, C.r[k], s, k == 0);
+                        if (rc) return rc;
+                    }
+                    nb = launch_eval_mem(E, half, part + off, 0, 1, s, &W, nullptr);
+                    VI_LAUNCH_CHECK("sumcheck eval + fold");
+                } else {
                     nb = launch_eval_mem(E, half, part + off, 0, 1, s);
                     VI_LAUNCH_CHECK("sumcheck eval");
+                    folded = false;
                 }
+                C.off[k] = off;
+                C.nb[k] = (unsigned short)nb;
+                off += (unsigned)nb * NSAMP;
             }
-            C.off[k] = off;
-            C.nb[k] = (unsigned short)nb;
-            off += (unsigned)nb * NSAMP;
         }
     } else {
         // beyond one descriptor: fold every table, then evaluate group by group, per round
