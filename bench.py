@@ -35,11 +35,14 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 # (profiles/k_lde_mid_k_ntt_fast__coset_lde_1024x2p16_to_2p18.md).  roofline.traffic is this figure divided by the
 # launches of a step, like roofline.achieved.
 LDE_TRAFFIC_BYTES_PER_STEP = 8.06e9
-# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU, same profile: per 512-row chunk 58.6 M in
-# the strided inverse launch, 296.8 M in k_lde_mid and 187.6 M in the final forward launch) and the rate at which
-# 1024 SIMDs issue them at 2.4 GHz, one per four cycles
-LDE_VALU_INSTS_PER_STEP = 2 * (58_621_952 + 296_779_776 + 187_564_032)
-VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / 4
+# VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU, same profile: per 512-row chunk 58.7 M in
+# the strided inverse launch, 296.9 M in k_lde_mid and 188.0 M in the final forward launch) and the rate at which
+# 1024 SIMDs issue the instruction classes these kernels consist of (carry, multiply, three-operand and shift
+# instructions: one per 4.16 cycles per SIMD, measured by `bench.py --valu-probe`,
+# profiles/valu_issue_rates__probe.md) at the 2.4 GHz peak clock
+LDE_VALU_INSTS_PER_STEP = 2 * (58_687_488 + 296_878_080 + 187_957_248)
+VALU_ISSUE_CYCLES_PER_INSTR = 4.16
+VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / VALU_ISSUE_CYCLES_PER_INSTR
 
 
 def _events(torch):
@@ -711,7 +714,9 @@ def main():
                                     "achieved_per_s": LDE_VALU_INSTS_PER_STEP / (lde["ms_per_step"] * 1e-3),
                                     "peak_per_s": VALU_ISSUE_PEAK_PER_S,
                                     "frac": LDE_VALU_INSTS_PER_STEP / (lde["ms_per_step"] * 1e-3) / VALU_ISSUE_PEAK_PER_S,
-                                    "source": "rocprofv3 --pmc SQ_INSTS_VALU of this command; not re-measured in this run"}},
+                                    "source": "instructions: rocprofv3 --pmc SQ_INSTS_VALU of this command; peak: 1024 SIMDs x "
+                                              "2.4 GHz / 4.16 cycles per instruction (bench.py --valu-probe, "
+                                              "profiles/valu_issue_rates__probe.md); neither re-measured in this run"}},
         "cpu_baseline": cpu,
         "extra": extra,
     }

@@ -39,7 +39,6 @@ namespace {
 VI_PROBE_KERNEL(k_add_u32, asm volatile("v_add_u32 %0, %0, %1\n v_add_u32 %1, %1, %2\n v_add_u32 %2, %2, %3\n v_add_u32 %3, %3, %0" : VI_A32);)
 VI_PROBE_KERNEL(k_add_co, asm volatile("v_add_co_u32 %0, vcc, %0, %1\n v_add_co_u32 %1, vcc, %1, %2\n v_add_co_u32 %2, vcc, %2, %3\n v_add_co_u32 %3, vcc, %3, %0" : VI_A32 : : "vcc");)
 VI_PROBE_KERNEL(k_addc_co, asm volatile("v_addc_co_u32 %0, vcc, %0, %1, vcc\n v_addc_co_u32 %1, vcc, %1, %2, vcc\n v_addc_co_u32 %2, vcc, %2, %3, vcc\n v_addc_co_u32 %3, vcc, %3, %0, vcc" : VI_A32 : : "vcc");)
-VI_PROBE_KERNEL(k_cndmask, asm volatile("v_cndmask_b32 %0, %0, %1, vcc\n v_cndmask_b32 %1, %1, %2, vcc\n v_cndmask_b32 %2, %2, %3, vcc\n v_cndmask_b32 %3, %3, %0, vcc" : VI_A32 : : "vcc");)
 VI_PROBE_KERNEL(k_alignbit, asm volatile("v_alignbit_b32 %0, %0, %1, 7\n v_alignbit_b32 %1, %1, %2, 9\n v_alignbit_b32 %2, %2, %3, 11\n v_alignbit_b32 %3, %3, %0, 13" : VI_A32);)
 VI_PROBE_KERNEL(k_add3, asm volatile("v_add3_u32 %0, %0, %1, %2\n v_add3_u32 %1, %1, %2, %3\n v_add3_u32 %2, %2, %3, %0\n v_add3_u32 %3, %3, %0, %1" : VI_A32);)
 VI_PROBE_KERNEL(k_xor, asm volatile("v_xor_b32 %0, %0, %1\n v_xor_b32 %1, %1, %2\n v_xor_b32 %2, %2, %3\n v_xor_b32 %3, %3, %0" : VI_A32);)
@@ -68,7 +67,6 @@ VI_PROBE_KERNEL(k_lshr, asm volatile("v_lshrrev_b32 %0, 3, %0\n v_lshrrev_b32 %1
 VI_PROBE_KERNEL(k_mov, asm volatile("v_mov_b32 %0, %1\n v_mov_b32 %1, %2\n v_mov_b32 %2, %3\n v_mov_b32 %3, %0" : VI_A32);)
 VI_PROBE_KERNEL(k_min, asm volatile("v_min_u32 %0, %0, %1\n v_min_u32 %1, %1, %2\n v_min_u32 %2, %2, %3\n v_min_u32 %3, %3, %0" : VI_A32);)
 VI_PROBE_KERNEL(k_cmp_u32, asm volatile("v_cmp_lt_u32 vcc, %0, %1\n v_cmp_lt_u32 vcc, %1, %2\n v_cmp_lt_u32 vcc, %2, %3\n v_cmp_lt_u32 vcc, %3, %0" : VI_A32 : : "vcc");)
-VI_PROBE_KERNEL(k_cnd_fresh, { uint32_t t0, t1, t2, t3; asm volatile("v_cndmask_b32 %0, %4, %5, vcc\n v_cndmask_b32 %1, %5, %6, vcc\n v_cndmask_b32 %2, %6, %7, vcc\n v_cndmask_b32 %3, %7, %4, vcc" : "=v"(t0), "=v"(t1), "=v"(t2), "=v"(t3) : "v"(a0), "v"(a1), "v"(a2), "v"(a3) : "vcc"); d0 += t0 ^ t1 ^ t2 ^ t3; })
 VI_PROBE_KERNEL(k_perm, asm volatile("v_perm_b32 %0, %0, %1, %2\n v_perm_b32 %1, %1, %2, %3\n v_perm_b32 %2, %2, %3, %0\n v_perm_b32 %3, %3, %0, %1" : VI_A32);)
 // how double-rate instructions behave next to others: a dependent chain, alternation with a full-rate class,
 // and pairs of each class
@@ -135,13 +133,13 @@ struct Probe {
 };
 const Probe PROBES[] = {
     {"v_add_u32", k_add_u32, 256},          {"v_add_co_u32", k_add_co, 256},       {"v_addc_co_u32", k_addc_co, 256},
-    {"v_cndmask_b32", k_cndmask, 256},      {"v_alignbit_b32", k_alignbit, 256},   {"v_add3_u32", k_add3, 256},
+    {"v_alignbit_b32", k_alignbit, 256},   {"v_add3_u32", k_add3, 256},
     {"v_xor_b32", k_xor, 256},              {"v_mul_lo_u32", k_mul_lo, 256},       {"v_mul_hi_u32", k_mul_hi, 256},
     {"v_mad_u64_u32", k_mad_u64_u32, 256},  {"v_lshl_add_u64", k_lshl_add_u64, 256}, {"v_cmp_lt_u64", k_cmp_u64, 256},
     {"v_mul_u32_u24", k_mul_u32_u24, 256},  {"v_fma_f64", k_fma_f64, 256},         {"modular add sequence (6 VALU)", k_mod_add_seq, 384},
     {"v_sub_u32", k_sub_u32, 256},          {"v_and_b32", k_and, 256},             {"v_or_b32", k_or, 256},
     {"v_lshlrev_b32", k_lshl, 256},         {"v_lshrrev_b32", k_lshr, 256},        {"v_mov_b32", k_mov, 256},
-    {"v_min_u32", k_min, 256},              {"v_cmp_lt_u32", k_cmp_u32, 256},      {"v_cndmask_b32, fresh destinations", k_cnd_fresh, 256},
+    {"v_min_u32", k_min, 256},              {"v_cmp_lt_u32", k_cmp_u32, 256},
     {"v_perm_b32", k_perm, 256},
     {"v_xor_b32, each reads the one before", k_xor_dependent, 256},
     {"v_xor_b32 / v_alignbit_b32 alternating", k_xor_align_alternating, 256},
