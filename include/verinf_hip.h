@@ -60,7 +60,8 @@ int vi_gl_unop(int op, const uint64_t *a, uint64_t arg, uint64_t *out, int64_t n
  * 7: the lazily reduced product, made canonical;  8 / 9: a * b + c with c = rotl(a, 17) ^ b, canonical / lazily
  * reduced then made canonical;  10: the five-word sum a b + b b + a a + ~a ~b + (2^64 - 1)^2 reduced;
  * 11: forty times a b summed in five words, reduced;
- * 100 + e, 0 <= e < 96: canonical a times 2^e (the compile-time shift twiddle). */
+ * 100 + e, 0 <= e < 96: canonical a times 2^e (the compile-time shift twiddle);
+ * 300 + e, 0 <= e < 192: the same for any exponent (2^96 = -1), in the form the coset loop of the fused LDE launch uses. */
 int vi_gl_probe(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream);
 
 /* Replaces gl_axpy (cuda_primitives.py:282-288, 1104-1106; gl_extras.cuh:33-41):

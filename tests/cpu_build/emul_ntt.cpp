@@ -58,6 +58,8 @@ void run_fast_u(const PassArgs &A) {
 }
 
 int g_allow_uniform = 1;
+int g_allow_merged = 1;
+long g_merged_runs = 0;                     // fused launches that took the split form of the coset factors
 
 // the same choice the HIP launcher makes: scalar-base addressing when the pass qualifies
 template <int A2, bool INV>
@@ -85,9 +87,19 @@ void run_fused(const PassArgs &Ai_in, const PassArgs &Af_in) {
         for (int tid = 0; tid < NTHREADS; ++tid)
             fast_stage1<A2, true>(Ai, tile, tid, 0, oks[tid], R(regs, tid), pw, Ai.twi, lds.data());
         for (int tid = 0; tid < NTHREADS; ++tid) fused_stage2_inv<A2>(Ai, tile, tid, lds.data(), R(coef, tid));
+        const bool mrg = Af.twm && Af.twim && Af.merge_unit > 0;       // the launcher's choice of k_lde_mid<A2, MRG>
+        if (mrg && tile == 0) ++g_merged_runs;
+        if (mrg)
+            for (int tid = 0; tid < NTHREADS; ++tid) fused_twist<A2>(Af, tile, tid, R(coef, tid));
         for (int t = 0; t < (1 << Af.log_rho); ++t) {
-            for (int tid = 0; tid < NTHREADS; ++tid) fused_stage1_fwd<A2>(Af, tile, tid, t, R(coef, tid), Af.twi, lds.data());
-            for (int tid = 0; tid < NTHREADS; ++tid) fused_stage2_fwd<A2>(Af, tile, tid, t, lds.data());
+            for (int tid = 0; tid < NTHREADS; ++tid) {
+                if (mrg) fused_stage1_fwd<A2, true>(Af, tile, tid, t, R(coef, tid), Af.twim + ((size_t)t << Af.a), lds.data());
+                else fused_stage1_fwd<A2, false>(Af, tile, tid, t, R(coef, tid), Af.twi, lds.data());
+            }
+            for (int tid = 0; tid < NTHREADS; ++tid) {
+                if (mrg) fused_stage2_fwd<A2, true>(Af, tile, tid, t, lds.data());
+                else fused_stage2_fwd<A2, false>(Af, tile, tid, t, lds.data());
+            }
         }
     }
 }
@@ -180,6 +192,8 @@ extern "C" {
 void emu_set_fast(int on) { g_use_fast = on; }
 void emu_set_uniform(int on) { g_allow_uniform = on; }
 void emu_set_fusion(int on) { g_allow_fusion = on; }
+void emu_set_merged(int on) { g_allow_merged = on; }
+long emu_merged_runs() { return g_merged_runs; }
 u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
 u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
 u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }
@@ -200,10 +214,14 @@ int emu_coset_lde(const u64 *in, long m, long w, long in_stride, int logK, int l
                   u64 *out) {
     Owned *oi = make_owned(logK, 1), *of = make_owned(logK, 0);
     std::vector<u64> pre = make_coset_pre(logK, logN, shift);
+    const bool mergeable = g_allow_merged && coset_mergeable(logK, logN);
+    if (mergeable) append_coset_merged(logK, logN, pre);
+    const u64 *merged = mergeable ? pre.data() + ((size_t)1 << logN) : nullptr;
     std::vector<u64> ws((size_t)lde_ws_elems(logK, logN, m));
     std::vector<PassArgs> passes;
     build_lde_passes(oi->T, of->T, pre.data(), logN, in, w, in_stride, out, (i64)1 << logN, ws.data(), m,
-                     passes, nullptr, 0, false, g_use_fast && g_allow_uniform && g_allow_fusion);
+                     passes, nullptr, 0, false, g_use_fast && g_allow_uniform && g_allow_fusion,
+                     merged);
     run_all(passes);
     delete oi;
     delete of;
@@ -214,10 +232,14 @@ int emu_coset_lde_ex(const u64 *in, long m, long w, long in_stride, int logK, in
                      u64 *coeffs, long coeffs_stride, u64 *out, int in_is_coeffs) {
     Owned *oi = make_owned(logK, 1), *of = make_owned(logK, 0);
     std::vector<u64> pre = make_coset_pre(logK, logN, shift);
+    const bool mergeable = g_allow_merged && coset_mergeable(logK, logN);
+    if (mergeable) append_coset_merged(logK, logN, pre);
+    const u64 *merged = mergeable ? pre.data() + ((size_t)1 << logN) : nullptr;
     std::vector<u64> ws((size_t)lde_ws_elems(logK, logN, m));
     std::vector<PassArgs> passes;
     build_lde_passes(oi->T, of->T, pre.data(), logN, in, w, in_stride, out, (i64)1 << logN, ws.data(), m,
-                     passes, coeffs, coeffs_stride, in_is_coeffs != 0, g_use_fast && g_allow_uniform && g_allow_fusion);
+                     passes, coeffs, coeffs_stride, in_is_coeffs != 0, g_use_fast && g_allow_uniform && g_allow_fusion,
+                     merged);
     run_all(passes);
     delete oi;
     delete of;

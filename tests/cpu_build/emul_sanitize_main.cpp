@@ -67,10 +67,12 @@ int main() {
         {16, 16, 1, 65536, 65536}, {8, 10, 0, 256, 256}, {12, 14, 2, 5, 8}, {14, 16, 2, 100, 128}, {14, 16, 2, 2816, 2816},
         {16, 18, 1, 4097, 4100}, {16, 18, 1, 4095, 4095}, {12, 14, 3, 257, 257},
     };
-    // per-element addressing, scalar-base addressing where it applies, and the fused middle launch of the LDE
-    for (int mode = 0; mode < 3; ++mode) {
+    // per-element addressing, scalar-base addressing where it applies, the fused middle launch of the LDE, and that
+    // launch with the coset factors split into shifts and per-coset twiddle tables
+    for (int mode = 0; mode < 4; ++mode) {
         emu_set_uniform(mode >= 1);
         emu_set_fusion(mode >= 2);
+        emu_set_merged(mode >= 3);
         for (auto &s : lde) bad += check_lde((int)s[0], (int)s[1], s[2], s[3], s[4]);
         bad += check_ntt(12, 3);
         bad += check_ntt(18, 1);

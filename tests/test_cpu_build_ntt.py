@@ -33,14 +33,24 @@ def emu():
     L.emu_set_fast.argtypes = [c_int]
     L.emu_set_uniform.argtypes = [c_int]
     L.emu_set_fusion.argtypes = [c_int]
+    L.emu_set_merged.argtypes = [c_int]
+    L.emu_merged_runs.restype = c_long
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
     L.emu_coset_lde_ex.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p, c_long, u64p, c_int]
     return L
 
 
-# (register-blocked passes, scalar-base addressing, fused middle launch of the LDE): every way a pass can run
-MODES = ((1, 1, 1), (1, 1, 0), (1, 0, 0), (0, 0, 0))
+# (register-blocked passes, scalar-base addressing, fused middle launch of the LDE, coset factors split into shifts
+# and per-coset twiddle tables inside that launch): every way a pass can run
+MODES = ((1, 1, 1, 1), (1, 1, 1, 0), (1, 1, 0, 0), (1, 0, 0, 0), (0, 0, 0, 0))
+
+
+def _set_mode(emu, fast, uni, fuse, merged):
+    emu.emu_set_fast(fast)
+    emu.emu_set_uniform(uni)
+    emu.emu_set_fusion(fuse)
+    emu.emu_set_merged(merged)
 
 
 def _p(a):
@@ -86,18 +96,14 @@ def test_ntt_passes_match_oracle(emu, logn, m):
     a = _rand((m, 1 << logn), 100 + logn)
     want = O.ntt_rows(a)
     # register-blocked passes with scalar-base and with per-element addressing, then the generic radix-2 passes
-    for fast, uni, fuse in MODES:
-        emu.emu_set_fast(fast)
-        emu.emu_set_uniform(uni)
-        emu.emu_set_fusion(fuse)
+    for mode in MODES:
+        _set_mode(emu, *mode)
         got = a.copy()
         emu.emu_ntt_batched(_p(got), m, logn, 0)
-        assert np.array_equal(got, want), (fast, uni, fuse)
+        assert np.array_equal(got, want), mode
         emu.emu_ntt_batched(_p(got), m, logn, 1)
-        assert np.array_equal(got, a), (fast, uni, fuse)
-    emu.emu_set_fast(1)
-    emu.emu_set_uniform(1)
-    emu.emu_set_fusion(1)
+        assert np.array_equal(got, a), mode
+    _set_mode(emu, 1, 1, 1, 1)
 
 
 def test_ntt_25_bit_split_is_well_formed(emu):
@@ -113,20 +119,22 @@ def test_ntt_25_bit_split_is_well_formed(emu):
                                            (12, 14, 2, 4096), (13, 15, 2, 5000), (14, 16, 1, 8192),
                                            (16, 18, 1, 65536), (10, 10, 3, 1000), (4, 7, 5, 11),
                                            (10, 12, 5, 1024), (11, 13, 3, 2000), (11, 12, 2, 2048),
-                                           (14, 16, 2, 2816), (12, 14, 3, 257), (16, 18, 1, 4097), (12, 14, 2, 63)])
+                                           (14, 16, 2, 2816), (12, 14, 3, 257), (16, 18, 1, 4097), (12, 14, 2, 63),
+                                           (10, 11, 3, 1024), (12, 13, 2, 3000), (12, 15, 1, 4096), (14, 15, 1, 16384)])
 def test_lde_passes_match_oracle(emu, logK, logN, m, w):
     msgs = _rand((m, w), 200 + logK)
     want = O.coset_lde_rows(msgs, 1 << logK, 1 << logN, 7)
-    for fast, uni, fuse in MODES:
-        emu.emu_set_fast(fast)
-        emu.emu_set_uniform(uni)
-        emu.emu_set_fusion(fuse)
+    for mode in MODES:
+        _set_mode(emu, *mode)
+        before = emu.emu_merged_runs()
         got = np.zeros((m, 1 << logN), dtype=np.uint64)
         emu.emu_coset_lde(_p(msgs), m, w, w, logK, logN, 7, _p(got))
-        assert np.array_equal(got, want), (fast, uni, fuse)
-    emu.emu_set_fast(1)
-    emu.emu_set_uniform(1)
-    emu.emu_set_fusion(1)
+        assert np.array_equal(got, want), mode
+        # K = L * L with L >= 64 (a tile then lies inside one row) and rate 1/2 or 1/4: the fused launch runs, and in
+        # its split form when allowed
+        splits = logK % 2 == 0 and logK >= 12 and 1 <= logN - logK <= 2
+        assert (emu.emu_merged_runs() > before) == (splits and mode == (1, 1, 1, 1)), mode
+    _set_mode(emu, 1, 1, 1, 1)
 
 
 def test_lde_strided_input_and_other_shift(emu):
@@ -148,10 +156,8 @@ def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w
     padded = np.zeros((m, K), dtype=np.uint64)
     padded[:, :w] = msgs
     want_c = O.ntt_rows(padded, inverse=True)
-    for fast, uni, fuse in MODES:
-        emu.emu_set_fast(fast)
-        emu.emu_set_uniform(uni)
-        emu.emu_set_fusion(fuse)
+    for mode in MODES:
+        _set_mode(emu, *mode)
         pitch = K + 3
         co = np.zeros((m, pitch), dtype=np.uint64)
         got = np.zeros((m, N), dtype=np.uint64)
@@ -176,6 +182,4 @@ def test_lde_with_coefficient_output_and_from_coefficients(emu, logK, logN, m, w
         got4 = np.zeros((m, N), dtype=np.uint64)
         emu.emu_coset_lde_ex(_p(full), m, K, K, logK, logN, 7, None, 0, _p(got4), 1)
         assert np.array_equal(got3, got4)
-    emu.emu_set_fast(1)
-    emu.emu_set_uniform(1)
-    emu.emu_set_fusion(1)
+    _set_mode(emu, 1, 1, 1, 1)

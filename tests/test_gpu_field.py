@@ -180,5 +180,7 @@ def test_device_field_primitives_one_by_one():
     assert run(11, xa, ya) == [40 * x * y % P for x, y in zip(xa, ya)]
     for e in range(96):
         assert run(100 + e, canon, canon) == [(x << e) % P for x in canon], e
+    for e in range(192):                                   # 2^96 = -1: the upper half are the negated shifts
+        assert run(300 + e, canon, canon) == [(x << e) % P for x in canon], e
     with pytest.raises(RuntimeError):
         _lib.check(L.vi_gl_probe(99, 0, 0, 0, 1, None))

@@ -65,6 +65,16 @@ __device__ __forceinline__ u64 shift_by(u64 v, int e) {
     }
 }
 
+// the same through the form used inside the coset loop of the fused LDE launch: any exponent below 192, 2^96 = -1
+template <int E>
+__device__ __forceinline__ u64 shift_pinned_by(u64 v, int e) {
+    if constexpr (E >= 192) return 0;
+    else {
+        if (e == E) return gl::mul_pow2c_pinned<E>(v);
+        return shift_pinned_by<E + 1>(v, e);
+    }
+}
+
 __global__ __launch_bounds__(BLOCK) void k_probe(int op, const u64 *a, const u64 *b, u64 *out, i64 n) {
     i64 stride = (i64)gridDim.x * BLOCK;
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) {
@@ -95,6 +105,7 @@ __global__ __launch_bounds__(BLOCK) void k_probe(int op, const u64 *a, const u64
             }
             r = gl::wide_reduce(A);
         }
+        else if (op >= 300) r = shift_pinned_by<0>(x, op - 300);
         else r = shift_by<0>(x, op - 100);
         out[i] = r;
     }
@@ -261,7 +272,7 @@ int vi_gl_axpy(uint64_t *y, uint64_t alpha, const uint64_t *x, int64_t n, void *
 }
 
 int vi_gl_probe(int op, const uint64_t *a, const uint64_t *b, uint64_t *out, int64_t n, void *stream) {
-    const bool shift = op >= 100 && op < 196;
+    const bool shift = (op >= 100 && op < 196) || (op >= 300 && op < 492);
     if (!shift && (op < 0 || op > 11)) return vi::fail(VI_EINVAL, "vi_gl_probe: op = %d", op);
     if (n < 0) return vi::fail(VI_EINVAL, "vi_gl_probe: n = %lld", (long long)n);
     if (n == 0) return VI_OK;

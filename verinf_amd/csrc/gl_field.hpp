@@ -333,22 +333,37 @@ __device__ __forceinline__ void mul_acc(u32 (&w)[5], u64 a, u64 b) {
 }
 
 // canonical v times 2^E, 0 <= E < 96, canonical result; s = 32 q + r moves v into limbs m0 m1 m2 at phi^q
-template <int E>
+// PIN: the three shifts as one asm block.  Plain shifts of a loop-invariant value are hoisted out of a loop even from
+// a branch that is not always taken (they are safe to speculate), and then stay live in registers across it; an asm
+// block stays where it is written.
+// NEG: minus the product, i.e. v times 2^(E + 96); for E >= 32 the last step is a subtraction whose operands swap, so
+// the sign is free.
+template <int E, bool PIN = false, bool NEG = false>
 __device__ __forceinline__ u64 mul_pow2(u64 v) {
     static_assert(E >= 0 && E < 96, "shift out of range");
-    if (E == 0) return v;
+    if (E == 0) return NEG ? sub(0, v) : v;
     constexpr int q = E >> 5, r = E & 31;
     const u32 v0 = (u32)v, v1 = (u32)(v >> 32);
-    const u32 m0 = v0 << r;
-    const u32 m1 = r ? __builtin_amdgcn_alignbit(v1, v0, (32 - r) & 31) : v1;
-    const u32 m2 = r ? (v1 >> ((32 - r) & 31)) : 0u;
+    u32 m0, m1, m2;
+    if constexpr (PIN && r != 0) {
+        asm("v_lshlrev_b32 %[m0], %[r], %[v0]\n\t"
+            "v_alignbit_b32 %[m1], %[v1], %[v0], %[c]\n\t"
+            "v_lshrrev_b32 %[m2], %[c], %[v1]"
+            : [m0] "=&v"(m0), [m1] "=&v"(m1), [m2] "=&v"(m2)
+            : [v0] "v"(v0), [v1] "v"(v1), [r] "n"(r), [c] "n"(32 - r));
+    } else {
+        m0 = v0 << r;
+        m1 = r ? __builtin_amdgcn_alignbit(v1, v0, (32 - r) & 31) : v1;
+        m2 = r ? (v1 >> ((32 - r) & 31)) : 0u;
+    }
     if (q == 0) {
         // m0 + m1 phi + m2 phi^2 = (m1:m0) + m2 (2^32 - 1)
         u64 w, st;
         asm("v_mad_u64_u32 %[w], %[st], %[m2], -1, %[x]"
             : [w] "=&v"(w), [st] "=&s"(st)
             : [m2] "v"(m2), [x] "v"(pack(m0, m1)));
-        return canon_tail((u32)w, (u32)(w >> 32), st);
+        const u64 x = canon_tail((u32)w, (u32)(w >> 32), st);
+        return NEG ? sub(0, x) : x;
     } else if (q == 1) {
         // m0 phi + m1 phi^2 + m2 phi^3 = (m0:0) + m1 (2^32 - 1) - m2
         u64 w, st;
@@ -356,6 +371,7 @@ __device__ __forceinline__ u64 mul_pow2(u64 v) {
             : [w] "=&v"(w), [st] "=&s"(st)
             : [m1] "v"(m1), [x] "v"(pack(0u, m0)));
         const u64 x = canon_tail((u32)w, (u32)(w >> 32), st);
+        if (NEG) return sub((u64)m2, x);                   // m2 = 0 when r = 0
         return r ? sub(x, (u64)m2) : x;
     } else {
         // m0 phi^2 + m1 phi^3 + m2 phi^4 = m0 (2^32 - 1) - (m2:m1); both operands are below p
@@ -366,7 +382,7 @@ __device__ __forceinline__ u64 mul_pow2(u64 v) {
             : [e0] "=&v"(e0), [e1] "=&v"(e1)
             : [m0] "v"(m0)
             : "vcc");
-        return sub(pack(e0, e1), pack(m1, m2));
+        return NEG ? sub(pack(m1, m2), pack(e0, e1)) : sub(pack(e0, e1), pack(m1, m2));
     }
 }
 
@@ -582,6 +598,19 @@ VI_HD u64 mul_pow2c(u64 x) {
     return dev::mul_pow2<E>(x);
 #else
     return mul_pow2(x, (u32)E);
+#endif
+}
+
+// x times 2^E for any exponent (2^192 = 1, 2^96 = -1), for use inside a branch of a loop on a value the loop does
+// not change (see dev::mul_pow2)
+template <int E>
+VI_HD u64 mul_pow2c_pinned(u64 x) {
+    constexpr int e = ((E % 192) + 192) % 192;
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (e < 96) return dev::mul_pow2<e, true, false>(x);
+    else return dev::mul_pow2<e - 96, true, true>(x);
+#else
+    return e < 96 ? mul_pow2(x, (u32)e) : sub(0, mul_pow2(x, (u32)(e - 96)));
 #endif
 }
 

@@ -13,6 +13,7 @@
 //     (layergkr/gpu.py:141-203), with the zero-extension fused into the first
 //     gather and the rho = N/K cosets written interleaved by the last pass, so the
 //     padded (m, N) buffer of the reference recipe is never materialised.
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -135,23 +136,26 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
 #ifndef VI_MID_MIN_WG
 #define VI_MID_MIN_WG 3
 #endif
-template <int A2>
+// MRG: the coset factors split into shift^i (once), a power of two per input, and factors carried by the twiddle
+// tables of each coset (ntt_plan.hpp, append_coset_merged).
+template <int A2, bool MRG>
 __global__ __launch_bounds__(NTHREADS, VI_MID_MIN_WG) void k_lde_mid(const PassArgs Ai_in, const PassArgs Af_in) {
     PassArgs Ai = Ai_in, Af = Af_in;
     Ai.is_final = 1;
     Af.is_final = 0;
     __shared__ u64 lds[TILE + (16 << A2)];
     __shared__ u64 twi_i[16 << A2];
-    __shared__ u64 twi_f[16 << A2];
+    __shared__ u64 twi_f[16 << A2];                        // MRG: the inner twiddles of the coset in hand
     const int tid = threadIdx.x;
     const i64 tile = blockIdx.x;
     constexpr int PER = (16 << A2) / NTHREADS > 0 ? (16 << A2) / NTHREADS : 1;
+    const u64 *src_f = MRG ? Af.twim : Af.twi;
     u64 ti[PER], tf[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const bool in = tid + i * NTHREADS < (16 << A2);
         ti[i] = in ? Ai.twi[tid + i * NTHREADS] : 0;
-        tf[i] = in ? Af.twi[tid + i * NTHREADS] : 0;
+        tf[i] = in ? src_f[tid + i * NTHREADS] : 0;
     }
     u64 reg[16], coef[16];
     u32 ok;
@@ -163,12 +167,20 @@ __global__ __launch_bounds__(NTHREADS, VI_MID_MIN_WG) void k_lde_mid(const PassA
     fast_stage1<A2, true>(Ai, tile, tid, 0, ok, reg, reg, twi_i, lds);         // no pre-multipliers on the inverse side
     __syncthreads();
     fused_stage2_inv<A2>(Ai, tile, tid, lds, coef);
+    if (MRG) fused_twist<A2>(Af, tile, tid, coef);
     const int rho = 1 << Af.log_rho;
     for (int t = 0; t < rho; ++t) {
         __syncthreads();                                   // every thread is done reading the tile of the step before
-        fused_stage1_fwd<A2>(Af, tile, tid, t, coef, twi_f, lds);
+        fused_stage1_fwd<A2, MRG>(Af, tile, tid, t, coef, twi_f, lds);
         __syncthreads();
-        fused_stage2_fwd<A2>(Af, tile, tid, t, lds);
+        fused_stage2_fwd<A2, MRG>(Af, tile, tid, t, lds);
+        // stage 1 of this coset is over everywhere, so its inner twiddles make way for the next coset's (fetched and
+        // stored in one place: held in registers across either stage they cost the kernel its fourth workgroup per CU)
+        if (MRG && t + 1 < rho) {
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+                if (tid + i * NTHREADS < (16 << A2)) twi_f[tid + i * NTHREADS] = src_f[((size_t)(t + 1) << Af.a) + tid + i * NTHREADS];
+        }
     }
 }
 
@@ -279,7 +291,9 @@ int get_pre(int logK, int logN, u64 shift, const u64 **out) {
             g_pre_used.erase(oldest);
         }
         u64 *d = nullptr;
-        int rc = upload(make_coset_pre(logK, logN, shift), &d);
+        std::vector<u64> h = make_coset_pre(logK, logN, shift);
+        if (coset_mergeable(logK, logN)) append_coset_merged(logK, logN, h);
+        int rc = upload(h, &d);
         if (rc) return rc;
         it = g_pre.emplace(key, d).first;
     }
@@ -322,11 +336,20 @@ int launch_fused(const PassArgs &Ai_in, const PassArgs &Af_in, hipStream_t s) {
     const i64 tiles = pass_tiles(Ai);
     if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
     dim3 grid((unsigned)tiles), block(NTHREADS);
-    switch (Ai.a - FAST_A1) {
-        case 1: hipLaunchKernelGGL(k_lde_mid<1>, grid, block, 0, s, Ai, Af); break;
-        case 2: hipLaunchKernelGGL(k_lde_mid<2>, grid, block, 0, s, Ai, Af); break;
-        case 3: hipLaunchKernelGGL(k_lde_mid<3>, grid, block, 0, s, Ai, Af); break;
-        default: hipLaunchKernelGGL(k_lde_mid<4>, grid, block, 0, s, Ai, Af); break;
+    if (Af.twm && Af.twim && Af.merge_unit > 0) {
+        switch (Ai.a - FAST_A1) {
+            case 1: hipLaunchKernelGGL((k_lde_mid<1, true>), grid, block, 0, s, Ai, Af); break;
+            case 2: hipLaunchKernelGGL((k_lde_mid<2, true>), grid, block, 0, s, Ai, Af); break;
+            case 3: hipLaunchKernelGGL((k_lde_mid<3, true>), grid, block, 0, s, Ai, Af); break;
+            default: hipLaunchKernelGGL((k_lde_mid<4, true>), grid, block, 0, s, Ai, Af); break;
+        }
+    } else {
+        switch (Ai.a - FAST_A1) {
+            case 1: hipLaunchKernelGGL((k_lde_mid<1, false>), grid, block, 0, s, Ai, Af); break;
+            case 2: hipLaunchKernelGGL((k_lde_mid<2, false>), grid, block, 0, s, Ai, Af); break;
+            case 3: hipLaunchKernelGGL((k_lde_mid<3, false>), grid, block, 0, s, Ai, Af); break;
+            default: hipLaunchKernelGGL((k_lde_mid<4, false>), grid, block, 0, s, Ai, Af); break;
+        }
     }
     VI_LAUNCH_CHECK("k_lde_mid");
     return VI_OK;
@@ -510,12 +533,15 @@ int coset_lde_impl(const char *who, const uint64_t *in, int64_t m, int64_t width
     if (!rc) rc = get_tables(logK, 0, &Tf);
     if (!rc) rc = get_pre(logK, logN, shift, &pre);
     if (rc) return rc;
+    // the split form of the coset factors: its tables lie behind the N words of pre
+    static const bool use_merged = []() { const char *e = getenv("VI_LDE_MERGED"); return !e || e[0] != '0'; }();
+    const u64 *merged = (use_merged && coset_mergeable(logK, logN)) ? pre + N : nullptr;
     for (i64 lo = 0; lo < m; lo += chunk) {
         i64 cnt = (m - lo < chunk) ? (m - lo) : chunk;
         std::vector<PassArgs> passes;
         build_lde_passes(*Ti, *Tf, pre, logN, in + lo * in_stride, width, in_stride, out ? out + lo * out_stride : nullptr,
                          out_stride, (u64 *)ws, cnt, passes, coeffs ? coeffs + lo * coeffs_stride : nullptr, coeffs_stride,
-                         in_is_coeffs);
+                         in_is_coeffs, true, merged);
         rc = launch_passes(passes, (hipStream_t)stream);
         if (rc) return rc;
     }

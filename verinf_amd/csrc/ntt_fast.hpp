@@ -521,42 +521,89 @@ VI_HD void fused_stage2_inv(const PassArgs &A, i64 tile, int tid, const u64 *lds
 }
 
 
-// Stage 1 and stage 2 of the first forward pass inside the fused launch.  The sixteen coefficients stay live in
-// registers over all cosets there, so the multipliers and twiddles are fetched four at a time, right before use,
-// instead of all sixteen ahead of the tile: other wavefronts cover the latency, and the kernel fits 128 registers.
+// x[n1] = c[n1] * 2^(39 M n1): the part w_N^(t n1 K/16) of the coset factors, M = t * merge_unit (2^96 = -1)
+template <int M>
+VI_HD void coset_shift(const u64 (&c)[16], u64 (&x)[16]) {
+    x[0] = c[0];
+    static_for<1, 16>([&](auto n_) {
+        constexpr int n1 = decltype(n_)::value;
+        constexpr int e = (39 * M * n1) % 192;
+        x[n1] = gl::mul_pow2c_pinned<e>(c[n1]);
+        if constexpr ((n1 & 3) == 3) VI_SCHED_FENCE();
+    });
+}
+
+// MRG: the part of the coset factors that does not depend on the coset, shift^i, applied to the coefficients once
 template <int A2>
-VI_HD void fused_stage1_fwd(const PassArgs &A, i64 tile, int tid, int t, const u64 (&coef)[16], const u64 *twi, u64 *lds) {
+VI_HD void fused_twist(const PassArgs &A, i64 tile, int tid, u64 (&coef)[16]) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
     const TileU U = tile_uniform<A2>(A, tile);
     const u32 off = lane_src_off<A2>(A, U, c, n2);
-    const URun pre = urun(A.pre + ((i64)t << A.logn) + U.pre_u);
-    u64 x[16];
+    const URun pre = urun(A.pre + U.pre_u);                // pre[0][i] = shift^i
 #pragma unroll
     for (int g = 0; g < 16; g += 4) {
         u64 pw[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) pw[j] = uload(pre, (u32)(g + j) << U.sh1, off);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) x[g + j] = gl::mul(coef[g + j], pw[j]);
+        for (int j = 0; j < 4; ++j) coef[g + j] = gl::mul(coef[g + j], pw[j]);
         VI_SCHED_FENCE();
     }
+}
+
+// Stage 1 and stage 2 of the first forward pass inside the fused launch.  The sixteen coefficients stay live in
+// registers over all cosets there, so the multipliers and twiddles are fetched four at a time, right before use,
+// instead of all sixteen ahead of the tile: other wavefronts cover the latency, and the kernel fits 128 registers.
+// MRG: the coefficients already carry shift^i (fused_twist), the coset's own factors are a shift per input here,
+// the inner twiddle table of coset t (twi) and the inter-pass table of coset t in stage 2.
+template <int A2, bool MRG>
+VI_HD void fused_stage1_fwd(const PassArgs &A, i64 tile, int tid, int t, const u64 (&coef)[16], const u64 *twi, u64 *lds) {
+    int c, n2;
+    s1_coords<A2>(A, tid, c, n2);
+    u64 x[16];
+    if constexpr (MRG) {
+        switch (t * A.merge_unit) {                        // the same for every thread of the launch
+            case 1: coset_shift<1>(coef, x); break;
+            case 2: coset_shift<2>(coef, x); break;
+            case 3: coset_shift<3>(coef, x); break;
+            default:
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[i] = coef[i];
+                break;
+        }
+    } else {
+        const TileU U = tile_uniform<A2>(A, tile);
+        const u32 off = lane_src_off<A2>(A, U, c, n2);
+        const URun pre = urun(A.pre + ((i64)t << A.logn) + U.pre_u);
+#pragma unroll
+        for (int g = 0; g < 16; g += 4) {
+            u64 pw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) pw[j] = uload(pre, (u32)(g + j) << U.sh1, off);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[g + j] = gl::mul(coef[g + j], pw[j]);
+            VI_SCHED_FENCE();
+        }
+    }
+    VI_SCHED_FENCE();
     dft_reg<4, false>(x);
     VI_SCHED_FENCE();
     const int st = (1 << logT(A)) + 1;
+    const bool all_k1 = MRG && t > 0;                      // coset t > 0: the k1 = 0 column carries w_N^(t n2 R)
 #pragma unroll
     for (int g = 0; g < 16; g += 4) {
 #pragma unroll
         for (int k1 = g; k1 < g + 4; ++k1) {
             u64 v = x[k1];
-            if (k1 > 0) v = gl::mul(v, twi[n2 * 16 + k1]);
+            if (k1 > 0 || all_k1) v = gl::mul(v, twi[n2 * 16 + k1]);
             lds[((k1 << A2) + n2) * st + c] = v;
         }
         VI_SCHED_FENCE();
     }
 }
 
-template <int A2>
+template <int A2, bool MRG>
 VI_HD void fused_stage2_fwd(const PassArgs &A, i64 tile, int tid, int t, const u64 *lds) {
     constexpr int E2 = 1 << A2;
     constexpr int G = E2 < 4 ? E2 : 4;
@@ -565,7 +612,7 @@ VI_HD void fused_stage2_fwd(const PassArgs &A, i64 tile, int tid, int t, const u
     const int c = tid & ((1 << lt) - 1);
     const TileU U = tile_uniform<A2>(A, tile);
     const URun dst = urun(A.dst + U.dst_u + (i64)t * A.dst_coset_stride);
-    const URun twr = urun(A.tw + U.tw_u);
+    const URun twr = urun(MRG ? A.twm + ((i64)t << A.logn) + U.tw_u : A.tw + U.tw_u);
 #pragma unroll
     for (int i = 0; i < 16 / E2; ++i) {
         const int k1 = (tid + i * NTHREADS) >> lt;

@@ -60,6 +60,10 @@ struct PassArgs {
     int uniform;                              // register-blocked kernel: every tile is addressed by scalar bases (ntt_fast.hpp)
     int n1_valid;                             // uniform pass: how many of a thread's sixteen stage-1 inputs exist
     int fuse_next;                            // last inverse pass of a coset extension: runs fused with the pass after it (dst may be null)
+    // first forward pass inside the fused launch, coset factors split up (null / 0: pre[t] is applied whole):
+    const u64 *twm;                           // [t][(k << logR) + r] = tw[(k << logR) + r] * w_N^(t r)
+    const u64 *twim;                          // [t][n2 * 16 + k1] = twi[n2 * 16 + k1] * w_N^(t n2 R)
+    int merge_unit;                           // w_N^(t n1 K/16) = 2^(39 * merge_unit * t * n1); merge_unit * t <= 3
 };
 
 VI_HD int logT(const PassArgs &A) { return TILE_LOG - A.a; }

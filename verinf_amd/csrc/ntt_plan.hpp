@@ -108,6 +108,41 @@ inline std::vector<u64> make_coset_pre(int logK, int logN, u64 shift) {
     return t;
 }
 
+// The coset factor (shift * w_N^t)^i of coefficient i = n1 K/16 + n2 R + r (first forward pass of K = L * L, R = L)
+// splits into shift^i, w_N^(t r), w_N^(t n2 R) and w_N^(t n1 K/16).  The last is a power of two when 16 rho <= 64
+// (w_64 = 2^39), the second rides on the inter-pass twiddle w_K^(k r) and the third on the inner twiddle
+// w_L^(n2 k1); shift^i does not depend on the coset and is applied once.  Only the fused launch uses this form.
+inline bool coset_mergeable(int logK, int logN) {
+    const Split sp = split_digits(logK);
+    const int log_rho = logN - logK;
+    return sp.p == 2 && sp.a[0] == sp.a[1] && fast_ok(sp.a[0]) && log_rho >= 1 && log_rho <= 2;
+}
+
+// appended behind pre: twm[t][(k << logR) + r] (rho * K words), then twim[t][n2 * 16 + k1] (rho * L words)
+inline void append_coset_merged(int logK, int logN, std::vector<u64> &t) {
+    const int log_rho = logN - logK, a = logK / 2, logR = a;
+    const i64 K = (i64)1 << logK, L = (i64)1 << a, R = (i64)1 << logR, rho = (i64)1 << log_rho;
+    const HostTables H = make_tables(logK, 0);
+    const u64 wN = root_of_unity(logN);
+    const size_t base = t.size();
+    t.resize(base + (size_t)(rho * K + rho * L));
+    u64 *twm = t.data() + base, *twim = twm + rho * K;
+    for (i64 c = 0; c < rho; ++c) {
+        const u64 wc = gl::pow(wN, (u64)c);                // w_N^t
+        std::vector<u64> pr((size_t)R);                    // w_N^(t r)
+        u64 cur = 1;
+        for (i64 r = 0; r < R; ++r) { pr[(size_t)r] = cur; cur = gl::mul(cur, wc); }
+        for (i64 k = 0; k < L; ++k)
+            for (i64 r = 0; r < R; ++r) twm[c * K + (k << logR) + r] = gl::mul(H.tw[0][(size_t)((k << logR) + r)], pr[(size_t)r]);
+        const u64 wr = gl::pow(wc, (u64)R);                // w_N^(t R)
+        u64 pn = 1;                                        // w_N^(t n2 R)
+        for (i64 n2 = 0; n2 < L / FAST_E1; ++n2) {
+            for (int k1 = 0; k1 < FAST_E1; ++k1) twim[c * L + n2 * FAST_E1 + k1] = gl::mul(H.twi[0][(size_t)(n2 * FAST_E1 + k1)], pn);
+            pn = gl::mul(pn, wr);
+        }
+    }
+}
+
 // device (or host) addresses of the tables of one (logn, direction)
 struct Tables {
     Split sp;
@@ -171,12 +206,13 @@ inline i64 lde_ws_elems(int logK, int logN, i64 m) {
 // in -> [inverse passes] -> coefficients -> [forward passes over rho cosets] -> out.
 // The coefficients live in the workspace unless the caller wants them (coeffs != nullptr: the
 // last inverse pass writes them there, row pitch coeffs_stride).  in_is_coeffs skips the
-// inverse passes: `in` already holds coefficients (width w, the rest zero).
+// inverse passes: `in` already holds coefficients (width w, the rest zero).  merged: the tables of
+// append_coset_merged() for this (K, N, shift), used by the fused launch when there is one.
 inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre, int logN,
                              const u64 *in, i64 w, i64 in_stride, u64 *out, i64 out_stride,
                              u64 *ws, i64 m, std::vector<PassArgs> &passes,
                              u64 *coeffs = nullptr, i64 coeffs_stride = 0, bool in_is_coeffs = false,
-                             bool allow_fuse = true) {
+                             bool allow_fuse = true, const u64 *merged = nullptr) {
     const int logK = Ti.logn, log_rho = logN - logK, p = Ti.sp.p;
     const i64 K = (i64)1 << logK;
     u64 *C = coeffs ? coeffs : ws, *S = ws + m * K;
@@ -226,6 +262,11 @@ inline void build_lde_passes(const Tables &Ti, const Tables &Tf, const u64 *pre,
             T1.fuse_next = 1;
             I0 = T0;
             I1 = T1;
+            if (merged && coset_mergeable(logK, logN)) {   // tables of append_coset_merged()
+                F0.twm = merged;
+                F0.twim = merged + (K << log_rho);
+                F0.merge_unit = 4 >> log_rho;
+            }
         }
     }
 }
