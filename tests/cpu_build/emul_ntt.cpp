@@ -34,7 +34,7 @@ Owned *make_owned(int logn, int inv) {
 
 int g_use_fast = 1;
 
-template <int A2, bool INV, bool UNI>
+template <int A2, bool INV, bool UNI, bool HALF = false>
 void run_fast_u(const PassArgs &A) {
     i64 tiles = pass_tiles(A);
     std::vector<u64> lds(fast_lds_words(A.a));
@@ -43,14 +43,14 @@ void run_fast_u(const PassArgs &A) {
     int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
     for (i64 tile = 0; tile < tiles; ++tile) {
         for (int tid = 0; tid < NTHREADS; ++tid)
-            fast_load<A2, UNI>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
+            fast_load<A2, UNI, HALF>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
         for (int t = 0; t < n_loop; ++t) {
             for (int tid = 0; tid < NTHREADS; ++tid)
             {
                 u64 pw[16] = {};
                 if (A.pre) fast_pre_load<A2, UNI>(A, tile, tid, t, pw);
-                fast_stage1<A2, INV>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
-                                     pw, A.twi, lds.data());
+                fast_stage1<A2, INV, HALF>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
+                                           pw, A.twi, lds.data());
             }
             for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds.data());
         }
@@ -59,6 +59,8 @@ void run_fast_u(const PassArgs &A) {
 
 int g_allow_uniform = 1;
 int g_allow_merged = 1;
+int g_allow_half = 1;
+long g_half_runs = 0;                       // first passes that skipped the zero half of their inputs
 long g_merged_runs = 0;                     // fused launches that took the split form of the coset factors
 
 // the same choice the HIP launcher makes: scalar-base addressing when the pass qualifies
@@ -66,7 +68,8 @@ template <int A2, bool INV>
 void run_fast(const PassArgs &A_in) {
     PassArgs A = A_in;
     A.uniform = (g_allow_uniform && pass_uniform(A, &A.n1_valid)) ? 1 : 0;
-    if (A.uniform) run_fast_u<A2, INV, true>(A);
+    if (INV && A.uniform && g_allow_half && upper_half_zero(A)) { ++g_half_runs; run_fast_u<A2, INV, true, true>(A); }
+    else if (A.uniform) run_fast_u<A2, INV, true>(A);
     else run_fast_u<A2, INV, false>(A);
 }
 
@@ -194,6 +197,8 @@ void emu_set_uniform(int on) { g_allow_uniform = on; }
 void emu_set_fusion(int on) { g_allow_fusion = on; }
 void emu_set_merged(int on) { g_allow_merged = on; }
 long emu_merged_runs() { return g_merged_runs; }
+void emu_set_half(int on) { g_allow_half = on; }
+long emu_half_runs() { return g_half_runs; }
 u64 emu_mul(u64 a, u64 b) { return gl::mul(a, b); }
 u64 emu_add(u64 a, u64 b) { return gl::add(a, b); }
 u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }

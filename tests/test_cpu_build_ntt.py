@@ -35,6 +35,8 @@ def emu():
     L.emu_set_fusion.argtypes = [c_int]
     L.emu_set_merged.argtypes = [c_int]
     L.emu_merged_runs.restype = c_long
+    L.emu_set_half.argtypes = [c_int]
+    L.emu_half_runs.restype = c_long
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
     L.emu_coset_lde_ex.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p, c_long, u64p, c_int]
@@ -143,6 +145,28 @@ def test_lde_strided_input_and_other_shift(emu):
     got = np.zeros((6, 256), dtype=np.uint64)
     emu.emu_coset_lde(_p(big), 6, 40, 100, 6, 8, 11, _p(got))
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("logK,w,pruned", [(14, 8192, True), (14, 4096, True), (14, 2816, True), (14, 8193, False),
+                                           (14, 7000, True), (14, 1024, True), (14, 1000, False), (16, 32768, True),
+                                           (16, 32769, False), (16, 100, False), (12, 2048, True), (12, 5, False),
+                                           (16, 4097, True), (13, 2048, True), (13, 4097, False)])
+def test_lde_of_rows_at_most_half_as_wide_as_the_transform(emu, logK, w, pruned):
+    """Source rows that end within the first eight of a thread's sixteen input planes: the first pass does not load
+    the zero half and skips the first butterfly level.  Same codewords with and without, and both equal the oracle's;
+    the counter says whether the pruned form ran (the width must cover at least one whole plane of K/16 words and end
+    within the first eight)."""
+    m = 2
+    msgs = _rand((m, w), 900 + w)
+    want = O.coset_lde_rows(msgs, 1 << logK, 1 << (logK + 2), 7)
+    for half in (1, 0):
+        emu.emu_set_half(half)
+        before = emu.emu_half_runs()
+        got = np.zeros((m, 1 << (logK + 2)), dtype=np.uint64)
+        emu.emu_coset_lde(_p(msgs), m, w, w, logK, logK + 2, 7, _p(got))
+        assert np.array_equal(got, want), half
+        assert (emu.emu_half_runs() > before) == bool(half and pruned), (half, emu.emu_half_runs() - before)
+    emu.emu_set_half(1)
 
 
 @pytest.mark.parametrize("logK,logN,m,w", [(5, 6, 4, 16), (9, 10, 3, 256), (12, 14, 2, 4096), (13, 15, 2, 5000),

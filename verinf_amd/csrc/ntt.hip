@@ -49,7 +49,9 @@ __global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
 // 120 registers).  The strided passes keep the run-time flag: compiled with it fixed to 0 they took 128
 // registers and spilled.
 // UNI: compiled for passes whose tiles are all addressed by scalar bases plus 32-bit thread offsets (pass_uniform).
-template <int A2, bool INV, bool FIN, bool UNI>
+// HALF: the first pass over source rows at most half as wide as the transform (upper_half_zero): eight of a thread's
+// sixteen inputs are zero, so they are not loaded and the first butterfly level of stage 1 is skipped.
+template <int A2, bool INV, bool FIN, bool UNI, bool HALF = false>
 __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     PassArgs A = A_in;
     if (FIN) A.is_final = 1;
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     u64 reg[16], pw[16];
     u32 ok;
     if (A.pre) fast_pre_load<A2, UNI>(A, tile, tid, t, pw);
-    fast_load<A2, UNI>(A, tile, tid, reg, ok);
+    fast_load<A2, UNI, HALF>(A, tile, tid, reg, ok);
     if (!A.is_final) {
         if (lane < count) twi[first + lane] = tw_wave;
         __builtin_amdgcn_wave_barrier();
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
             if (tid + i * NTHREADS < (16 << A2)) twi[tid + i * NTHREADS] = tw_mine[i];
         __syncthreads();
     }
-    fast_stage1<A2, INV>(A, tile, tid, t, ok, reg, pw, twi, lds);
+    fast_stage1<A2, INV, HALF>(A, tile, tid, t, ok, reg, pw, twi, lds);
     __syncthreads();
     fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds);
 }
@@ -316,7 +318,9 @@ template <int A2>
 void launch_fast_a(const PassArgs &A_in, dim3 grid, dim3 block, hipStream_t s) {
     PassArgs A = A_in;
     A.uniform = pass_uniform(A, &A.n1_valid) ? 1 : 0;
-    if (A.uniform) launch_fast_u<A2, true>(A, grid, block, s);
+    if (A.uniform && A.inverse && upper_half_zero(A))
+        hipLaunchKernelGGL((k_ntt_fast<A2, true, false, true, true>), grid, block, 0, s, A);
+    else if (A.uniform) launch_fast_u<A2, true>(A, grid, block, s);
     else launch_fast_u<A2, false>(A, grid, block, s);
 }
 

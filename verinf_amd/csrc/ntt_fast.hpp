@@ -47,7 +47,9 @@ VI_HD constexpr int brev(int i) {
 // in-register transform of 2^A points, natural order in and out; inputs must be
 // canonical, outputs are canonical.  Every exponent is a compile-time constant, so a
 // twiddle is two or three fixed shifts and one fold (gl::mul_pow2c).
-template <int A, bool INV>
+// HALF: the upper half of the inputs, x[N/2 ..], is zero (a source row no wider than half the transform): the first
+// level's butterflies (x[m], x[m + N/2]) -> (sum, difference) are copies.
+template <int A, bool INV, bool HALF = false>
 VI_HD void dft_reg(u64 (&x)[1 << A]) {
     constexpr int N = 1 << A;
     u64 y[N];
@@ -61,7 +63,9 @@ VI_HD void dft_reg(u64 (&x)[1 << A]) {
             constexpr int j = b & (half - 1), i0 = ((b >> s) << (s + 1)) + j, i1 = i0 + half;
             constexpr int e = level_exp<A, INV>(s, j);
             const u64 u = y[i0];
-            if constexpr (e < 96) {
+            if constexpr (HALF && s == 0) {                // y[i1] = x[brev(i0) + N/2] = 0
+                y[i1] = u;
+            } else if constexpr (e < 96) {
                 const u64 v = gl::mul_pow2c<e>(y[i1]);
                 gl::bfly(u, v, y[i0], y[i1]);
             } else {                                   // 2^e = -2^(e-96)
@@ -163,6 +167,14 @@ inline bool pass_uniform(const PassArgs &A, int *n1_valid) {
     return (((i64)1 << A.log_rho) - 1) * A.src_coset_stride + n < ((i64)1 << 29);
 }
 
+// a uniform first pass whose source rows end within the first eight of a thread's sixteen input planes: inputs
+// 8 .. 15 are zero for every thread (A.n1_valid as set by pass_uniform)
+inline bool upper_half_zero(const PassArgs &A) {
+    if (A.is_final || A.pre || A.n1_valid > 8) return false;
+    const int sh1 = (A.a - 4) + A.logR;
+    return A.n1_valid < 8 || A.src_width == ((i64)8 << sh1);
+}
+
 template <int A2>
 VI_HD TileU tile_uniform(const PassArgs &A, i64 tile) {
     TileU U;
@@ -258,26 +270,31 @@ VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
 // the batch, a point past the source width) reads word 0 of the source instead and is zeroed in fast_fix.  With
 // the load inside the test, and the reduction mod p right behind it, every second load waited for the one
 // before -- eight memory round trips per tile instead of one.
-template <int A2, bool UNI>
+// HALF (uniform passes whose source rows end within the first eight planes, upper_half_zero()): inputs 8 .. 15 are
+// not loaded.
+template <int A2, bool UNI, bool HALF = false>
 VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &ok) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
     if constexpr (UNI) {
+        constexpr int NL = HALF ? 8 : 16;
         const TileU U = tile_uniform<A2>(A, tile);
         const u32 off = lane_src_off<A2>(A, U, c, n2);
         // an input past the source width reads input 0 instead (and is zeroed in fast_fix): the choice is the same
         // for every thread, so it is made on the scalar base
         const URun src = urun(A.src + U.src_u);
 #pragma unroll
-        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = uload(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off);
+        for (int n1 = 0; n1 < NL; ++n1) reg[n1] = uload(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off);
+#pragma unroll
+        for (int n1 = NL; n1 < 16; ++n1) reg[n1] = 0;
         ok = A.n1_valid >= 16 ? 0xFFFFu : ((1u << A.n1_valid) - 1u);
-        if (A.n1_valid < 16) {
+        if (A.n1_valid < NL) {
             // the plane the width ends in: this thread's input there exists if its offset is below the remainder
             const u32 rem = (u32)(A.src_width - ((i64)A.n1_valid << U.sh1));
             const bool mine = (u32)U.pre_u + off < rem;           // pre_u: index of the tile's first column inside the row
             const u64 v = uload(src, 0u, mine ? off + ((u32)A.n1_valid << U.sh1) : 0u);     // the others read word 0 of the tile
 #pragma unroll
-            for (int n1 = 0; n1 < 16; ++n1) reg[n1] = (n1 == A.n1_valid) ? v : reg[n1];
+            for (int n1 = 0; n1 < NL; ++n1) reg[n1] = (n1 == A.n1_valid) ? v : reg[n1];
             ok |= mine ? (1u << A.n1_valid) : 0u;
         }
         return;
@@ -295,16 +312,18 @@ VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &
 }
 
 // zero for the elements that do not exist, caller data reduced mod p
+template <bool HALF = false>
 VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
+    constexpr int NL = HALF ? 8 : 16;                      // HALF: inputs 8 .. 15 are zeros already
     // both as blocks behind one test each, so that the passes that need neither (all elements there, source
     // written by an earlier pass) skip them: as per-element selects they ran in every pass
-    if (ok != 0xFFFFu) {
+    if (ok != (HALF ? 0xFFu : 0xFFFFu)) {
 #pragma unroll
-        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = ((ok >> n1) & 1) ? reg[n1] : 0;
+        for (int n1 = 0; n1 < NL; ++n1) reg[n1] = ((ok >> n1) & 1) ? reg[n1] : 0;
     }
     if (A.canon_src) {
 #pragma unroll
-        for (int n1 = 0; n1 < 16; ++n1) reg[n1] = gl::canon(reg[n1]);
+        for (int n1 = 0; n1 < NL; ++n1) reg[n1] = gl::canon(reg[n1]);
     }
 }
 
@@ -332,7 +351,7 @@ VI_HD void fast_pre_load(const PassArgs &A, i64 tile, int tid, int t_loop, u64 (
     for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[R.valid ? (i64)((n1 << A2) + n2) << sh : 0];
 }
 
-template <int A2, bool INV>
+template <int A2, bool INV, bool HALF = false>
 VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok, const u64 (&reg)[16],
                        const u64 (&pw)[16], const u64 *twi, u64 *lds) {
     int c, n2;
@@ -340,7 +359,7 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok,
     u64 x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = reg[i];
-    fast_fix(A, ok, x);
+    fast_fix<HALF>(A, ok, x);
     if (A.pre) {
 #pragma unroll
         for (int g = 0; g < 16; g += 4) {
@@ -350,7 +369,7 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok,
         }
     }
     VI_SCHED_FENCE();
-    dft_reg<4, INV>(x);
+    dft_reg<4, INV, HALF>(x);
     VI_SCHED_FENCE();
     const int st = (1 << logT(A)) + 1;
 #pragma unroll
