@@ -98,10 +98,10 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     } else {
 #pragma unroll
         for (int i = 0; i < (int)(sizeof(tw_mine) / sizeof(u64)); ++i)
-            if (tid + i * NTHREADS < (16 << A2)) twi[tid + i * NTHREADS] = tw_mine[i];
+            if (tid + i * NTHREADS < (16 << A2)) twi[twi_slot<A2, FIN>((tid + i * NTHREADS) >> 4, (tid + i * NTHREADS) & 15)] = tw_mine[i];
         __syncthreads();
     }
-    fast_stage1<A2, INV, HALF>(A, tile, tid, t, ok, reg, pw, twi, lds);
+    fast_stage1<A2, INV, HALF, FIN>(A, tile, tid, t, ok, reg, pw, twi, lds);
     __syncthreads();
     fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds);
 }
@@ -125,9 +125,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
     if (A.pre) fast_pre_load<A2, false>(A, tile, tid, 0, pw);
     fast_load<A2, false>(A, tile, tid, reg, ok);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) twi[tid + i * NTHREADS] = tw_mine[i];
+    for (int i = 0; i < 2; ++i) twi[twi_slot<A2, true>((tid + i * NTHREADS) >> 4, (tid + i * NTHREADS) & 15)] = tw_mine[i];
     __syncthreads();
-    fast_stage1<A2, INV>(A, tile, tid, 0, ok, reg, pw, twi, lds);
+    fast_stage1<A2, INV, false, true>(A, tile, tid, 0, ok, reg, pw, twi, lds);
     __syncthreads();
     fast_stage2_512<INV>(A, tile, tid, lds);
 }
@@ -164,9 +164,12 @@ __global__ __launch_bounds__(NTHREADS, VI_MID_MIN_WG) void k_lde_mid(const PassA
     fast_load<A2, true>(Ai, tile, tid, reg, ok);
 #pragma unroll
     for (int i = 0; i < PER; ++i)
-        if (tid + i * NTHREADS < (16 << A2)) { twi_i[tid + i * NTHREADS] = ti[i]; twi_f[tid + i * NTHREADS] = tf[i]; }
+        if (tid + i * NTHREADS < (16 << A2)) {
+            twi_i[twi_slot<A2, true>((tid + i * NTHREADS) >> 4, (tid + i * NTHREADS) & 15)] = ti[i];
+            twi_f[tid + i * NTHREADS] = tf[i];
+        }
     __syncthreads();
-    fast_stage1<A2, true>(Ai, tile, tid, 0, ok, reg, reg, twi_i, lds);         // no pre-multipliers on the inverse side
+    fast_stage1<A2, true, false, true>(Ai, tile, tid, 0, ok, reg, reg, twi_i, lds);   // no pre-multipliers on the inverse side
     __syncthreads();
     fused_stage2_inv<A2>(Ai, tile, tid, lds, coef);
     if (MRG) fused_twist<A2>(Af, tile, tid, coef);

@@ -327,6 +327,13 @@ VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
     }
 }
 
+// Where w_L^(n2 k1) sits in a workgroup's LDS copy of the inner twiddle table.  In a final pass consecutive lanes
+// hold consecutive n2, and the table's own order [n2][k1] would put sixteen lanes on two LDS banks, so the kernels
+// keep the copy of a final pass as [k1][n2] (TWT); in a strided pass sixteen lanes share one n2 (a broadcast) and
+// the order stays.
+template <int A2, bool TWT>
+VI_HD constexpr int twi_slot(int n2, int k1) { return TWT ? (k1 << A2) + n2 : n2 * 16 + k1; }
+
 // phase 2: optional coset pre-multiplier, 16-point transform, w_L^(n2 k1), into LDS
 // twi: w_L^(n2 k1) at [n2 * 16 + k1]
 // the coset pre-multipliers of this thread's sixteen inputs (a column that does not exist takes those of
@@ -351,7 +358,7 @@ VI_HD void fast_pre_load(const PassArgs &A, i64 tile, int tid, int t_loop, u64 (
     for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[R.valid ? (i64)((n1 << A2) + n2) << sh : 0];
 }
 
-template <int A2, bool INV, bool HALF = false>
+template <int A2, bool INV, bool HALF = false, bool TWT = false>
 VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok, const u64 (&reg)[16],
                        const u64 (&pw)[16], const u64 *twi, u64 *lds) {
     int c, n2;
@@ -377,7 +384,7 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok,
 #pragma unroll
         for (int k1 = g; k1 < g + 4; ++k1) {
             u64 v = x[k1];
-            if (k1 > 0) v = gl::mul(v, twi[n2 * 16 + k1]);
+            if (k1 > 0) v = gl::mul(v, twi[twi_slot<A2, TWT>(n2, k1)]);
             lds[((k1 << A2) + n2) * st + c] = v;
         }
         VI_SCHED_FENCE();
