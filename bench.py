@@ -36,11 +36,11 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 # launches of a step, like roofline.achieved.
 LDE_TRAFFIC_BYTES_PER_STEP = 8.06e9
 # VALU wave-instructions one LDE step issues (rocprofv3 --pmc SQ_INSTS_VALU, same profile: per 512-row chunk 58.7 M in
-# the strided inverse launch, 296.9 M in k_lde_mid and 188.0 M in the final forward launch) and the rate at which
+# the strided inverse launch, 290.1 M in k_lde_mid and 188.1 M in the final forward launch) and the rate at which
 # 1024 SIMDs issue the instruction classes these kernels consist of (carry, multiply, three-operand and shift
 # instructions: one per 4.16 cycles per SIMD, measured by `bench.py --valu-probe`,
 # profiles/valu_issue_rates__probe.md) at the 2.4 GHz peak clock
-LDE_VALU_INSTS_PER_STEP = 2 * (58_687_488 + 296_878_080 + 187_957_248)
+LDE_VALU_INSTS_PER_STEP = 2 * (58_687_488 + 290_062_336 + 188_088_320)
 VALU_ISSUE_CYCLES_PER_INSTR = 4.16
 VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / VALU_ISSUE_CYCLES_PER_INSTR
 

@@ -109,7 +109,10 @@ int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, 
  * width = 0 is the zero polynomial: zero rows are written and `in` is not read.
  * The workspace may be smaller than vi_coset_lde_workspace_bytes(m, K, N): rows
  * are then processed in chunks; vi_coset_lde_min_workspace_bytes(K, N) is the
- * least that is accepted (one row). */
+ * least that is accepted (one row).
+ * Environment: VI_LDE_MERGED=0 (read once per process) makes the fused middle launch apply the coset factors
+ * (shift * w_N^t)^i as one multiplication per coefficient and coset instead of split into shift^i, a power of two
+ * and per-coset twiddle tables; same results, for measurements only. */
 size_t vi_coset_lde_workspace_bytes(int64_t m, int64_t K, int64_t N);
 size_t vi_coset_lde_min_workspace_bytes(int64_t K, int64_t N);
 /* Number of kernel launches one vi_coset_lde call with these arguments issues
