@@ -71,6 +71,13 @@ def test_coefficients_and_codewords_in_one_call(cp, K, N, m, w):
     assert np.array_equal(to_np(code), want)
     co2, none = cp.coset_lde_with_coeffs(to_dev(msgs), K, N, 7, need_codewords=False)
     assert none is None and np.array_equal(to_np(co2), want_c)
+    # in place: the padded matrix becomes the coefficients (what encode_messages does with its own buffer)
+    own = to_dev(padded)
+    co3, code3 = cp.coset_lde_with_coeffs(own, K, N, 7, in_place=True)
+    assert co3.data_ptr() == own.data_ptr() and np.array_equal(to_np(own), want_c) and np.array_equal(to_np(code3), want)
+    if w < K:
+        with pytest.raises(RuntimeError):
+            cp.coset_lde_with_coeffs(to_dev(msgs), K, N, 7, in_place=True)     # not (m, K)
     # the reference's two-step form gives the same coefficients
     ref = to_dev(padded)
     cp.ntt_inverse_batched(ref)

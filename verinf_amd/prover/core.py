@@ -5,8 +5,8 @@ encoder `_coset_encode_codewords` (:702-743), served by the fused device pipelin
 The reference builds `padded = [message | row_prg pad]`, clones it, runs the inverse
 NTT for the row polynomials, multiplies by materialised powers of the coset shift,
 copies into a zeroed (m, N) buffer and runs the forward NTT.  Here the pad is
-generated straight into the padded matrix and ONE library call turns it into both the
-row polynomials and the codewords; no (m, N) staging buffer, no expanded powers.
+generated straight into the padded matrix and ONE library call turns that matrix, in place, into
+the row polynomials and writes the codewords; no clone, no (m, N) staging buffer, no expanded powers.
 Everything else of that module (the interactive protocol, blinding rows, openings)
 is outside this package.
 """
@@ -92,6 +92,7 @@ def encode_messages(messages: torch.Tensor, cfg: LigeroConfig, *, master_seed: t
         padded = torch.empty((m, cfg.K_DEG), dtype=torch.uint64, device=messages.device)
         padded.view(torch.int64)[:, :cfg.ELL] = messages.view(torch.int64)
         row_prg(master_seed, row_offset, m, slack, out=padded[:, cfg.ELL:])
-    else:
-        padded = messages
-    return coset_lde_with_coeffs(padded, cfg.K_DEG, cfg.N_LIG, cfg.coset_shift, need_codewords=need_codewords)
+        # `padded` is ours: the row polynomials take its place
+        return coset_lde_with_coeffs(padded, cfg.K_DEG, cfg.N_LIG, cfg.coset_shift, need_codewords=need_codewords,
+                                     in_place=True)
+    return coset_lde_with_coeffs(messages, cfg.K_DEG, cfg.N_LIG, cfg.coset_shift, need_codewords=need_codewords)

@@ -235,13 +235,20 @@ def coset_lde(messages, k_deg, n_lig, shift=GLOBAL_G, out=None):
     return out
 
 
-def coset_lde_with_coeffs(messages, k_deg, n_lig, shift=GLOBAL_G, need_codewords=True, out=None):
+def coset_lde_with_coeffs(messages, k_deg, n_lig, shift=GLOBAL_G, need_codewords=True, out=None, in_place=False):
     """As coset_lde, but also returns the row polynomials the pipeline passes through:
     (coeffs (m, K), codewords (m, N) or None).  One call stands for
     `row_polys = padded.clone(); ntt_inverse_batched(row_polys); _coset_encode_codewords(row_polys)`
-    (prover/core.py:795-802); need_codewords=False stops after the coefficients."""
+    (prover/core.py:795-802); need_codewords=False stops after the coefficients.
+    in_place: `messages` is a contiguous (m, K) tensor the caller gives up; the coefficients overwrite it and it is
+    returned as `coeffs` (the reference's clone has no counterpart then)."""
     k_deg, n_lig, m, w, in_stride = _lde_args(messages, k_deg, n_lig)
-    coeffs = torch.empty((m, k_deg), dtype=torch.uint64, device=messages.device)
+    if in_place:
+        if w != k_deg or in_stride != k_deg:
+            raise RuntimeError("coset_lde_with_coeffs(in_place=True) needs a contiguous (m, K_DEG) tensor")
+        coeffs = messages
+    else:
+        coeffs = torch.empty((m, k_deg), dtype=torch.uint64, device=messages.device)
     out = _lde_out(out, m, n_lig, messages.device) if need_codewords else None
     if m == 0:
         return coeffs, out
