@@ -136,7 +136,11 @@ def test_lde_golden(cp, golden_dir):
                                            (9, 10, 3, 256), (10, 10, 3, 1000), (10, 12, 7, 1024), (11, 13, 3, 2000), (4, 7, 5, 11), (12, 14, 16, 4096),
                                            (13, 15, 5, 5000), (14, 16, 9, 8192), (16, 18, 5, 65536),
                                            (16, 17, 3, 40000), (17, 19, 2, 1 << 17), (18, 20, 2, 200000), (20, 22, 1, 1 << 20),
-                                           (8, 14, 3, 256), (12, 18, 2, 4000)])
+                                           (8, 14, 3, 256), (12, 18, 2, 4000),
+                                           # rows at most half as wide as the transform (the first pass skips the zero
+                                           # half), with and without a partly filled plane; rate 1/2 in the fused launch
+                                           (14, 16, 3, 2816), (14, 16, 2, 4096), (16, 18, 2, 4097), (16, 18, 1, 32768),
+                                           (12, 13, 3, 2048), (14, 15, 2, 16384), (13, 15, 2, 2048)])
 def test_lde_matches_oracle(cp, logK, logN, m, w):
     msgs = rand_field((m, w), 200 + logK)
     got = cp.coset_lde(to_dev(msgs), 1 << logK, 1 << logN, 7)
