@@ -67,6 +67,11 @@ VI_PROBE_KERNEL(k_lshr, asm volatile("v_lshrrev_b32 %0, 3, %0\n v_lshrrev_b32 %1
 VI_PROBE_KERNEL(k_mov, asm volatile("v_mov_b32 %0, %1\n v_mov_b32 %1, %2\n v_mov_b32 %2, %3\n v_mov_b32 %3, %0" : VI_A32);)
 VI_PROBE_KERNEL(k_min, asm volatile("v_min_u32 %0, %0, %1\n v_min_u32 %1, %1, %2\n v_min_u32 %2, %2, %3\n v_min_u32 %3, %3, %0" : VI_A32);)
 VI_PROBE_KERNEL(k_cmp_u32, asm volatile("v_cmp_lt_u32 vcc, %0, %1\n v_cmp_lt_u32 vcc, %1, %2\n v_cmp_lt_u32 vcc, %2, %3\n v_cmp_lt_u32 vcc, %3, %0" : VI_A32 : : "vcc");)
+VI_PROBE_KERNEL(k_lshl_b64, asm volatile("v_lshlrev_b64 %0, 3, %0\n v_lshlrev_b64 %1, 5, %1\n v_lshlrev_b64 %2, 7, %2\n v_lshlrev_b64 %3, 9, %3" : VI_D64);)
+VI_PROBE_KERNEL(k_lshr_b64, asm volatile("v_lshrrev_b64 %0, 3, %0\n v_lshrrev_b64 %1, 5, %1\n v_lshrrev_b64 %2, 7, %2\n v_lshrrev_b64 %3, 9, %3" : VI_D64);)
+VI_PROBE_KERNEL(k_subb_co, asm volatile("v_subb_co_u32 %0, vcc, %0, %1, vcc\n v_subb_co_u32 %1, vcc, %1, %2, vcc\n v_subb_co_u32 %2, vcc, %2, %3, vcc\n v_subb_co_u32 %3, vcc, %3, %0, vcc" : VI_A32 : : "vcc");)
+VI_PROBE_KERNEL(k_bfe, asm volatile("v_bfe_u32 %0, %0, 3, 20\n v_bfe_u32 %1, %1, 5, 20\n v_bfe_u32 %2, %2, 7, 20\n v_bfe_u32 %3, %3, 9, 20" : VI_A32);)
+VI_PROBE_KERNEL(k_lshl_or, asm volatile("v_lshl_or_b32 %0, %0, 3, %1\n v_lshl_or_b32 %1, %1, 5, %2\n v_lshl_or_b32 %2, %2, 7, %3\n v_lshl_or_b32 %3, %3, 9, %0" : VI_A32);)
 VI_PROBE_KERNEL(k_perm, asm volatile("v_perm_b32 %0, %0, %1, %2\n v_perm_b32 %1, %1, %2, %3\n v_perm_b32 %2, %2, %3, %0\n v_perm_b32 %3, %3, %0, %1" : VI_A32);)
 // how double-rate instructions behave next to others: a dependent chain, alternation with a full-rate class,
 // and pairs of each class
@@ -141,6 +146,8 @@ const Probe PROBES[] = {
     {"v_lshlrev_b32", k_lshl, 256},         {"v_lshrrev_b32", k_lshr, 256},        {"v_mov_b32", k_mov, 256},
     {"v_min_u32", k_min, 256},              {"v_cmp_lt_u32", k_cmp_u32, 256},
     {"v_perm_b32", k_perm, 256},
+    {"v_lshlrev_b64", k_lshl_b64, 256},     {"v_lshrrev_b64", k_lshr_b64, 256},
+    {"v_subb_co_u32", k_subb_co, 256},      {"v_bfe_u32", k_bfe, 256},             {"v_lshl_or_b32", k_lshl_or, 256},
     {"v_xor_b32, each reads the one before", k_xor_dependent, 256},
     {"v_xor_b32 / v_alignbit_b32 alternating", k_xor_align_alternating, 256},
     {"v_xor_b32 x2 / v_alignbit_b32 x2", k_xor_align_pairs, 256},
