@@ -121,7 +121,7 @@ def cpu_baseline_lde(torch, msgs, out, rows, reps):
             "bit_exact_vs_gpu": bool(np.array_equal(got, want))}
 
 
-def _time_proof(torch, gpu, terms, coin, reps=8):
+def _time_proof(torch, gpu, terms, coin, reps=24):
     """-> (best wall ms incl. the read-back of the samples, best device ms by HIP events) of prove_terms_gpu"""
     wall, dev = [], []
     s, e = _events(torch)
@@ -266,7 +266,8 @@ def bench_kquant(torch, steps=20, cpu=True):
     raw = torch.randint(0, 256, (nb, 144), generator=g, dtype=torch.uint8, device="cuda")
     hd = (torch.randn((nb, 2), generator=g, device="cuda") * 0.01).abs().to(torch.float16).view(torch.uint8)
     raw[:, 0:4] = hd.reshape(nb, 4)
-    for _ in range(3):
+    # a launch is 60 us: enough of them before the clock starts that the chip is out of its idle power state
+    for _ in range(3 * steps):
         kq.kquant_to_field(raw, "Q4_K", 4096)
     torch.cuda.synchronize()
     s, e = _events(torch)
@@ -284,7 +285,8 @@ def bench_kquant(torch, steps=20, cpu=True):
             other[:, 208:210] = hd.reshape(nb, 4)[:, :2]
         else:
             other[:, 0:4] = hd.reshape(nb, 4)
-        kq.kquant_to_field(other, qt, 4096)
+        for _ in range(3 * steps):
+            kq.kquant_to_field(other, qt, 4096)
         torch.cuda.synchronize()
         s.record()
         for _ in range(steps):
@@ -331,21 +333,21 @@ def bench_hash(torch, steps=10, cpu=True):
     m, n = 1024, 1 << 18
     g = torch.Generator(device="cuda").manual_seed(9)
     mat = torch.randint(-(1 << 63), (1 << 63) - 1, (m, n), generator=g, dtype=torch.int64, device="cuda").view(torch.uint64)
-    for _ in range(2):
+    for _ in range(steps):                              # ~10 ms of the same work before the clock starts
         dig = cp.hash_columns_streamed(mat)
         root, _ = cp.merkle_build_blake3(dig)
     torch.cuda.synchronize()
-    s, e, e2 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t_hash = t_tree = 0.0
-    for _ in range(steps):
-        s.record()
+    # the steps are queued back to back (no host wait in between) with an event after each part
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for i in range(steps):
+        ev[i][0].record()
         dig = cp.hash_columns_streamed(mat)
-        e.record()
+        ev[i][1].record()
         root, _ = cp.merkle_build_blake3(dig)
-        e2.record()
-        torch.cuda.synchronize()
-        t_hash += s.elapsed_time(e)
-        t_tree += e.elapsed_time(e2)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    t_hash = sum(a.elapsed_time(b) for a, b, _ in ev)
+    t_tree = sum(b.elapsed_time(c) for _, b, c in ev)
     hash_ms, tree_ms = t_hash / steps, t_tree / steps
     alg = 8 * m * n + 32 * n
     res = {"matrix": "1024 x 2^18 uint64", "hash_columns_ms": hash_ms, "hash_gbs_algorithmic": alg / hash_ms / 1e6,
