@@ -368,6 +368,36 @@ def bench_hash(torch, steps=10, cpu=True):
     return res
 
 
+def bench_ntt(torch, steps=20):
+    """ntt_forward_batched / ntt_inverse_batched (prover/cuda_primitives.py:388-409) over 2^26 points as rows of
+    2^8 ... 2^20: in place, round trip checked."""
+    from verinf_amd.prover import cuda_primitives as cp
+    res = {}
+    for logn in (8, 9, 12, 16, 20):
+        rows = rand_field(torch, (1 << (26 - logn), 1 << logn), 40 + logn)
+        keep = rows.clone()
+        for _ in range(steps):
+            cp.ntt_forward_batched(rows)
+            cp.ntt_inverse_batched(rows)
+        torch.cuda.synchronize()
+        s, e = _events(torch)
+        s.record()
+        for _ in range(steps):
+            cp.ntt_forward_batched(rows)
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / steps
+        for _ in range(steps):
+            cp.ntt_inverse_batched(rows)
+        torch.cuda.synchronize()
+        res[f"rows_of_2^{logn}"] = {"forward_ms": ms, "points_per_s": (1 << 26) / (ms * 1e-3),
+                                    "gbs_algorithmic": 16 * (1 << 26) / (ms * 1e-3) / 1e9,
+                                    "round_trip_is_identity": bool(torch.equal(rows, keep))}
+        del rows, keep
+        torch.cuda.empty_cache()
+    return res
+
+
 def bench_layer(torch, check=True):
     """Config 5: one Llama-2-7B-shape layer proof core.  Commit = coset LDE of every weight
     and activation row at the production geometry ELL = 8192, K = 2^14, N = 2^16 (a row of
@@ -640,7 +670,7 @@ def main():
     ap.add_argument("--copy-probe", action="store_true")
     ap.add_argument("--valu-probe", action="store_true", help="issue rate of the integer VALU instruction classes")
     ap.add_argument("--ws-mb", type=int, default=0, help="override the LDE workspace size (MiB); 0 = library default")
-    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer", "hash", "gatebatch"], default=None,
+    ap.add_argument("--only", choices=["sumcheck", "kquant", "layer", "hash", "gatebatch", "ntt"], default=None,
                     help="run just one of the extra legs and print its JSON (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -669,6 +699,9 @@ def main():
         return
     if args.only == "gatebatch":
         print(json.dumps(bench_gate_batch(torch)))
+        return
+    if args.only == "ntt":
+        print(json.dumps(bench_ntt(torch)))
         return
 
     lde, msgs, out = bench_lde(torch, args.steps, args.warmup, args.ws_mb)
