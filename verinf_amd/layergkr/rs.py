@@ -130,7 +130,23 @@ class Commit:
     (the `mat=` branch of rs.py:176-187).  Hashing happens on first use of `root`,
     `levels` or `open`, so callers that only encode and combine do not pay for it."""
 
-    def __init__(self, cfg: Config, mat):
+    def __init__(self, cfg: Config, codewords=None, mat=None):
+        """`codewords`: rows as Python lists (the reference's host backend, rs.py:176-193; here they are uploaded
+        and committed on the device like any other matrix) or a device tensor; `mat=`: the (rows, N_LIG) device
+        tensor of the reference's device backend."""
+        if mat is None:
+            if codewords is None:
+                raise ValueError("Commit needs codewords or mat")
+            mat = codewords
+        if not isinstance(mat, torch.Tensor):
+            from . import gpu
+            if not gpu.available():
+                raise RuntimeError("verinf_amd.rs.Commit needs a GPU (there is no CPU fallback)")
+            rows = [[int(v) % P for v in row] for row in mat]
+            if any(len(row) != cfg.N_LIG for row in rows):
+                raise ValueError("a codeword has N_LIG entries")
+            signed = [[v - (1 << 64) if v >= (1 << 63) else v for v in row] for row in rows]
+            mat = torch.tensor(signed, dtype=torch.int64, device="cuda").view(torch.uint64).reshape(len(rows), cfg.N_LIG)
         self.cfg = cfg
         self.mat = mat
         self._root = None
