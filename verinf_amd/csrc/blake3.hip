@@ -9,7 +9,7 @@
 // other way: k_chunk_cvs gives every (1 KiB chunk, column) pair its own thread -- lanes
 // run along the columns, so the eight 8-byte loads of a 64-byte block are each one
 // coalesced 512-byte wavefront access -- and stores the chunk's chaining value;
-// k_merge_level then halves the number of chaining values per launch.  Pairing adjacent
+// k_merge_levels then quarters the number of chaining values per launch.  Pairing adjacent
 // nodes and carrying an odd last node up unchanged reproduces BLAKE3's left-full tree,
 // and the last merge carries the ROOT flag.  The chunk stage is therefore a streaming
 // pass over the matrix with as many independent threads as the GPU wants, and it can be
@@ -112,27 +112,45 @@ __global__ __launch_bounds__(BLOCK) void k_chunk_cvs(const u64 *__restrict__ row
     for (int i = 0; i < 8; ++i) o[i] = cv[i];
 }
 
-// One level of BLAKE3's internal tree over `count` nodes per column: node pairs (2i, 2i+1)
-// become a parent, an odd last node moves up unchanged.  in/out: [node][col][8 words].
-__global__ __launch_bounds__(BLOCK) void k_merge_level(const u32 *__restrict__ in, i64 count, i64 n, int is_root_level,
-                                                       u32 *__restrict__ out) {
+// BLAKE3's internal tree over `count` nodes per column, LV levels per launch: node pairs (2i, 2i+1) become a parent,
+// an odd last node moves up unchanged.  in/out: [node][col][8 words].  The thread of (column, i) forms node i of
+// level LV above the input level from the up to 2^LV input nodes under it (2^LV - 1 compressions, the lower ones
+// first), so the levels in between are never written.  cnt[j] = nodes of level j (cnt[0] = count of the input
+// level); the merge of the last two nodes of a level is the root.
+template <int LV>
+__device__ __forceinline__ void merge_node(const u32 *__restrict__ in, i64 n, i64 col, i64 idx, const i64 (&cnt)[4], u32 (&o)[8]) {
+    if constexpr (LV == 0) {
+        const u32 *p = in + (idx * n + col) * 8;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o[k] = p[k];
+    } else {
+        if (2 * idx + 1 >= cnt[LV - 1]) {
+            merge_node<LV - 1>(in, n, col, 2 * idx, cnt, o);
+            return;
+        }
+        u32 l[8], r[8], m[16];
+        merge_node<LV - 1>(in, n, col, 2 * idx, cnt, l);
+        merge_node<LV - 1>(in, n, col, 2 * idx + 1, cnt, r);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { m[k] = l[k]; m[8 + k] = r[k]; o[k] = IV[k]; }
+        compress(o, m, 0, 64, PARENT | (cnt[LV - 1] == 2 ? ROOT : 0u));
+    }
+}
+
+template <int LV>
+__global__ __launch_bounds__(BLOCK) void k_merge_levels(const u32 *__restrict__ in, i64 count, i64 n, i64 idx0, u32 *__restrict__ out) {
     const i64 col = (i64)blockIdx.x * BLOCK + threadIdx.x;
     if (col >= n) return;
-    const i64 i = blockIdx.y;                       // parent index
-    const u32 *l = in + ((2 * i) * n + col) * 8;
-    u32 *o = out + (i * n + col) * 8;
-    if (2 * i + 1 >= count) {
+    i64 cnt[4];
+    cnt[0] = count;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) o[k] = l[k];
-        return;
-    }
-    const u32 *r = in + ((2 * i + 1) * n + col) * 8;
-    u32 m[16], cv[8];
+    for (int j = 1; j < 4; ++j) cnt[j] = (cnt[j - 1] + 1) / 2;
+    const i64 i = idx0 + blockIdx.y;
+    u32 o[8];
+    merge_node<LV>(in, n, col, i, cnt, o);
+    u32 *dst = out + (i * n + col) * 8;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { m[k] = l[k]; m[8 + k] = r[k]; cv[k] = IV[k]; }
-    compress(cv, m, 0, 64, PARENT | (is_root_level ? ROOT : 0u));
-#pragma unroll
-    for (int k = 0; k < 8; ++k) o[k] = cv[k];
+    for (int k = 0; k < 8; ++k) dst[k] = o[k];
 }
 
 // Merkle level over 32-byte nodes: parent i = BLAKE3(node[2i] || node[2i+1]), the odd last
@@ -354,19 +372,30 @@ int vi_hash_columns_finalize(int64_t n, int64_t n_chunks_total, void *ws, size_t
     u32 *a = (u32 *)ws;                               // n_chunks_total nodes
     u32 *b = a + (size_t)n_chunks_total * n * 8;      // ceil(n_chunks_total / 2) nodes
     i64 count = n_chunks_total;
+    if (count == 1) {
+        VI_HIP(hipMemcpyAsync(digests, a, (size_t)n * 32, hipMemcpyDeviceToDevice, s));
+        return VI_OK;
+    }
+    // MERGE_LEVELS levels of the tree per launch; the launch that reaches the root writes the digests themselves
+    // (through a copy when the caller's buffer is not word-aligned)
+    constexpr int MERGE_LEVELS = 2;
+    const bool direct = ((uintptr_t)digests & 3) == 0;
     while (count > 1) {
-        const i64 parents = (count + 1) / 2;
-        for (i64 lo = 0; lo < parents; lo += 65535) {             // grid.y limit
-            const i64 cnt = parents - lo < 65535 ? parents - lo : 65535;
+        int lv = 0;
+        i64 top = count;
+        while (top > 1 && lv < MERGE_LEVELS) { top = (top + 1) / 2; ++lv; }
+        u32 *dst = (top == 1 && direct) ? (u32 *)digests : b;
+        for (i64 lo = 0; lo < top; lo += 65535) {                 // grid.y limit
+            const i64 cnt = top - lo < 65535 ? top - lo : 65535;
             dim3 grid((unsigned)((n + BLOCK - 1) / BLOCK), (unsigned)cnt);
-            hipLaunchKernelGGL(k_merge_level, grid, dim3(BLOCK), 0, s, (const u32 *)(a + (size_t)(2 * lo) * n * 8), count - 2 * lo,
-                               (i64)n, parents == 1 ? 1 : 0, b + (size_t)lo * n * 8);
-            VI_LAUNCH_CHECK("k_merge_level");
+            if (lv == 1) hipLaunchKernelGGL(k_merge_levels<1>, grid, dim3(BLOCK), 0, s, (const u32 *)a, count, (i64)n, lo, dst);
+            else hipLaunchKernelGGL(k_merge_levels<2>, grid, dim3(BLOCK), 0, s, (const u32 *)a, count, (i64)n, lo, dst);
+            VI_LAUNCH_CHECK("k_merge_levels");
         }
         u32 *t = a; a = b; b = t;
-        count = parents;
+        count = top;
     }
-    VI_HIP(hipMemcpyAsync(digests, a, (size_t)n * 32, hipMemcpyDeviceToDevice, s));
+    if (!direct) VI_HIP(hipMemcpyAsync(digests, a, (size_t)n * 32, hipMemcpyDeviceToDevice, s));
     return VI_OK;
 }
 
