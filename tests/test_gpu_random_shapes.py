@@ -39,6 +39,36 @@ def test_lde_random_geometries(cp):
         assert torch.equal(cp.coset_extend(co, K, N, shift), got), (case, "extend")
 
 
+def test_lde_random_widths_around_the_plane_boundaries(cp):
+    """Transform lengths whose middle launch is fused (K = L * L) and their neighbours, rates 1 to 1/8, source widths at
+    and around multiples of K/16 (a thread's input planes: the first pass skips the zero half of its inputs, whole or
+    partly filled planes), and a workspace of one to three rows, which forces row chunks."""
+    from verinf_amd import _lib
+    L = _lib.lib()
+    rng = random.Random(5)
+    for case in range(40):
+        logK = rng.choice([12, 12, 13, 14, 14, 16, 11, 10])
+        logN = logK + rng.choice([0, 1, 2, 2, 3])
+        K, N = 1 << logK, 1 << logN
+        unit = K // 16
+        w = rng.choice([K, K // 2, K // 4, unit, unit + 1, 8 * unit - 1, 8 * unit + 1, 3 * unit + rng.randint(0, unit - 1),
+                        rng.randint(1, K), 7 * unit, 9 * unit, K - 1])
+        m = rng.choice([1, 2, 3, 5]) if logN >= 17 else rng.choice([1, 2, 7, 33])
+        pitch = w + rng.choice([0, 0, 1, 5, 64])
+        shift = rng.choice([7, 7, 1, rng.randrange(2, P)])
+        big = rand_field((m, pitch), 5000 + case)
+        view = to_dev(big).view(torch.int64)[:, :w].view(torch.uint64)
+        want = O.coset_lde_rows(np.ascontiguousarray(big[:, :w]), K, N, shift)
+        got = cp.coset_lde(view, K, N, shift)
+        assert np.array_equal(to_np(got), want), (case, logK, logN, m, w, pitch, shift)
+        out2 = torch.empty((m, N), dtype=torch.uint64, device="cuda")
+        ws_bytes = L.vi_coset_lde_min_workspace_bytes(K, N) * rng.choice([1, 2, 3])
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        _lib.check(L.vi_coset_lde(view.data_ptr(), m, w, pitch, K, N, shift, out2.data_ptr(), N, ws.data_ptr(), ws_bytes,
+                                  _lib.stream_ptr()))
+        assert torch.equal(out2, got), (case, "chunked")
+
+
 def test_ntt_random_sizes_round_trip_and_oracle(cp):
     rng = random.Random(7)
     for case in range(25):
