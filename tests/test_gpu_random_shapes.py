@@ -82,6 +82,17 @@ def test_ntt_random_sizes_round_trip_and_oracle(cp):
         assert np.array_equal(to_np(rows), a), (case, logn, m, "inverse")
 
 
+def test_hash_tree_shapes_up_to_a_hundred_chunks(cp):
+    """Chunk counts whose BLAKE3 tree has an odd node on some level, a single node, exact powers of two, and the 86
+    chunks of an 11008-row matrix: the merge launches take two levels of the tree at a time."""
+    rng = random.Random(3)
+    for chunks in (1, 2, 3, 4, 5, 6, 7, 8, 9, 15, 16, 17, 31, 33, 43, 64, 85, 86, 87, 100):
+        m = (chunks - 1) * 128 + rng.choice([1, 7, 64, 127, 128])
+        n = rng.choice([1, 3, 64, 65, 300])
+        a = rand_field((m, n), 9000 + chunks)
+        assert np.array_equal(to_np(cp.hash_columns_streamed(to_dev(a))), O.hash_columns(a)), (chunks, m, n)
+
+
 def test_hash_random_shapes_and_slabs(cp):
     rng = random.Random(11)
     for case in range(30):
