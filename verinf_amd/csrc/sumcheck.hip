@@ -330,6 +330,171 @@ struct FoldOut {
 // a product term's last factor into the bracket of its point, the bracket times the common factor into the
 // thread's sample.  D.skip1: S(1) is not summed (the proof's finishing kernel takes it from the claim).
 // FOLD: see FoldOut (one row of workgroups only: a table's last fetch must belong to the thread that fetched it first).
+// where the tables of a descriptor are: in memory at the descriptor's own addresses, or packed in LDS
+struct TabGlobal {
+    const Desc &D;
+    __device__ __forceinline__ const u64 *src(int t) const { return D.src[t]; }
+    __device__ __forceinline__ u64 *dst(int t) const { return D.dst[t]; }
+};
+struct TabLds {
+    u64 *base;
+    int pitch;                               // words between tables
+    __device__ __forceinline__ const u64 *src(int t) const { return base + t * pitch; }
+    __device__ __forceinline__ u64 *dst(int t) const { return base + t * pitch; }
+};
+
+// Pair i of a round of `half` pairs: the samples of the factored sum into acc and, with FOLD, the tables folded by r
+// (row ty of ny rows of workgroups takes its share of the terms).
+template <int NS, bool FOLD, class TAB>
+__device__ __forceinline__ void eval_mem_pair(const Desc &D, const FoldOut &W, const LinFoldDesc *V, const TAB &T, u64 r, int skip1,
+                                              i64 i, i64 half, int ty, int ny, gl::Wide (&acc)[NS]) {
+    // the factored form described at Desc, every factor fetched from its table.  Loads go out in batches ahead
+    // of the arithmetic that uses them (the common factor first, used last; four linear terms; two factor slots
+    // of a product): one thread's loads are otherwise a chain of round trips to memory.  A slot past the end of
+    // its list repeats a valid load (a cache hit) with coefficient 0 or is skipped by a wavefront-uniform test.
+    u64 v_lo = 0, v_hi = 0;              // the virtual table's pair
+    if (FOLD && W.virt >= 0) {
+        gl::Wide L, H;
+        gl::wide_zero(L);
+        gl::wide_zero(H);
+        for (int k0 = 0; k0 < V->n; k0 += 4) {
+            u64 a[4], b[4], c[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const bool on = k0 + u < V->n;
+                const u64 *f = V->src[on ? k0 + u : k0];
+                a[u] = f[i];
+                b[u] = f[half + i];
+                c[u] = on ? V->coeff[k0 + u] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                gl::wide_mul_acc(L, c[u], a[u]);
+                gl::wide_mul_acc(H, c[u], b[u]);
+            }
+        }
+        v_lo = gl::wide_reduce(L);
+        v_hi = gl::wide_reduce(H);
+        T.dst(W.virt)[i] = gl::mul_add(r, gl::sub(v_hi, v_lo), v_lo);
+    }
+    u64 com_lo = 0, com_hi = 0;
+    if (D.common >= 0) {
+        if (FOLD && D.common == W.virt) {
+            com_lo = v_lo;
+            com_hi = v_hi;
+        } else {
+            const u64 *f = T.src(D.common);
+            com_lo = f[i];
+            com_hi = f[half + i];
+        }
+    }
+    u64 lin[NS];
+    {
+        gl::Wide L, H;
+        gl::wide_zero(L);
+        gl::wide_zero(H);
+        for (int k0 = ty; k0 < D.n_lin; k0 += 4 * ny) {
+            u64 a[4], b[4], c[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int k = k0 + u * ny;
+                const bool on = k < D.n_lin;
+                const int t = D.lin_idx[on ? k : k0];
+                if (FOLD && t == W.virt) {
+                    a[u] = v_lo;
+                    b[u] = v_hi;
+                } else {
+                    const u64 *f = T.src(t);
+                    a[u] = f[i];
+                    b[u] = f[half + i];
+                }
+                c[u] = on ? D.lin_coeff[k] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                gl::wide_mul_acc(L, c[u], a[u]);
+                gl::wide_mul_acc(H, c[u], b[u]);
+                if (FOLD) {
+                    const int k = k0 + u * ny;
+                    if (k < D.n_lin && W.wb_lin[k]) {
+                        const u64 lo = gl::canon(a[u]), hi = gl::canon(b[u]);
+                        T.dst(D.lin_idx[k])[i] = gl::mul_add(r, gl::sub(hi, lo), lo);
+                    }
+                }
+            }
+        }
+        const u64 c0 = ty == 0 ? D.c0 : 0;
+        const u64 l0 = gl::wide_reduce(L), l1 = gl::wide_reduce(H);
+        const u64 ld = gl::sub(l1, l0);
+        u64 lc = gl::addc(l0, c0);
+#pragma unroll
+        for (int x = 0; x < NS; ++x) {
+            lin[x] = lc;
+            if (D.n_lin && x + 1 < NS) lc = gl::addc(lc, ld);
+        }
+    }
+    gl::Wide br[NS];                     // the product terms of the bracket, per point
+#pragma unroll
+    for (int x = 0; x < NS; ++x) gl::wide_zero(br[x]);
+    for (int k = ty; k < D.n_terms; k += ny) {
+        u64 prod[NS];
+#pragma unroll
+        for (int x = 0; x < NS; ++x) prod[x] = D.coeff[k];
+        const int j1 = D.term_off[k + 1];
+        for (int j = D.term_off[k]; j < j1; j += 2) {
+            const bool two = j + 1 < j1;
+            const int t0 = D.fidx[j], t1 = D.fidx[two ? j + 1 : j];
+            u64 a0, b0, a1, b1;
+            if (FOLD && t0 == W.virt) { a0 = v_lo; b0 = v_hi; }
+            else { const u64 *f0 = T.src(t0); a0 = f0[i]; b0 = f0[half + i]; }
+            if (FOLD && t1 == W.virt) { a1 = v_lo; b1 = v_hi; }
+            else { const u64 *f1 = T.src(t1); a1 = f1[i]; b1 = f1[half + i]; }
+            // the value of a factor at x = 0, 1, 2, ...: lo, hi, then steps of hi - lo
+            u64 cur = gl::canon(a0), nxt = gl::canon(b0);
+            u64 dif = gl::sub(nxt, cur);
+            if (FOLD && W.wb_fac[j]) T.dst(t0)[i] = gl::mul_add(r, dif, cur);
+            const bool last0 = !two && j + 1 == j1;
+#pragma unroll
+            for (int x = 0; x < NS; ++x) {
+                if (x <= D.deg && !(skip1 && x == 1)) {
+                    if (last0) gl::wide_mul_acc(br[x], prod[x], cur);
+                    else prod[x] = gl::mul_lazy(prod[x], cur);
+                }
+                if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
+            }
+            if (two) {
+                cur = gl::canon(a1);
+                nxt = gl::canon(b1);
+                dif = gl::sub(nxt, cur);
+                if (FOLD && W.wb_fac[j + 1]) T.dst(t1)[i] = gl::mul_add(r, dif, cur);
+                const bool last1 = j + 2 == j1;
+#pragma unroll
+                for (int x = 0; x < NS; ++x) {
+                    if (x <= D.deg && !(skip1 && x == 1)) {
+                        if (last1) gl::wide_mul_acc(br[x], prod[x], cur);
+                        else prod[x] = gl::mul_lazy(prod[x], cur);
+                    }
+                    if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
+                }
+            }
+        }
+    }
+    {
+        u64 cur = 1, nxt = 1, dif = 0;
+        if (D.common >= 0) {
+            cur = gl::canon(com_lo);
+            nxt = gl::canon(com_hi);
+            dif = gl::sub(nxt, cur);
+            if (FOLD && W.wb_common) T.dst(D.common)[i] = gl::mul_add(r, dif, cur);
+        }
+#pragma unroll
+        for (int x = 0; x < NS; ++x) {
+            if (x <= D.deg && !(skip1 && x == 1)) gl::wide_mul_acc(acc[x], gl::addc(lin[x], gl::wide_reduce(br[x])), cur);
+            if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
+        }
+    }
+}
+
 template <int NS, bool FOLD>
 __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, const FoldOut W, const LinFoldDesc V, i64 half, u64 *partial,
                                                     int accumulate, u64 scale) {
@@ -339,153 +504,9 @@ __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, const FoldOut 
     gl::Wide acc[NS];
 #pragma unroll
     for (int x = 0; x < NS; ++x) gl::wide_zero(acc[x]);
-    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride) {
-        // the factored form described at Desc, every factor fetched from its table.  Loads go out in batches ahead
-        // of the arithmetic that uses them (the common factor first, used last; four linear terms; two factor slots
-        // of a product): one thread's loads are otherwise a chain of round trips to memory.  A slot past the end of
-        // its list repeats a valid load (a cache hit) with coefficient 0 or is skipped by a wavefront-uniform test.
-        u64 v_lo = 0, v_hi = 0;              // the virtual table's pair
-        if (FOLD && W.virt >= 0) {
-            gl::Wide L, H;
-            gl::wide_zero(L);
-            gl::wide_zero(H);
-            for (int k0 = 0; k0 < V.n; k0 += 4) {
-                u64 a[4], b[4], c[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const bool on = k0 + u < V.n;
-                    const u64 *f = V.src[on ? k0 + u : k0];
-                    a[u] = f[i];
-                    b[u] = f[half + i];
-                    c[u] = on ? V.coeff[k0 + u] : 0;
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    gl::wide_mul_acc(L, c[u], a[u]);
-                    gl::wide_mul_acc(H, c[u], b[u]);
-                }
-            }
-            v_lo = gl::wide_reduce(L);
-            v_hi = gl::wide_reduce(H);
-            D.dst[W.virt][i] = gl::mul_add(W.r, gl::sub(v_hi, v_lo), v_lo);
-        }
-        u64 com_lo = 0, com_hi = 0;
-        if (D.common >= 0) {
-            if (FOLD && D.common == W.virt) {
-                com_lo = v_lo;
-                com_hi = v_hi;
-            } else {
-                const u64 *f = D.src[D.common];
-                com_lo = f[i];
-                com_hi = f[half + i];
-            }
-        }
-        u64 lin[NS];
-        {
-            gl::Wide L, H;
-            gl::wide_zero(L);
-            gl::wide_zero(H);
-            for (int k0 = ty; k0 < D.n_lin; k0 += 4 * ny) {
-                u64 a[4], b[4], c[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int k = k0 + u * ny;
-                    const bool on = k < D.n_lin;
-                    const int t = D.lin_idx[on ? k : k0];
-                    if (FOLD && t == W.virt) {
-                        a[u] = v_lo;
-                        b[u] = v_hi;
-                    } else {
-                        const u64 *f = D.src[t];
-                        a[u] = f[i];
-                        b[u] = f[half + i];
-                    }
-                    c[u] = on ? D.lin_coeff[k] : 0;
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    gl::wide_mul_acc(L, c[u], a[u]);
-                    gl::wide_mul_acc(H, c[u], b[u]);
-                    if (FOLD) {
-                        const int k = k0 + u * ny;
-                        if (k < D.n_lin && W.wb_lin[k]) {
-                            const u64 lo = gl::canon(a[u]), hi = gl::canon(b[u]);
-                            D.dst[D.lin_idx[k]][i] = gl::mul_add(W.r, gl::sub(hi, lo), lo);
-                        }
-                    }
-                }
-            }
-            const u64 c0 = ty == 0 ? D.c0 : 0;
-            const u64 l0 = gl::wide_reduce(L), l1 = gl::wide_reduce(H);
-            const u64 ld = gl::sub(l1, l0);
-            u64 lc = gl::addc(l0, c0);
-#pragma unroll
-            for (int x = 0; x < NS; ++x) {
-                lin[x] = lc;
-                if (D.n_lin && x + 1 < NS) lc = gl::addc(lc, ld);
-            }
-        }
-        gl::Wide br[NS];                     // the product terms of the bracket, per point
-#pragma unroll
-        for (int x = 0; x < NS; ++x) gl::wide_zero(br[x]);
-        for (int k = ty; k < D.n_terms; k += ny) {
-            u64 prod[NS];
-#pragma unroll
-            for (int x = 0; x < NS; ++x) prod[x] = D.coeff[k];
-            const int j1 = D.term_off[k + 1];
-            for (int j = D.term_off[k]; j < j1; j += 2) {
-                const bool two = j + 1 < j1;
-                const int t0 = D.fidx[j], t1 = D.fidx[two ? j + 1 : j];
-                u64 a0, b0, a1, b1;
-                if (FOLD && t0 == W.virt) { a0 = v_lo; b0 = v_hi; }
-                else { const u64 *f0 = D.src[t0]; a0 = f0[i]; b0 = f0[half + i]; }
-                if (FOLD && t1 == W.virt) { a1 = v_lo; b1 = v_hi; }
-                else { const u64 *f1 = D.src[t1]; a1 = f1[i]; b1 = f1[half + i]; }
-                // the value of a factor at x = 0, 1, 2, ...: lo, hi, then steps of hi - lo
-                u64 cur = gl::canon(a0), nxt = gl::canon(b0);
-                u64 dif = gl::sub(nxt, cur);
-                if (FOLD && W.wb_fac[j]) D.dst[t0][i] = gl::mul_add(W.r, dif, cur);
-                const bool last0 = !two && j + 1 == j1;
-#pragma unroll
-                for (int x = 0; x < NS; ++x) {
-                    if (x <= D.deg && !(D.skip1 && x == 1)) {
-                        if (last0) gl::wide_mul_acc(br[x], prod[x], cur);
-                        else prod[x] = gl::mul_lazy(prod[x], cur);
-                    }
-                    if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
-                }
-                if (two) {
-                    cur = gl::canon(a1);
-                    nxt = gl::canon(b1);
-                    dif = gl::sub(nxt, cur);
-                    if (FOLD && W.wb_fac[j + 1]) D.dst[t1][i] = gl::mul_add(W.r, dif, cur);
-                    const bool last1 = j + 2 == j1;
-#pragma unroll
-                    for (int x = 0; x < NS; ++x) {
-                        if (x <= D.deg && !(D.skip1 && x == 1)) {
-                            if (last1) gl::wide_mul_acc(br[x], prod[x], cur);
-                            else prod[x] = gl::mul_lazy(prod[x], cur);
-                        }
-                        if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
-                    }
-                }
-            }
-        }
-        {
-            u64 cur = 1, nxt = 1, dif = 0;
-            if (D.common >= 0) {
-                cur = gl::canon(com_lo);
-                nxt = gl::canon(com_hi);
-                dif = gl::sub(nxt, cur);
-                if (FOLD && W.wb_common) D.dst[D.common][i] = gl::mul_add(W.r, dif, cur);
-            }
-#pragma unroll
-            for (int x = 0; x < NS; ++x) {
-                if (x <= D.deg && !(D.skip1 && x == 1)) gl::wide_mul_acc(acc[x], gl::addc(lin[x], gl::wide_reduce(br[x])), cur);
-                if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
-            }
-        }
-    }
+    const TabGlobal T{D};
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride)
+        eval_mem_pair<NS, FOLD>(D, W, &V, T, W.r, D.skip1, i, half, ty, ny, acc);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
     for (int x = 0; x < NS; ++x) {
@@ -1230,6 +1251,78 @@ int vi_sumcheck_prove(const uint64_t *const *tables, uint64_t *const *work, int 
 
 #include "sumcheck_fast.hpp"
 
+namespace {
+
+// ---- the last rounds of a sum whose tables are read from memory, in one workgroup -----------------------------
+// Once all tables of a round fit a workgroup's LDS together, one launch runs every remaining round: the tables are
+// copied in (reduced mod p on the way); a round evaluates its pairs with the walk of k_eval_mem over the LDS copies
+// (eval_mem_pair), the terms dealt over as many rows of threads as the workgroup has for the round's pairs -- a
+// thread's walk over all terms is what a small round costs --, leaves ONE row of partial sums for k_finish, and then
+// folds every table in place.  Small rounds are otherwise a fold launch and an evaluation launch each, both bound by
+// launch latency.  The folded tables are not written back.
+constexpr int TAIL_MEM_WORDS = 7168;            // 56 KiB of table words
+
+struct TailRounds {
+    u64 r[MAX_ROUNDS];                          // challenge of round k
+    unsigned off[MAX_ROUNDS];                   // word offset of round k's row in the workspace
+    int k0, k1;                                 // rounds k0 .. k1 - 1; round 0 of a proof sums S(1), later ones do not
+};
+
+template <int NS>
+__global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const TailRounds R, int size, u64 *part) {
+    __shared__ u64 tab[TAIL_MEM_WORDS];
+    __shared__ u64 red[TAIL_THREADS / 64][NSAMP];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    for (int t = 0; t < D.n_tables; ++t) {
+        const u64 *src = D.src[t];
+        for (int i = tid; i < size; i += TAIL_THREADS) tab[t * size + i] = gl::canon(src[i]);
+    }
+    __syncthreads();
+    const TabLds T{tab, size};
+    const FoldOut none = {};
+    int half = size >> 1, log_half = 0;
+    while ((1 << log_half) < half) ++log_half;
+    for (int k = R.k0; k < R.k1; ++k, half >>= 1, --log_half) {
+        gl::Wide acc[NS];
+#pragma unroll
+        for (int x = 0; x < NS; ++x) gl::wide_zero(acc[x]);
+        const int skip1 = k > 0 ? 1 : 0;
+        if (half >= TAIL_THREADS) {
+            for (int i = tid; i < half; i += TAIL_THREADS)
+                eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, 0, 1, acc);
+        } else {
+            // row ty of ny takes its share of the terms of pair i
+            const int ny = TAIL_THREADS >> log_half, ty = tid >> log_half, i = tid & (half - 1);
+            eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, ty, ny, acc);
+        }
+#pragma unroll
+        for (int x = 0; x < NS; ++x) {
+            const u64 v = wave_sum(gl::wide_reduce(acc[x]));
+            if (lane == 0) red[w][x] = v;
+        }
+        __syncthreads();                                   // the wavefronts' sums are there; every read of this round is done
+        if (tid < NSAMP) {
+            u64 v = 0;
+            if (tid < NS) {
+                v = red[0][tid];
+                for (int j = 1; j < TAIL_THREADS / 64; ++j) v = gl::add(v, red[j][tid]);
+            }
+            part[R.off[k] + tid] = v;
+        }
+        // fold in place: entry i of a table from entries i and half + i, each by one thread
+        const u64 r = R.r[k];
+        for (int e = tid; e < (D.n_tables << log_half); e += TAIL_THREADS) {
+            const int t = e >> log_half, i = e & (half - 1);
+            u64 *p = tab + t * size;
+            const u64 lo = p[i];
+            p[i] = gl::mul_add(r, gl::sub(p[half + i], lo), lo);
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace
+
 extern "C" {
 
 size_t vi_sumcheck_prove_coins_workspace_bytes(int64_t size) {
@@ -1523,6 +1616,24 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
                     rc = fold_tables(k == 1 ? D.src : (const uint64_t *const *)D.dst, D.dst, n_tables, 2 * half, C.r[k - 1], s, k == 1);
                     if (rc) return rc;
                     folded = true;
+                }
+                if ((i64)n_tables * 2 * half <= TAIL_MEM_WORDS) {
+                    // every table of this round fits one workgroup's LDS: all remaining rounds in one launch
+                    TailRounds R;
+                    for (int j = 0; j < MAX_ROUNDS; ++j) { R.r[j] = C.r[j]; R.off[j] = 0; }
+                    R.k0 = k;
+                    R.k1 = v;
+                    for (int j = k; j < v; ++j) {
+                        R.off[j] = off;
+                        C.off[j] = off;
+                        C.nb[j] = 1;
+                        if (j > 0) C.skip_mask |= 1ull << j;
+                        off += NSAMP;
+                    }
+                    if (E.deg <= 3) hipLaunchKernelGGL(k_tail_mem<4>, dim3(1), dim3(TAIL_THREADS), 0, s, E, R, (int)(2 * half), part);
+                    else hipLaunchKernelGGL(k_tail_mem<NSAMP>, dim3(1), dim3(TAIL_THREADS), 0, s, E, R, (int)(2 * half), part);
+                    VI_LAUNCH_CHECK("sumcheck tail (tables from memory)");
+                    break;
                 }
                 if (k > 0) {
                     E.skip1 = 1;
