@@ -1260,29 +1260,28 @@ namespace {
 // thread's walk over all terms is what a small round costs --, leaves ONE row of partial sums for k_finish, and then
 // folds every table in place.  Small rounds are otherwise a fold launch and an evaluation launch each, both bound by
 // launch latency.  The folded tables are not written back.
-constexpr int TAIL_MEM_WORDS = 7168;            // 56 KiB of table words
+constexpr int TAIL_MEM_WORDS = 6400;            // 50 KiB of table words
 
-struct TailRounds {
-    u64 r[MAX_ROUNDS];                          // challenge of round k
-    unsigned off[MAX_ROUNDS];                   // word offset of round k's row in the workspace
-    int k0, k1;                                 // rounds k0 .. k1 - 1; round 0 of a proof sums S(1), later ones do not
-};
-
+// C: the proof's rounds; those before C.n_prior have left their partial sums in the workspace, the launch runs the
+// rest and finishes the proof like k_finish (round 0 of a proof sums S(1), later ones do not).
+// rows: power of two, rows of threads that have a share of the terms.
 template <int NS>
-__global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const TailRounds R, int size, u64 *part) {
+__global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const ChainDesc C, int rows, int size, const u64 *part, u64 *out) {
     __shared__ u64 tab[TAIL_MEM_WORDS];
     __shared__ u64 red[TAIL_THREADS / 64][NSAMP];
+    __shared__ FinishShared sh;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     for (int t = 0; t < D.n_tables; ++t) {
         const u64 *src = D.src[t];
         for (int i = tid; i < size; i += TAIL_THREADS) tab[t * size + i] = gl::canon(src[i]);
     }
+    finish_begin(C, part, sh);                             // the earlier rounds' sums and the Lagrange bases: sh.raw[k < n_prior], sh.lag
     __syncthreads();
     const TabLds T{tab, size};
     const FoldOut none = {};
     int half = size >> 1, log_half = 0;
     while ((1 << log_half) < half) ++log_half;
-    for (int k = R.k0; k < R.k1; ++k, half >>= 1, --log_half) {
+    for (int k = C.n_prior; k < C.n_rounds; ++k, half >>= 1, --log_half) {
         gl::Wide acc[NS];
 #pragma unroll
         for (int x = 0; x < NS; ++x) gl::wide_zero(acc[x]);
@@ -1291,9 +1290,12 @@ __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const T
             for (int i = tid; i < half; i += TAIL_THREADS)
                 eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, 0, 1, acc);
         } else {
-            // row ty of ny takes its share of the terms of pair i
-            const int ny = TAIL_THREADS >> log_half, ty = tid >> log_half, i = tid & (half - 1);
-            eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, ty, ny, acc);
+            // row ty of ny takes its share of the terms of pair i; no more rows than there are shares (every row pays
+            // for the common factor and the reductions of its sums, and the workgroup has one CU to run on)
+            int ny = TAIL_THREADS >> log_half;
+            if (ny > rows) ny = rows;
+            const int ty = tid >> log_half, i = tid & (half - 1);
+            if (ty < ny) eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, ty, ny, acc);
         }
 #pragma unroll
         for (int x = 0; x < NS; ++x) {
@@ -1301,16 +1303,13 @@ __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const T
             if (lane == 0) red[w][x] = v;
         }
         __syncthreads();                                   // the wavefronts' sums are there; every read of this round is done
-        if (tid < NSAMP) {
-            u64 v = 0;
-            if (tid < NS) {
-                v = red[0][tid];
-                for (int j = 1; j < TAIL_THREADS / 64; ++j) v = gl::add(v, red[j][tid]);
-            }
-            part[R.off[k] + tid] = v;
+        if (tid < NS) {
+            u64 v = red[0][tid];
+            for (int j = 1; j < TAIL_THREADS / 64; ++j) v = gl::add(v, red[j][tid]);
+            sh.raw[k][tid] = v;
         }
         // fold in place: entry i of a table from entries i and half + i, each by one thread
-        const u64 r = R.r[k];
+        const u64 r = C.r[k];
         for (int e = tid; e < (D.n_tables << log_half); e += TAIL_THREADS) {
             const int t = e >> log_half, i = e & (half - 1);
             u64 *p = tab + t * size;
@@ -1319,6 +1318,7 @@ __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const T
         }
         __syncthreads();
     }
+    finish_samples(C, sh, out);
 }
 
 }  // namespace
@@ -1619,21 +1619,15 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
                 }
                 if ((i64)n_tables * 2 * half <= TAIL_MEM_WORDS) {
                     // every table of this round fits one workgroup's LDS: all remaining rounds in one launch
-                    TailRounds R;
-                    for (int j = 0; j < MAX_ROUNDS; ++j) { R.r[j] = C.r[j]; R.off[j] = 0; }
-                    R.k0 = k;
-                    R.k1 = v;
-                    for (int j = k; j < v; ++j) {
-                        R.off[j] = off;
-                        C.off[j] = off;
-                        C.nb[j] = 1;
-                        if (j > 0) C.skip_mask |= 1ull << j;
-                        off += NSAMP;
-                    }
-                    if (E.deg <= 3) hipLaunchKernelGGL(k_tail_mem<4>, dim3(1), dim3(TAIL_THREADS), 0, s, E, R, (int)(2 * half), part);
-                    else hipLaunchKernelGGL(k_tail_mem<NSAMP>, dim3(1), dim3(TAIL_THREADS), 0, s, E, R, (int)(2 * half), part);
+                    const int shares = std::max(std::max(E.n_terms, (E.n_lin + 3) / 4), 1);
+                    int rows = 1;
+                    while (rows < shares) rows <<= 1;
+                    for (int j = std::max(k, 1); j < v; ++j) C.skip_mask |= 1ull << j;
+                    C.n_prior = k;
+                    if (E.deg <= 3) hipLaunchKernelGGL(k_tail_mem<4>, dim3(1), dim3(TAIL_THREADS), 0, s, E, C, rows, (int)(2 * half), (const u64 *)part, samples);
+                    else hipLaunchKernelGGL(k_tail_mem<NSAMP>, dim3(1), dim3(TAIL_THREADS), 0, s, E, C, rows, (int)(2 * half), (const u64 *)part, samples);
                     VI_LAUNCH_CHECK("sumcheck tail (tables from memory)");
-                    break;
+                    return VI_OK;                          // the tail has written every round's samples
                 }
                 if (k > 0) {
                     E.skip1 = 1;
