@@ -134,9 +134,9 @@ def test_more_tables_than_fit_in_registers(mods):
     _check(gpu, tabs, terms, 13, as_tensor=True)
 
 
-@pytest.mark.parametrize("nt,v", [(9, 1), (9, 4), (12, 9), (25, 8), (26, 8), (50, 7), (51, 7), (64, 6), (10, 11)])
+@pytest.mark.parametrize("nt,v", [(9, 1), (9, 4), (12, 9), (22, 8), (23, 8), (44, 7), (45, 7), (64, 6), (10, 11)])
 def test_last_rounds_from_lds_around_the_capacity(mods, nt, v):
-    """More tables than fit registers, at sizes around what one workgroup's LDS holds of them (6400 words in all): the
+    """More tables than fit registers, at sizes around what one workgroup's LDS holds of them (5632 words in all): the
     whole proof inside the single-workgroup launch (round 0 included, which sums every sample), a proof whose first
     rounds run as separate launches, table counts just below and just above the capacity at a size, a common factor
     with linear terms, and a term of degree five (eight samples kept per pair)."""

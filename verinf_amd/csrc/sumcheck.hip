@@ -1260,7 +1260,8 @@ namespace {
 // thread's walk over all terms is what a small round costs --, leaves ONE row of partial sums for k_finish, and then
 // folds every table in place.  Small rounds are otherwise a fold launch and an evaluation launch each, both bound by
 // launch latency.  The folded tables are not written back.
-constexpr int TAIL_MEM_WORDS = 6400;            // 50 KiB of table words
+constexpr int TAIL_MEM_WORDS = 5632;            // 44 KiB of table words
+constexpr int TAIL_MEM_ROUNDS = 9;              // nine or more tables share the words: a table has at most 2^9
 
 // C: the proof's rounds; those before C.n_prior have left their partial sums in the workspace, the launch runs the
 // rest and finishes the proof like k_finish (round 0 of a proof sums S(1), later ones do not).
@@ -1268,7 +1269,7 @@ constexpr int TAIL_MEM_WORDS = 6400;            // 50 KiB of table words
 template <int NS>
 __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const ChainDesc C, int rows, int size, const u64 *part, u64 *out) {
     __shared__ u64 tab[TAIL_MEM_WORDS];
-    __shared__ u64 red[TAIL_THREADS / 64][NSAMP];
+    __shared__ u64 wsum[TAIL_MEM_ROUNDS][TAIL_THREADS / 64][NS];     // per round and wavefront
     __shared__ FinishShared sh;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     for (int t = 0; t < D.n_tables; ++t) {
@@ -1297,17 +1298,26 @@ __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const C
             const int ty = tid >> log_half, i = tid & (half - 1);
             if (ty < ny) eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, ty, ny, acc);
         }
+        // the wavefront's sums of this round, the samples side by side so that their shuffles are in flight together;
+        // the wavefronts are added up for all rounds at once behind the loop
+        {
+            u64 v[NS];
 #pragma unroll
-        for (int x = 0; x < NS; ++x) {
-            const u64 v = wave_sum(gl::wide_reduce(acc[x]));
-            if (lane == 0) red[w][x] = v;
+            for (int x = 0; x < NS; ++x) v[x] = gl::wide_reduce(acc[x]);
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                u64 o[NS];
+#pragma unroll
+                for (int x = 0; x < NS; ++x) o[x] = __shfl_xor(v[x], off, 64);
+#pragma unroll
+                for (int x = 0; x < NS; ++x) v[x] = gl::addc(v[x], o[x]);
+            }
+            if (lane == 0) {
+#pragma unroll
+                for (int x = 0; x < NS; ++x) wsum[k - C.n_prior][w][x] = v[x];
+            }
         }
-        __syncthreads();                                   // the wavefronts' sums are there; every read of this round is done
-        if (tid < NS) {
-            u64 v = red[0][tid];
-            for (int j = 1; j < TAIL_THREADS / 64; ++j) v = gl::add(v, red[j][tid]);
-            sh.raw[k][tid] = v;
-        }
+        __syncthreads();                                   // every read of this round's tables is done
         // fold in place: entry i of a table from entries i and half + i, each by one thread
         const u64 r = C.r[k];
         for (int e = tid; e < (D.n_tables << log_half); e += TAIL_THREADS) {
@@ -1318,6 +1328,17 @@ __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const C
         }
         __syncthreads();
     }
+    // the rounds of this launch: thread (round, sample) adds up the wavefronts
+    {
+        const int n_mine = C.n_rounds - C.n_prior;
+        if (tid < n_mine * NS) {
+            const int kk = tid / NS, x = tid - kk * NS;
+            u64 v = wsum[kk][0][x];
+            for (int j = 1; j < TAIL_THREADS / 64; ++j) v = gl::add(v, wsum[kk][j][x]);
+            sh.raw[C.n_prior + kk][x] = v;
+        }
+    }
+    __syncthreads();
     finish_samples(C, sh, out);
 }
 
@@ -1617,7 +1638,7 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
                     if (rc) return rc;
                     folded = true;
                 }
-                if ((i64)n_tables * 2 * half <= TAIL_MEM_WORDS) {
+                if ((i64)n_tables * 2 * half <= TAIL_MEM_WORDS && v - k <= TAIL_MEM_ROUNDS) {
                     // every table of this round fits one workgroup's LDS: all remaining rounds in one launch
                     const int shares = std::max(std::max(E.n_terms, (E.n_lin + 3) / 4), 1);
                     int rows = 1;
