@@ -1600,6 +1600,22 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
                 default: return prove_fast_shape<4, 1>(F, size, C, part, samples, s);
             }
         }
+        // a whole proof whose tables fit one workgroup's LDS together: one launch (k_tail_mem), whatever the table count
+        if ((i64)n_tables * size <= TAIL_MEM_WORDS && v <= TAIL_MEM_ROUNDS) {
+            Desc M;
+            rc = fill_desc(M, tables, work, n_tables, term_off, factor_idx, coeffs, n_terms, true, who, true);
+            if (rc) return rc;
+            const int shares = std::max(std::max(M.n_terms, (M.n_lin + 3) / 4), 1);
+            int rows = 1;
+            while (rows < shares) rows <<= 1;
+            C.scale = M.out_scale;
+            C.n_prior = 0;
+            for (int j = 1; j < v; ++j) C.skip_mask |= 1ull << j;
+            if (M.deg <= 3) hipLaunchKernelGGL(k_tail_mem<4>, dim3(1), dim3(TAIL_THREADS), 0, s, M, C, rows, (int)size, (const u64 *)part, samples);
+            else hipLaunchKernelGGL(k_tail_mem<NSAMP>, dim3(1), dim3(TAIL_THREADS), 0, s, M, C, rows, (int)size, (const u64 *)part, samples);
+            VI_LAUNCH_CHECK("sumcheck in one workgroup");
+            return VI_OK;
+        }
         // any other sum of at most one descriptor: one launch per round, queued back to back
         i64 half = size / 2;
         unsigned off = 0;
