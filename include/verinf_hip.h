@@ -93,8 +93,11 @@ int vi_poly_eval(const uint64_t *coeffs, int64_t m, int64_t d, const uint64_t *p
  * (prover/cuda_primitives.py:347-409, 1111-1114; prover/kernels/ntt.cuh:667-770):
  * in-place natural-order transform of each of the m contiguous rows of length n
  * (a power of two >= 2): X[k] = sum_j x[j] w^(jk), w = 7^((p-1)/n); the inverse
- * uses w^-1 and multiplies by n^-1.  Rows of 1024 elements or more are transformed in
- * several passes and need vi_ntt_workspace_bytes(m, n) bytes of scratch (0 for shorter rows). */
+ * uses w^-1 and multiplies by n^-1.  Rows of more than 4096 elements are transformed in
+ * several passes and need vi_ntt_workspace_bytes(m, n) bytes of scratch (0 for shorter rows:
+ * up to 512 elements are one pass, 1024 .. 4096 one launch of two digits that meet in LDS).
+ * Environment: VI_NTT_ROW=0 (read once per process) runs rows of 1024 .. 4096 elements as two
+ * passes through the workspace instead; vi_ntt_workspace_bytes then reports what that needs. */
 size_t vi_ntt_workspace_bytes(int64_t m, int64_t n);
 int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, size_t ws_bytes,
                    void *stream);

@@ -18,9 +18,10 @@ struct Owned {
     Tables T;
 };
 
-Owned *make_owned(int logn, int inv) {
+Owned *make_owned(int logn, int inv, bool row = false) {
     Owned *o = new Owned();
-    o->H = make_tables(logn, inv);
+    const Split rs = row_split(logn);
+    o->H = make_tables(logn, inv, row ? &rs : nullptr);
     o->twl = make_twl(inv);
     o->T.sp = o->H.sp;
     o->T.logn = logn;
@@ -108,6 +109,28 @@ void run_fused(const PassArgs &Ai_in, const PassArgs &Af_in) {
 }
 
 int g_allow_fusion = 1;
+int g_allow_row = 1;
+long g_row_runs = 0;                        // transforms of short rows that ran as the single launch
+
+// the single launch for rows of 2^10 .. 2^12 points, phase by phase like k_ntt_row
+template <int A0, bool INV, bool UNI = false>
+void run_row(const PassArgs &P0, const PassArgs &P1_in) {
+    PassArgs P1 = P1_in;
+    P1.is_final = 1;
+    const i64 tiles = pass_tiles(P1);
+    std::vector<u64> lds(TILE + 256), twi(256);
+    std::vector<u64> regs((size_t)NTHREADS * 16);
+    auto R = [&](int tid) -> u64(&)[16] { return *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]); };
+    for (int tid = 0; tid < NTHREADS; ++tid) twi[twi_slot<4, true>(tid >> 4, tid & 15)] = P1.twi[tid];
+    ++g_row_runs;
+    for (i64 tile = 0; tile < tiles; ++tile) {
+        for (int tid = 0; tid < NTHREADS; ++tid) row_stage0<A0, INV>(P0, tile, tid, lds.data());
+        for (int tid = 0; tid < NTHREADS; ++tid) row_gather(lds.data(), tid, R(tid));
+        for (int tid = 0; tid < NTHREADS; ++tid)
+            fast_stage1<4, INV, false, true>(P1, tile, tid, 0, 0xFFFFu, R(tid), R(tid), twi.data(), lds.data());
+        for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<4, INV, UNI>(P1, tile, tid, 0, lds.data());
+    }
+}
 
 // runs passes[q] (and passes[q + 1] with it when the two fuse); returns how many passes it consumed
 int run_passes_at(const std::vector<PassArgs> &passes, size_t q);
@@ -205,7 +228,33 @@ u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }
 u64 emu_mul_pow2(u64 x, unsigned s) { return gl::mul_pow2(x, s); }
 u64 emu_inv(u64 x) { return gl::inv(x); }
 
+void emu_set_row(int on) { g_allow_row = on; }
+long emu_row_runs() { return g_row_runs; }
+
 int emu_ntt_batched(u64 *buf, long m, int logn, int inverse) {
+    if (g_use_fast && g_allow_row && row_single_ok(logn)) {
+        Owned *o = make_owned(logn, inverse, true);
+        PassArgs P0, P1;
+        build_row_passes(o->T, buf, m, P0, P1);
+        int nv = 16;
+        const bool uni = g_allow_uniform && pass_uniform(P1, &nv) && nv == 16;
+        switch (P0.a * 2 + (inverse ? 1 : 0)) {
+            case 4: run_row<2, false>(P0, P1); break;
+            case 5: run_row<2, true>(P0, P1); break;
+            case 6: run_row<3, false>(P0, P1); break;
+            case 7: run_row<3, true>(P0, P1); break;
+            case 8:                                        // the launcher's choice: scalar-base stores when the last digit qualifies
+                if (uni) run_row<4, false, true>(P0, P1);
+                else run_row<4, false>(P0, P1);
+                break;
+            default:
+                if (uni) run_row<4, true, true>(P0, P1);
+                else run_row<4, true>(P0, P1);
+                break;
+        }
+        delete o;
+        return 1;
+    }
     Owned *o = make_owned(logn, inverse);
     std::vector<u64> ws(o->T.sp.p > 1 ? (size_t)m << logn : 1);
     std::vector<PassArgs> passes;

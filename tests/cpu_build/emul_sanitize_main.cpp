@@ -58,6 +58,16 @@ int main() {
         bad += check_ntt(10, 5);
     }
     emu_set_fast(1);
+    // rows of 2^10 .. 2^12 points: the single launch (tiles of 4, 2 and 1 rows, the last one partly empty) and the two passes
+    for (int row = 0; row < 2; ++row) {
+        emu_set_row(row);
+        bad += check_ntt(10, 7);
+        bad += check_ntt(10, 1);
+        bad += check_ntt(11, 1);
+        bad += check_ntt(11, 4);
+        bad += check_ntt(12, 1);
+    }
+    emu_set_row(1);
     const long lde[][5] = {
         // logK logN m width in_stride
         {4, 6, 3, 16, 16},   {4, 6, 3, 9, 11},    {5, 7, 130, 32, 32}, {6, 8, 65, 33, 64},   {8, 10, 17, 256, 300},

@@ -37,6 +37,8 @@ def emu():
     L.emu_merged_runs.restype = c_long
     L.emu_set_half.argtypes = [c_int]
     L.emu_half_runs.restype = c_long
+    L.emu_set_row.argtypes = [c_int]
+    L.emu_row_runs.restype = c_long
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
     L.emu_coset_lde.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p]
     L.emu_coset_lde_ex.argtypes = [u64p, c_long, c_long, c_long, c_int, c_int, c_uint64, u64p, c_long, u64p, c_int]
@@ -106,6 +108,35 @@ def test_ntt_passes_match_oracle(emu, logn, m):
         emu.emu_ntt_batched(_p(got), m, logn, 1)
         assert np.array_equal(got, a), mode
     _set_mode(emu, 1, 1, 1, 1)
+
+
+@pytest.mark.parametrize("logn,m", [(10, 1), (10, 4), (10, 7), (11, 1), (11, 3), (11, 8), (12, 1), (12, 2), (12, 5)])
+def test_short_rows_in_one_launch(emu, logn, m):
+    """Rows of 2^10 .. 2^12 points run as one launch (first digit, exchange through LDS, last digit) and as the two
+    passes longer rows take: both against the oracle, with row counts that fill the last tile and that do not, and
+    with words at and above p in the input (reduced on load)."""
+    a = _rand((m, 1 << logn), 900 + 13 * logn + m)
+    raw = a.copy()
+    raw[0, :5] = np.array([P, P + 1, (1 << 64) - 1, P - 1, 0], dtype=np.uint64)
+    a[0, :5] = raw[0, :5] % np.uint64(P)
+    want = O.ntt_rows(a)
+    _set_mode(emu, 1, 1, 1, 1)
+    for row in (1, 0):
+        emu.emu_set_row(row)
+        before = emu.emu_row_runs()
+        got = raw.copy()
+        assert emu.emu_ntt_batched(_p(got), m, logn, 0) == (1 if row else 2)
+        assert np.array_equal(got, want), row
+        emu.emu_ntt_batched(_p(got), m, logn, 1)
+        assert np.array_equal(got, a), row
+        assert emu.emu_row_runs() - before == (2 if row else 0)
+    emu.emu_set_row(1)
+    # lengths on either side keep their own schedule
+    for other in (9, 13):
+        before = emu.emu_row_runs()
+        b = _rand((2, 1 << other), 7)
+        emu.emu_ntt_batched(_p(b), 2, other, 0)
+        assert emu.emu_row_runs() == before
 
 
 def test_ntt_25_bit_split_is_well_formed(emu):

@@ -51,6 +51,39 @@ def test_batched_ntt_matches_oracle(cp, logn, m):
     assert np.array_equal(to_np(rows), a)
 
 
+_SWITCHED_OFF = """
+import numpy as np
+from oracle import oracle as O
+from tests.gpu_util import rand_field, to_dev, to_np
+from verinf_amd.prover import cuda_primitives as cp
+for logn, m in ((10, 6), (11, 3), (12, 5)):
+    a = rand_field((m, 1 << logn), 500 + logn)
+    rows = to_dev(a)
+    cp.ntt_forward_batched(rows)
+    assert np.array_equal(to_np(rows), O.ntt_rows(a)), logn
+    cp.ntt_inverse_batched(rows)
+    assert np.array_equal(to_np(rows), a), logn
+for logK, m in ((12, 5), (16, 2)):
+    a = rand_field((m, 1 << logK), 600 + logK)
+    got = to_np(cp.coset_lde(to_dev(a), 1 << logK, 4 << logK))
+    assert np.array_equal(got, O.coset_lde_rows(a, 1 << logK, 4 << logK)), logK
+print("switched-off paths agree")
+"""
+
+
+def test_the_schedules_the_environment_switches_select():
+    """VI_NTT_ROW=0 (rows of 2^10 .. 2^12 points as two passes through a workspace) and VI_LDE_MERGED=0 (the coset
+    factors applied whole in the fused launch) are read once per process, so they are set for a child process,
+    which compares both schedules with the oracle; this process runs the default ones."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, VI_NTT_ROW="0", VI_LDE_MERGED="0")
+    res = subprocess.run([sys.executable, "-c", _SWITCHED_OFF], cwd=root, env=env, capture_output=True, text=True,
+                         timeout=280)
+    assert res.returncode == 0 and "switched-off paths agree" in res.stdout, res.stdout + res.stderr
+
+
 def test_config1_plumbing(cp):
     """The small plumbing workload: 16 x 2^12 (seed 0), forward, inverse, then LDE to 2^14 with shift 7."""
     a = rand_field((16, 1 << 12), 0)

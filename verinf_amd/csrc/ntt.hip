@@ -5,7 +5,8 @@
 // 32..256 points run in k_ntt_fast (two register-blocked 16 / 2..16-point transforms with one LDS crossing,
 // ntt_fast.hpp), 512 points in k_ntt_512, and the last inverse pass of an LDE together with the first forward pass in
 // k_lde_mid (the coefficients never leave the registers); k_ntt_pass, radix-2 levels in LDS, is left with digits
-// below 32 points.  The host side (ntt_plan.hpp) decides the digit split, owns the cached tables and strings
+// below 32 points.  Whole rows of 2^10 .. 2^12 points are one launch of k_ntt_row (a 4..16-point digit, then a
+// 256-point one, both crossings in LDS).  The host side (ntt_plan.hpp) decides the digit split, owns the cached tables and strings
 // passes together into
 //   * vi_ntt_batched  -- in-place natural-order transform of (m, n) rows
 //     (prover/cuda_primitives.py:388-409);
@@ -132,6 +133,30 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
     fast_stage2_512<INV>(A, tile, tid, lds);
 }
 
+// Rows of 2^10 .. 2^12 points: the whole transform in one launch (row_stage0), 16 >> A0 rows per workgroup.  The
+// tile crosses LDS twice (first digit -> last digit, and inside the last digit) and HBM not at all in between.
+// UNI: the last digit's stores through scalar-base addressing (rows of 2^12 points: a tile is one whole row).
+template <int A0, bool INV, bool UNI>
+__global__ __launch_bounds__(NTHREADS, 4) void k_ntt_row(const PassArgs P0, const PassArgs P1_in) {
+    PassArgs P1 = P1_in;
+    P1.is_final = 1;
+    __shared__ u64 lds[TILE + 256];                        // 16 columns of ROW_ST words, then 256 rows of 17
+    __shared__ u64 twi[256];
+    static_assert(16 * ROW_ST <= TILE + 256, "the columns of the first digit fit the exchange buffer of the last");
+    const int tid = threadIdx.x;
+    const i64 tile = blockIdx.x;
+    const u64 tw_mine = P1.twi[tid];
+    row_stage0<A0, INV>(P0, tile, tid, lds);
+    twi[twi_slot<4, true>(tid >> 4, tid & 15)] = tw_mine;
+    __syncthreads();
+    u64 reg[16];
+    row_gather(lds, tid, reg);
+    __syncthreads();                                       // every thread has its inputs: the buffer is free again
+    fast_stage1<4, INV, false, true>(P1, tile, tid, 0, 0xFFFFu, reg, reg, twi, lds);
+    __syncthreads();
+    fast_stage2<4, INV, UNI>(P1, tile, tid, 0, lds);
+}
+
 // The last inverse pass and the first forward pass of a coset extension in one launch (fused_stage2_inv): the
 // coefficients stay in registers between the two, so they are neither written to nor read back from HBM (unless the
 // caller wants them), and the rho cosets are expanded by a loop inside the workgroup.
@@ -198,7 +223,7 @@ struct DeviceTables {
 };
 
 std::mutex g_mu;
-std::map<std::tuple<int, int, int>, DeviceTables *> g_tables;        // (device, logn, inverse)
+std::map<std::tuple<int, int, int>, DeviceTables *> g_tables;        // (device, logn, inverse + 2 * row split)
 std::map<std::pair<int, int>, u64 *> g_twl;                          // (device, inverse)
 std::map<std::tuple<int, int, int, u64>, u64 *> g_pre;               // (device, logK, logN, shift)
 
@@ -229,14 +254,16 @@ int get_twl(int dev, int inv, const u64 **out) {
 
 // tables of one (logn, direction) on the current device; built on first use (which allocates and copies
 // synchronously; later calls with the same length only look the tables up)
-int get_tables(int logn, int inv, const Tables **out) {
+// row: the tables of the single-launch split of a short row (row_split) instead of split_digits
+int get_tables(int logn, int inv, const Tables **out, bool row = false) {
     int dev = 0;
     VI_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_mu);
-    auto key = std::make_tuple(dev, logn, inv);
+    auto key = std::make_tuple(dev, logn, inv + (row ? 2 : 0));
     auto it = g_tables.find(key);
     if (it == g_tables.end()) {
-        HostTables H = make_tables(logn, inv);
+        const Split rs = row_split(logn);
+        HostTables H = make_tables(logn, inv, row ? &rs : nullptr);
         DeviceTables *D = new DeviceTables();
         D->T.sp = H.sp;
         D->T.logn = logn;
@@ -390,6 +417,37 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
     return VI_OK;
 }
 
+// VI_NTT_ROW=0 (read once per process): rows of 2^10 .. 2^12 points as two launches through a workspace, like longer rows
+bool row_launch_on() {
+    static const bool on = []() { const char *e = getenv("VI_NTT_ROW"); return !(e && e[0] == '0'); }();
+    return on;
+}
+
+int launch_row(const PassArgs &P0, const PassArgs &P1, hipStream_t s) {
+    const i64 tiles = pass_tiles(P1);
+    if (tiles > 0x7FFFFFFF) return vi::fail(VI_EINVAL, "ntt pass: %lld tiles exceed the grid limit", (long long)tiles);
+    dim3 grid((unsigned)tiles), block(NTHREADS);
+    int nv = 16;
+    const bool uni = pass_uniform(P1, &nv) && nv == 16;
+    switch (P0.a * 2 + (P0.inverse ? 1 : 0)) {
+        case 4: hipLaunchKernelGGL((k_ntt_row<2, false, false>), grid, block, 0, s, P0, P1); break;
+        case 5: hipLaunchKernelGGL((k_ntt_row<2, true, false>), grid, block, 0, s, P0, P1); break;
+        case 6: hipLaunchKernelGGL((k_ntt_row<3, false, false>), grid, block, 0, s, P0, P1); break;
+        case 7: hipLaunchKernelGGL((k_ntt_row<3, true, false>), grid, block, 0, s, P0, P1); break;
+        case 8:
+            if (uni) hipLaunchKernelGGL((k_ntt_row<4, false, true>), grid, block, 0, s, P0, P1);
+            else hipLaunchKernelGGL((k_ntt_row<4, false, false>), grid, block, 0, s, P0, P1);
+            break;
+        case 9:
+            if (uni) hipLaunchKernelGGL((k_ntt_row<4, true, true>), grid, block, 0, s, P0, P1);
+            else hipLaunchKernelGGL((k_ntt_row<4, true, false>), grid, block, 0, s, P0, P1);
+            break;
+        default: return vi::fail(VI_EINVAL, "k_ntt_row: first digit of 2^%d points", P0.a);
+    }
+    VI_LAUNCH_CHECK("k_ntt_row");
+    return VI_OK;
+}
+
 // rows per launch so that grids stay below 2^31 tiles
 i64 max_rows_per_launch(int logn) { return ((i64)1 << 40) >> logn; }
 
@@ -412,6 +470,7 @@ extern "C" {
 
 size_t vi_ntt_workspace_bytes(int64_t m, int64_t n) {
     if (m <= 0 || !vi::is_pow2(n) || n < 2) return 0;
+    if (row_launch_on() && row_single_ok(vi::ilog2(n))) return 0;
     return split_digits(vi::ilog2(n)).p > 1 ? (size_t)m * (size_t)n * sizeof(u64) : 0;
 }
 
@@ -424,6 +483,18 @@ int vi_ntt_batched(uint64_t *rows, int64_t m, int64_t n, int inverse, void *ws, 
     if (!rows) return vi::fail(VI_EINVAL, "vi_ntt_batched: null rows");
     const int logn = vi::ilog2(n);
     const Tables *T = nullptr;
+    if (row_launch_on() && row_single_ok(logn)) {
+        int rc = get_tables(logn, inverse ? 1 : 0, &T, true);
+        if (rc) return rc;
+        const i64 cap = max_rows_per_launch(logn);
+        for (i64 lo = 0; lo < m; lo += cap) {
+            PassArgs P0, P1;
+            build_row_passes(*T, rows + lo * n, (m - lo < cap) ? (m - lo) : cap, P0, P1);
+            rc = launch_row(P0, P1, (hipStream_t)stream);
+            if (rc) return rc;
+        }
+        return VI_OK;
+    }
     int rc = get_tables(logn, inverse ? 1 : 0, &T);
     if (rc) return rc;
     i64 chunk = m;

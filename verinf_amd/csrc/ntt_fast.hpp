@@ -661,6 +661,58 @@ VI_HD void fused_stage2_fwd(const PassArgs &A, i64 tile, int tid, int t, const u
     }
 }
 
+// Rows of 2^(A0 + 8) points in one launch, A0 = 2, 3 or 4.  A tile is 16 >> A0 whole rows.  Thread r < 256 first
+// runs the 2^A0-point transforms over the elements r, r + 256, r + 512, ... of each of the tile's rows (the strided
+// first digit: P0 with a = A0, logR = 8) and multiplies by the inter-pass twiddles; the results go to LDS as the
+// sixteen 256-point columns [row, k][r] the last digit (P1, a = 8) works on, each padded to ROW_ST words so that the
+// four columns a wavefront gathers from start on alternating halves of the banks.  The last digit is the
+// register-blocked final pass (fast_stage1 / fast_stage2) with the gather from LDS in the place of its load.
+constexpr int ROW_ST = 256 + 16;
+template <int A0, bool INV>
+VI_HD void row_stage0(const PassArgs &A, i64 tile, int tid, u64 *lds) {
+    static_assert(NTHREADS == 256 && A0 >= 2 && A0 <= 4, "one thread per residue mod 256");
+    constexpr int E0 = 1 << A0, NSUB = 16 / E0;
+    u64 x[16], tw[E0];
+    u32 ok = 0;
+#pragma unroll
+    for (int j = 0; j < NSUB; ++j) {
+        const i64 row = tile * NSUB + j;
+#pragma unroll
+        for (int n1 = 0; n1 < E0; ++n1) {
+            const i64 idx = ((i64)n1 << 8) + tid;
+            const bool there = row < A.n_rows && idx < A.src_width;
+            ok |= there ? (1u << (j * E0 + n1)) : 0u;
+            x[j * E0 + n1] = A.src[there ? row * A.src_row_stride + idx : 0];
+        }
+    }
+    // w_n^(k r), the same for every row; row 0 of the table is 1 forward and 1/n inverse
+#pragma unroll
+    for (int k = 0; k < E0; ++k) tw[k] = (k > 0 || INV) ? A.tw[(k << 8) + tid] : 1;
+    fast_fix(A, ok, x);
+    VI_SCHED_FENCE();
+#pragma unroll
+    for (int j = 0; j < NSUB; ++j) {
+        u64 y[E0];
+#pragma unroll
+        for (int n1 = 0; n1 < E0; ++n1) y[n1] = x[j * E0 + n1];
+        dft_reg<A0, INV>(y);
+#pragma unroll
+        for (int k = 0; k < E0; ++k) {
+            u64 v = y[k];
+            if (k > 0 || INV) v = gl::mul(v, tw[k]);
+            lds[(j * E0 + k) * ROW_ST + tid] = v;
+        }
+        VI_SCHED_FENCE();
+    }
+}
+
+// the stage-1 inputs of the last digit, x[n1 * 16 + n2] of column c, out of the columns row_stage0 left in LDS
+VI_HD void row_gather(const u64 *lds, int tid, u64 (&reg)[16]) {
+    const int c = tid >> 4, n2 = tid & 15;
+#pragma unroll
+    for (int n1 = 0; n1 < 16; ++n1) reg[n1] = lds[c * ROW_ST + (n1 << 4) + n2];
+}
+
 // can passes Ai (last inverse) and Af (first forward, expanding into cosets) run as one fused launch?
 inline bool passes_fusable(const PassArgs &Ai_in, const PassArgs &Af_in) {
     PassArgs Ai = Ai_in, Af = Af_in;

@@ -31,6 +31,17 @@ inline Split split_digits(int logn) {
     return s;
 }
 
+// Rows of 2^10 .. 2^12 points as ONE launch (k_ntt_row): a first digit of 4, 8 or 16 points at stride 256 and a last
+// digit of 256 points, the tile (whole rows) staying in LDS between the two.
+inline bool row_single_ok(int logn) { return logn >= 10 && logn <= TILE_LOG; }
+inline Split row_split(int logn) {
+    Split s{};
+    s.p = 2;
+    s.a[0] = logn - MAX_A;
+    s.a[1] = MAX_A;
+    return s;
+}
+
 // host copies of the tables of one (logn, direction)
 struct HostTables {
     int logn, inverse;
@@ -40,11 +51,11 @@ struct HostTables {
     u64 scale;                  // 1/n when inverse and single pass, else 1
 };
 
-inline HostTables make_tables(int logn, int inv) {
+inline HostTables make_tables(int logn, int inv, const Split *split = nullptr) {
     HostTables H;
     H.logn = logn;
     H.inverse = inv;
-    H.sp = split_digits(logn);
+    H.sp = split ? *split : split_digits(logn);
     u64 n_inv = inverse(((u64)1 << logn) % gl::P);
     H.scale = (inv && H.sp.p == 1) ? n_inv : 1;
     int used = 0;
@@ -190,6 +201,20 @@ inline void build_ntt_passes(const Tables &T, u64 *buf, u64 *ws, i64 m, std::vec
         A.src_row_stride = A.dst_row_stride = n;
         out.push_back(A);
     }
+}
+
+// The same transform for rows of 2^10 .. 2^12 points as the pass pair of one k_ntt_row launch (T: tables of
+// row_split(logn)); no workspace.
+inline void build_row_passes(const Tables &T, u64 *buf, i64 m, PassArgs &P0, PassArgs &P1) {
+    const i64 n = (i64)1 << T.logn;
+    P0 = base_pass(T, 0, m);
+    P1 = base_pass(T, 1, m);
+    P0.src = buf;
+    P0.canon_src = 1;
+    P0.dst = nullptr;                                      // the intermediate stays in LDS
+    P1.src = nullptr;
+    P1.dst = buf;
+    P0.src_row_stride = P0.dst_row_stride = P1.src_row_stride = P1.dst_row_stride = n;
 }
 
 // Coset LDE of m rows:  in (m rows of `w` values, pitch in_stride)  ->  out (m, N).
