@@ -34,12 +34,26 @@ constexpr int MAX_DEG = 7;                  // samples per round <= 8
 constexpr int NSAMP = MAX_DEG + 1;
 constexpr int REG_TABLES = 8;               // tables a thread can keep in registers
 
+// A list of small numbers (< 256) inside a kernel argument, four to a 32-bit word.  An index that is the same for a
+// whole wavefront is then a scalar load of the word and a scalar shift.  As `unsigned char[N]` the compiler fetched an
+// entry with a byte load per lane from the argument segment: a round trip to memory in front of the table address, and
+// so of the table loads, that depend on it -- once per term of a thread's walk over the sum.
+template <int N>
+struct Bytes {
+    u32 w[(N + 3) / 4];
+    __host__ __device__ __forceinline__ int operator[](int j) const { return (int)((w[j >> 2] >> ((j & 3) * 8)) & 0xFFu); }
+    __host__ void set(int j, int v) {
+        const int sh = (j & 3) * 8;
+        w[j >> 2] = (w[j >> 2] & ~(0xFFu << sh)) | (((u32)v & 0xFFu) << sh);
+    }
+};
+
 struct Desc {
     const u64 *src[VI_SC_MAX_TABLES];
     u64 *dst[VI_SC_MAX_TABLES];
     u64 coeff[VI_SC_MAX_TERMS];
-    unsigned char term_off[VI_SC_MAX_TERMS + 1];
-    unsigned char fidx[VI_SC_MAX_FACTORS];
+    Bytes<VI_SC_MAX_TERMS + 1> term_off;
+    Bytes<VI_SC_MAX_FACTORS> fidx;
     // Several terms are stored factored:
     //   S(x) = common(x) * ( c0 + sum_k lin_coeff[k] f_lin[k](x) + sum_k coeff[k] prod_j f_kj(x) )
     // where `common` is a table every term contains (eq(z, .) in a batched gate check, layergkr/relations.py:117-121;
@@ -47,7 +61,7 @@ struct Desc {
     // factor is linear in x (its coefficient is applied once per pair to the value and the step of that factor,
     // not once per evaluation point), and coeff / term_off / fidx keep only the terms with two or more factors left.
     u64 lin_coeff[VI_SC_MAX_TERMS];
-    unsigned char lin_idx[VI_SC_MAX_TERMS];
+    Bytes<VI_SC_MAX_TERMS> lin_idx;
     u64 c0;
     int n_lin, common;
     int n_tables, n_terms, deg;
@@ -319,8 +333,8 @@ struct FoldOut {
     u64 r;
     int virt;
     int wb_common;
-    unsigned char wb_lin[VI_SC_MAX_TERMS];
-    unsigned char wb_fac[VI_SC_MAX_FACTORS];
+    Bytes<VI_SC_MAX_TERMS> wb_lin;
+    Bytes<VI_SC_MAX_FACTORS> wb_fac;
 };
 
 // NS: evaluation points kept per pair (4 when the degree is at most 3, else NSAMP).
@@ -345,9 +359,16 @@ struct TabLds {
 
 // Pair i of a round of `half` pairs: the samples of the factored sum into acc and, with FOLD, the tables folded by r
 // (row ty of ny rows of workgroups takes its share of the terms).
-template <int NS, bool FOLD, class TAB>
-__device__ __forceinline__ void eval_mem_pair(const Desc &D, const FoldOut &W, const LinFoldDesc *V, const TAB &T, u64 r, int skip1,
-                                              i64 i, i64 half, int ty, int ny, gl::Wide (&acc)[NS]) {
+// a thread's sample sums: five-word integers reduced at the end (k_tail_mem, whose threads see few pairs), or residues
+// added up pair by pair (k_eval_mem: twelve registers fewer, for one more wavefront per SIMD)
+__device__ __forceinline__ void acc_mul_add(gl::Wide &A, u64 a, u64 b) { gl::wide_mul_acc(A, a, b); }
+__device__ __forceinline__ void acc_mul_add(u64 &A, u64 a, u64 b) { A = gl::mul_add(a, b, A); }
+
+// SKIP: 1 = S(1) is not summed (the caller derives it from the round's known total), 0 = it is, -1 = as skip1 says
+template <int NS, bool FOLD, int SKIP, class TAB, class ACC>
+__device__ __forceinline__ void eval_mem_pair(const Desc &D, const FoldOut &W, const LinFoldDesc *V, const TAB &T, u64 r, int skip1_rt,
+                                              i64 i, i64 half, int ty, int ny, ACC (&acc)[NS]) {
+    const bool skip1 = SKIP < 0 ? skip1_rt != 0 : SKIP != 0;
     // the factored form described at Desc, every factor fetched from its table.  Loads go out in batches ahead
     // of the arithmetic that uses them (the common factor first, used last; four linear terms; two factor slots
     // of a product): one thread's loads are otherwise a chain of round trips to memory.  A slot past the end of
@@ -489,28 +510,29 @@ __device__ __forceinline__ void eval_mem_pair(const Desc &D, const FoldOut &W, c
         }
 #pragma unroll
         for (int x = 0; x < NS; ++x) {
-            if (x <= D.deg && !(skip1 && x == 1)) gl::wide_mul_acc(acc[x], gl::addc(lin[x], gl::wide_reduce(br[x])), cur);
+            if (x <= D.deg && !(skip1 && x == 1)) acc_mul_add(acc[x], gl::addc(lin[x], gl::wide_reduce(br[x])), cur);
             if (x + 1 < NS) cur = (x == 0) ? nxt : gl::addc(cur, dif);
         }
     }
 }
 
-template <int NS, bool FOLD>
+// SKIP1: D.skip1, fixed at compile time (the sample at 1 and everything that leads to it are not in the kernel then)
+template <int NS, bool FOLD, bool SKIP1>
 __global__ __launch_bounds__(BLOCK) void k_eval_mem(const Desc D, const FoldOut W, const LinFoldDesc V, i64 half, u64 *partial,
                                                     int accumulate, u64 scale) {
     __shared__ u64 red[BLOCK / 64][NSAMP];
     const int ty = blockIdx.y, ny = gridDim.y;
     const i64 stride = (i64)gridDim.x * BLOCK;
-    gl::Wide acc[NS];
+    u64 acc[NS];
 #pragma unroll
-    for (int x = 0; x < NS; ++x) gl::wide_zero(acc[x]);
+    for (int x = 0; x < NS; ++x) acc[x] = 0;
     const TabGlobal T{D};
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < half; i += stride)
-        eval_mem_pair<NS, FOLD>(D, W, &V, T, W.r, D.skip1, i, half, ty, ny, acc);
+        eval_mem_pair<NS, FOLD, SKIP1 ? 1 : 0>(D, W, &V, T, W.r, 0, i, half, ty, ny, acc);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
     for (int x = 0; x < NS; ++x) {
-        u64 v = wave_sum(gl::wide_reduce(acc[x]));
+        u64 v = wave_sum(acc[x]);
         if (lane == 0) red[w][x] = v;
     }
     __syncthreads();
@@ -608,16 +630,16 @@ void factor_terms(Desc &D, const int *term_off, const int *factor_idx, int n_ter
         if (nr == 0) {
             D.c0 = gl::add(D.c0, c);
         } else if (nr == 1) {
-            D.lin_idx[D.n_lin] = (unsigned char)rest[0];
+            D.lin_idx.set(D.n_lin, rest[0]);
             D.lin_coeff[D.n_lin++] = c;
         } else {
             D.coeff[n_prod] = c;
-            D.term_off[n_prod] = (unsigned char)n_fac;
-            for (int i = 0; i < nr; ++i) D.fidx[n_fac++] = (unsigned char)rest[i];
+            D.term_off.set(n_prod, n_fac);
+            for (int i = 0; i < nr; ++i) D.fidx.set(n_fac++, rest[i]);
             ++n_prod;
         }
     }
-    D.term_off[n_prod] = (unsigned char)n_fac;
+    D.term_off.set(n_prod, n_fac);
     D.n_terms = n_prod;
     // the first product term's coefficient leaves the sum: one multiplication per evaluation point less
     if (n_prod >= 1 && D.coeff[0] > 1) {
@@ -662,12 +684,12 @@ int fill_desc(Desc &D, const uint64_t *const *src, uint64_t *const *dst, int n_t
         if (nf < 1 || nf > MAX_DEG) return vi::fail(VI_EINVAL, "%s: term %d has %d factors (1..%d)", who, k, nf, MAX_DEG);
         if (nf > D.deg) D.deg = nf;
         D.coeff[k] = coeffs[k] % gl::P;
-        D.term_off[k] = (unsigned char)term_off[k];
+        D.term_off.set(k, term_off[k]);
     }
-    D.term_off[n_terms] = (unsigned char)term_off[n_terms];
+    D.term_off.set(n_terms, term_off[n_terms]);
     for (int j = 0; j < term_off[n_terms]; ++j) {
         if (factor_idx[j] < 0 || factor_idx[j] >= n_tables) return vi::fail(VI_EINVAL, "%s: factor index %d out of range", who, factor_idx[j]);
-        D.fidx[j] = (unsigned char)factor_idx[j];
+        D.fidx.set(j, factor_idx[j]);
     }
     D.coeff_at_end = (n_terms == 1);
     if (n_terms == 1 && n_tables <= REG_TABLES && !mem_path) D.out_scale = D.coeff[0];     // k_eval_mem applies it per term instead
@@ -779,8 +801,8 @@ int launch_round(const Desc &D, i64 half, u64 r, u64 *partial, int nb, u64 *out,
 // the common factor's values being used at the very end): W.wb_*.  Tables of D that no term fetches are returned in
 // `unused` (they are folded by a launch of their own).
 void fill_fold_flags(const Desc &D, FoldOut &W, std::vector<int> &unused) {
-    for (int k = 0; k < VI_SC_MAX_TERMS; ++k) W.wb_lin[k] = 0;
-    for (int j = 0; j < VI_SC_MAX_FACTORS; ++j) W.wb_fac[j] = 0;
+    for (int k = 0; k < VI_SC_MAX_TERMS; ++k) W.wb_lin.set(k, 0);
+    for (int j = 0; j < VI_SC_MAX_FACTORS; ++j) W.wb_fac.set(j, 0);
     W.wb_common = 0;
     std::vector<int> last_lin(D.n_tables, -1), last_fac(D.n_tables, -1);
     for (int k = 0; k < D.n_lin; ++k) last_lin[D.lin_idx[k]] = k;
@@ -790,17 +812,19 @@ void fill_fold_flags(const Desc &D, FoldOut &W, std::vector<int> &unused) {
     for (int t = 0; t < D.n_tables; ++t) {
         if (t == W.virt) continue;                       // written where it is formed
         if (t == D.common) W.wb_common = 1;
-        else if (last_fac[t] >= 0) W.wb_fac[last_fac[t]] = 1;
-        else if (last_lin[t] >= 0) W.wb_lin[last_lin[t]] = 1;
+        else if (last_fac[t] >= 0) W.wb_fac.set(last_fac[t], 1);
+        else if (last_lin[t] >= 0) W.wb_lin.set(last_lin[t], 1);
         else unused.push_back(t);
     }
 }
 
 // k_eval_mem over `half` pairs: returns the number of partial slots written (x workgroups times term rows).
 // W != NULL: the launch also writes every table folded by W->r (D.dst), see FoldOut.
-int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 scale, hipStream_t s,
-                    const FoldOut *W = nullptr, const LinFoldDesc *V = nullptr) {
-    // a grid-stride loop: no more workgroups than are resident at once (see resident_blocks), looked up per device
+// one instantiation of k_eval_mem over a grid-stride loop: no more workgroups than are resident at once (see
+// resident_blocks), looked up per instantiation and device
+template <int NS, bool FOLD, bool SKIP1>
+int launch_eval_mem_as(const Desc &D, const FoldOut &w, const LinFoldDesc &v, i64 half, u64 *partial, int accumulate, u64 scale,
+                       hipStream_t s) {
     static std::mutex mu;
     static int caps[64] = {0};
     int dev = 0;
@@ -808,27 +832,35 @@ int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 s
     int cap;
     {
         std::lock_guard<std::mutex> lock(mu);
-        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem<4, true>, 64);
+        if (!caps[dev]) caps[dev] = resident_blocks(k_eval_mem<NS, FOLD, SKIP1>, 64);
         cap = caps[dev];
     }
     int nbx = blocks_for(half);
     if (nbx > cap) nbx = cap;
     int ny = 1;
-    if (!W)
+    if (!FOLD)
         while (ny < 16 && nbx * ny * 2 <= 1024) ny *= 2;     // deal the terms out while the grid is below ~4 workgroups per CU
+    const dim3 grid(nbx, ny), block(BLOCK);
+    hipLaunchKernelGGL((k_eval_mem<NS, FOLD, SKIP1>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
+    return nbx * ny;
+}
+
+int launch_eval_mem(const Desc &D, i64 half, u64 *partial, int accumulate, u64 scale, hipStream_t s,
+                    const FoldOut *W = nullptr, const LinFoldDesc *V = nullptr) {
     static const FoldOut no_fold = {};
     static const LinFoldDesc no_virt = {};
     const FoldOut &w = W ? *W : no_fold;
     const LinFoldDesc &v = V ? *V : no_virt;
-    const dim3 grid(nbx, ny), block(BLOCK);
-    if (W) {
-        if (D.deg <= 3) hipLaunchKernelGGL((k_eval_mem<4, true>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
-        else hipLaunchKernelGGL((k_eval_mem<NSAMP, true>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
-    } else {
-        if (D.deg <= 3) hipLaunchKernelGGL((k_eval_mem<4, false>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
-        else hipLaunchKernelGGL((k_eval_mem<NSAMP, false>), grid, block, 0, s, D, w, v, half, partial, accumulate, scale);
+    switch ((W ? 4 : 0) + (D.deg <= 3 ? 2 : 0) + (D.skip1 ? 1 : 0)) {
+        case 7: return launch_eval_mem_as<4, true, true>(D, w, v, half, partial, accumulate, scale, s);
+        case 6: return launch_eval_mem_as<4, true, false>(D, w, v, half, partial, accumulate, scale, s);
+        case 5: return launch_eval_mem_as<NSAMP, true, true>(D, w, v, half, partial, accumulate, scale, s);
+        case 4: return launch_eval_mem_as<NSAMP, true, false>(D, w, v, half, partial, accumulate, scale, s);
+        case 3: return launch_eval_mem_as<4, false, true>(D, w, v, half, partial, accumulate, scale, s);
+        case 2: return launch_eval_mem_as<4, false, false>(D, w, v, half, partial, accumulate, scale, s);
+        case 1: return launch_eval_mem_as<NSAMP, false, true>(D, w, v, half, partial, accumulate, scale, s);
+        default: return launch_eval_mem_as<NSAMP, false, false>(D, w, v, half, partial, accumulate, scale, s);
     }
-    return nbx * ny;
 }
 
 // fold `n` tables by r: up to REG_TABLES through the register kernel, more through k_fold_many (FOLD_MANY per launch)
@@ -1289,14 +1321,14 @@ __global__ __launch_bounds__(TAIL_THREADS) void k_tail_mem(const Desc D, const C
         const int skip1 = k > 0 ? 1 : 0;
         if (half >= TAIL_THREADS) {
             for (int i = tid; i < half; i += TAIL_THREADS)
-                eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, 0, 1, acc);
+                eval_mem_pair<NS, false, -1>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, 0, 1, acc);
         } else {
             // row ty of ny takes its share of the terms of pair i; no more rows than there are shares (every row pays
             // for the common factor and the reductions of its sums, and the workgroup has one CU to run on)
             int ny = TAIL_THREADS >> log_half;
             if (ny > rows) ny = rows;
             const int ty = tid >> log_half, i = tid & (half - 1);
-            if (ty < ny) eval_mem_pair<NS, false>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, ty, ny, acc);
+            if (ty < ny) eval_mem_pair<NS, false, -1>(D, none, nullptr, T, 0, skip1, (i64)i, (i64)half, ty, ny, acc);
         }
         // the wavefront's sums of this round, the samples side by side so that their shuffles are in flight together;
         // the wavefronts are added up for all rounds at once behind the loop
