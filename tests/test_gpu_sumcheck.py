@@ -135,13 +135,15 @@ def test_more_tables_than_fit_in_registers(mods):
 
 
 @pytest.mark.parametrize("nt,v", [(9, 1), (9, 4), (12, 9), (22, 8), (23, 8), (44, 7), (45, 7), (64, 6), (10, 11),
-                                  (3, 1), (3, 9), (5, 9), (5, 10), (6, 5), (8, 9), (8, 10), (7, 3)])
+                                  (3, 1), (3, 9), (5, 9), (5, 10), (6, 5), (8, 9), (8, 10), (7, 3),
+                                  (5, 13), (8, 12), (3, 16), (2, 11)])
 def test_last_rounds_from_lds_around_the_capacity(mods, nt, v):
     """Sums at sizes around what one workgroup's LDS holds of their tables (5632 words in all, nine rounds): the
     whole proof inside the single-workgroup launch (round 0 included, which sums every sample), a proof whose first
     rounds run as separate launches, table counts just below and just above the capacity at a size, a common factor
     with linear terms, and a term of degree five (eight samples kept per pair).  With at most eight tables the sizes
-    above the capacity run one launch per round with the tables in registers, and both must agree with the oracle."""
+    above the capacity run one launch per round with the tables in registers until the tables fit, fold them into
+    place and hand over to the single-workgroup launch; all must agree with the oracle."""
     gpu, _ = mods
     r = random.Random(1000 * nt + v)
     tabs = [rand_field(1 << v, 3000 + 37 * nt + j) for j in range(nt)]
@@ -151,6 +153,19 @@ def test_last_rounds_from_lds_around_the_capacity(mods, nt, v):
     if 6 <= nt <= 12:
         terms5 = [(r.randrange(P), [j, (j + 1) % nt]) for j in range(nt)] + [(5, [1, 2, 3, 4, 5])]
         _check(gpu, tabs, terms5, 11 * nt + v, as_tensor=True)
+
+
+@pytest.mark.parametrize("v", [4, 11, 14])
+def test_single_term_sums_with_a_coefficient(mods, v):
+    """One term with a coefficient other than 1 (applied once at the end by the register kernels, per term by the
+    single-workgroup launch, so these proofs keep one launch per round above the LDS capacity and are one launch
+    below it): a factor twice in the term, five distinct factors, and the coefficient 1, which does hand over."""
+    gpu, _ = mods
+    r = random.Random(77 + v)
+    tabs = [rand_field(1 << v, 8100 + j) for j in range(5)]
+    _check(gpu, tabs[:2], [(r.randrange(2, P), [0, 0, 1])], 3 * v, as_tensor=True)
+    _check(gpu, tabs, [(r.randrange(2, P), [0, 1, 2, 3, 4])], 5 * v, as_tensor=True)
+    _check(gpu, tabs, [(1, [0, 1, 2, 3, 4])], 7 * v, as_tensor=True)
 
 
 def _layer_gate_batch(n_had, n_resc, n_bool, n_aff, v, seed):

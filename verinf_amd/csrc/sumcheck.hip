@@ -1654,8 +1654,30 @@ int prove_coins_impl(const char *who, const uint64_t *const *tables, uint64_t *c
         const bool regs = n_tables <= REG_TABLES;
         C.scale = D.out_scale;
         if (regs) {
+            // the same sum as k_tail_mem reads it (a single term's coefficient per term there, at the end here: the
+            // two must scale the samples alike for the tail to take over part of the way)
+            Desc M;
+            rc = fill_desc(M, tables, work, n_tables, term_off, factor_idx, coeffs, n_terms, true, who, true);
+            if (rc) return rc;
+            const bool tail_ok = M.out_scale == D.out_scale;
             for (int k = 0; k < v; ++k, half >>= 1) {
                 int nb;
+                if (k > 0 && tail_ok && (i64)n_tables * 2 * half <= TAIL_MEM_WORDS && v - k <= TAIL_MEM_ROUNDS) {
+                    // every table of this round fits one workgroup's LDS: fold into place, then all remaining rounds
+                    // in one launch
+                    rc = fold_tables(k == 1 ? D.src : (const uint64_t *const *)D.dst, D.dst, n_tables, 2 * half, C.r[k - 1], s, k == 1);
+                    if (rc) return rc;
+                    for (int t = 0; t < n_tables; ++t) M.src[t] = D.dst[t];
+                    const int shares = std::max(std::max(M.n_terms, (M.n_lin + 3) / 4), 1);
+                    int rows = 1;
+                    while (rows < shares) rows <<= 1;
+                    for (int j = k; j < v; ++j) C.skip_mask |= 1ull << j;
+                    C.n_prior = k;
+                    if (M.deg <= 3) hipLaunchKernelGGL(k_tail_mem<4>, dim3(1), dim3(TAIL_THREADS), 0, s, M, C, rows, (int)(2 * half), (const u64 *)part, samples);
+                    else hipLaunchKernelGGL(k_tail_mem<NSAMP>, dim3(1), dim3(TAIL_THREADS), 0, s, M, C, rows, (int)(2 * half), (const u64 *)part, samples);
+                    VI_LAUNCH_CHECK("sumcheck tail (tables folded into place)");
+                    return VI_OK;
+                }
                 if (k == 0) {
                     nb = launch_round<0>(D, half, 0, part + off, blocks_for(half), nullptr, 1, 0, 0, s);
                     VI_LAUNCH_CHECK("sumcheck eval");
