@@ -59,6 +59,7 @@ void run_fast_u(const PassArgs &A) {
 }
 
 int g_allow_uniform = 1;
+long g_single_uniform_runs = 0;             // single-pass transforms that ran with scalar-base addressing
 int g_allow_merged = 1;
 int g_allow_half = 1;
 long g_half_runs = 0;                       // first passes that skipped the zero half of their inputs
@@ -69,6 +70,7 @@ template <int A2, bool INV>
 void run_fast(const PassArgs &A_in) {
     PassArgs A = A_in;
     A.uniform = (g_allow_uniform && pass_uniform(A, &A.n1_valid)) ? 1 : 0;
+    if (A.uniform && A.is_final && A.ndig == 0) ++g_single_uniform_runs;
     if (INV && A.uniform && g_allow_half && upper_half_zero(A)) { ++g_half_runs; run_fast_u<A2, INV, true, true>(A); }
     else if (A.uniform) run_fast_u<A2, INV, true>(A);
     else run_fast_u<A2, INV, false>(A);
@@ -135,25 +137,34 @@ void run_row(const PassArgs &P0, const PassArgs &P1_in) {
 // runs passes[q] (and passes[q + 1] with it when the two fuse); returns how many passes it consumed
 int run_passes_at(const std::vector<PassArgs> &passes, size_t q);
 
-template <bool INV>
-void run_512(const PassArgs &A_in) {
-    PassArgs A = A_in;
-    A.is_final = 1;
+template <bool INV, bool UNI>
+void run_512_u(const PassArgs &A) {
     i64 tiles = pass_tiles(A);
     std::vector<u64> lds(fast_lds_words(A.a));
     std::vector<u64> regs((size_t)NTHREADS * 16);
     std::vector<u32> oks(NTHREADS);
     for (i64 tile = 0; tile < tiles; ++tile) {
         for (int tid = 0; tid < NTHREADS; ++tid)
-            fast_load<5, false>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
+            fast_load<5, UNI>(A, tile, tid, *reinterpret_cast<u64(*)[16]>(&regs[(size_t)tid * 16]), oks[tid]);
         for (int tid = 0; tid < NTHREADS; ++tid) {
             u64 pw[16] = {};
             if (A.pre) fast_pre_load<5, false>(A, tile, tid, 0, pw);
             fast_stage1<5, INV>(A, tile, tid, 0, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]), pw,
                                 A.twi, lds.data());
         }
-        for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2_512<INV>(A, tile, tid, lds.data());
+        for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2_512<INV, UNI>(A, tile, tid, lds.data());
     }
+}
+
+// the launcher's choice: contiguous whole tiles through scalar-base addressing
+template <bool INV>
+void run_512(const PassArgs &A_in) {
+    PassArgs A = A_in;
+    A.is_final = 1;
+    A.uniform = (g_allow_uniform && pass_uniform(A, &A.n1_valid)) ? 1 : 0;
+    if (A.uniform) ++g_single_uniform_runs;
+    if (A.uniform) run_512_u<INV, true>(A);
+    else run_512_u<INV, false>(A);
 }
 
 void run_pass(const PassArgs &A) {
@@ -228,6 +239,7 @@ u64 emu_sub(u64 a, u64 b) { return gl::sub(a, b); }
 u64 emu_mul_pow2(u64 x, unsigned s) { return gl::mul_pow2(x, s); }
 u64 emu_inv(u64 x) { return gl::inv(x); }
 
+long emu_single_uniform_runs() { return g_single_uniform_runs; }
 void emu_set_row(int on) { g_allow_row = on; }
 long emu_row_runs() { return g_row_runs; }
 

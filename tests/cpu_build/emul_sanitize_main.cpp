@@ -68,6 +68,9 @@ int main() {
         bad += check_ntt(12, 1);
     }
     emu_set_row(1);
+    // single-pass transforms over whole tiles (scalar-base addressing) and over a batch that ends inside a tile
+    const int whole[][2] = {{5, 128}, {6, 64}, {7, 64}, {8, 16}, {8, 32}, {9, 8}, {9, 16}, {8, 15}, {9, 7}};
+    for (auto &s : whole) bad += check_ntt(s[0], s[1]);
     const long lde[][5] = {
         // logK logN m width in_stride
         {4, 6, 3, 16, 16},   {4, 6, 3, 9, 11},    {5, 7, 130, 32, 32}, {6, 8, 65, 33, 64},   {8, 10, 17, 256, 300},

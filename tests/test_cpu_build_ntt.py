@@ -37,6 +37,7 @@ def emu():
     L.emu_merged_runs.restype = c_long
     L.emu_set_half.argtypes = [c_int]
     L.emu_half_runs.restype = c_long
+    L.emu_single_uniform_runs.restype = c_long
     L.emu_set_row.argtypes = [c_int]
     L.emu_row_runs.restype = c_long
     L.emu_ntt_batched.argtypes = [u64p, c_long, c_int, c_int]
@@ -137,6 +138,29 @@ def test_short_rows_in_one_launch(emu, logn, m):
         b = _rand((2, 1 << other), 7)
         emu.emu_ntt_batched(_p(b), 2, other, 0)
         assert emu.emu_row_runs() == before
+
+
+@pytest.mark.parametrize("logn,m,whole", [(5, 128, True), (5, 256, True), (5, 129, False), (6, 64, True), (7, 32, True), (7, 96, True),
+                                          (8, 16, True), (8, 48, True), (8, 17, False), (9, 8, True), (9, 24, True), (9, 9, False)])
+def test_single_pass_rows_in_whole_tiles(emu, logn, m, whole):
+    """A transform of at most 512 points is one pass over tiles of 4096 / n rows.  When the batch is a whole number of
+    tiles (and the rows are contiguous) the tiles are addressed through scalar bases; a batch that is not keeps the
+    per-element path.  Both against the oracle, forward and inverse, with words at and above p in the input."""
+    a = _rand((m, 1 << logn), 1300 + 17 * logn + m)
+    raw = a.copy()
+    raw[m - 1, -3:] = np.array([P, P + 7, (1 << 64) - 1], dtype=np.uint64)
+    a[m - 1, -3:] = raw[m - 1, -3:] % np.uint64(P)
+    want = O.ntt_rows(a)
+    for uni in (1, 0):
+        _set_mode(emu, 1, uni, 1, 1)
+        before = emu.emu_single_uniform_runs()
+        got = raw.copy()
+        emu.emu_ntt_batched(_p(got), m, logn, 0)
+        assert np.array_equal(got, want), uni
+        emu.emu_ntt_batched(_p(got), m, logn, 1)
+        assert np.array_equal(got, a), uni
+        assert emu.emu_single_uniform_runs() - before == (2 if (uni and whole) else 0)
+    _set_mode(emu, 1, 1, 1, 1)
 
 
 def test_ntt_25_bit_split_is_well_formed(emu):

@@ -42,7 +42,8 @@ def test_ntt_small_sizes_match_definition(cp, n):
 
 @pytest.mark.parametrize("logn,m", [(1, 5), (3, 1000), (5, 77), (8, 33), (9, 9), (10, 6), (11, 5), (12, 16), (13, 3),
                                     (14, 8), (15, 8), (16, 8), (17, 2), (18, 3), (20, 2),
-                                    (10, 1), (10, 1023), (11, 1), (11, 514), (12, 1), (12, 257)])
+                                    (10, 1), (10, 1023), (11, 1), (11, 514), (12, 1), (12, 257),
+                                    (5, 128), (5, 1280), (6, 64), (7, 32), (8, 16), (8, 4096), (9, 8), (9, 1032)])
 def test_batched_ntt_matches_oracle(cp, logn, m):
     a = rand_field((m, 1 << logn), 100 + logn)
     rows = to_dev(a)

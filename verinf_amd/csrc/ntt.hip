@@ -109,7 +109,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
 
 
 // 512-point rows: one pass, 16 x 32 (fast_stage2_512); eight rows (or row-coset pairs) per workgroup
-template <bool INV>
+template <bool INV, bool UNI>
 __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
     PassArgs A = A_in;
     A.is_final = 1;
@@ -123,14 +123,14 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
     for (int i = 0; i < 2; ++i) tw_mine[i] = A.twi[tid + i * NTHREADS];
     u64 reg[16], pw[16];
     u32 ok;
-    if (A.pre) fast_pre_load<A2, false>(A, tile, tid, 0, pw);
-    fast_load<A2, false>(A, tile, tid, reg, ok);
+    if (A.pre) fast_pre_load<A2, false>(A, tile, tid, 0, pw);      // never in a uniform pass
+    fast_load<A2, UNI>(A, tile, tid, reg, ok);
 #pragma unroll
     for (int i = 0; i < 2; ++i) twi[twi_slot<A2, true>((tid + i * NTHREADS) >> 4, (tid + i * NTHREADS) & 15)] = tw_mine[i];
     __syncthreads();
     fast_stage1<A2, INV, false, true>(A, tile, tid, 0, ok, reg, pw, twi, lds);
     __syncthreads();
-    fast_stage2_512<INV>(A, tile, tid, lds);
+    fast_stage2_512<INV, UNI>(A, tile, tid, lds);
 }
 
 // Rows of 2^10 .. 2^12 points: the whole transform in one launch (row_stage0), 16 >> A0 rows per workgroup.  The
@@ -407,8 +407,15 @@ int launch_passes(const std::vector<PassArgs> &passes, hipStream_t s) {
             if (!A.is_final && A.loop_cosets) grid.x <<= A.log_rho;       // tiles * rho <= 2^31 by max_rows_per_launch
             launch_fast(A, grid, block, s);
         } else if (fast512_ok(A.a) && A.twi && A.is_final) {
-            if (A.inverse) hipLaunchKernelGGL(k_ntt_512<true>, grid, block, 0, s, A);
-            else hipLaunchKernelGGL(k_ntt_512<false>, grid, block, 0, s, A);
+            PassArgs U = A;
+            U.is_final = 1;
+            U.uniform = pass_uniform(U, &U.n1_valid) ? 1 : 0;
+            switch ((U.inverse ? 2 : 0) + U.uniform) {
+                case 0: hipLaunchKernelGGL((k_ntt_512<false, false>), grid, block, 0, s, U); break;
+                case 1: hipLaunchKernelGGL((k_ntt_512<false, true>), grid, block, 0, s, U); break;
+                case 2: hipLaunchKernelGGL((k_ntt_512<true, false>), grid, block, 0, s, U); break;
+                default: hipLaunchKernelGGL((k_ntt_512<true, true>), grid, block, 0, s, U); break;
+            }
         } else {
             hipLaunchKernelGGL(k_ntt_pass, grid, block, 0, s, A);
         }

@@ -138,6 +138,7 @@ struct TileU {
     int sh2;          // log2 of the element stride between a thread's stage-2 outputs k2, k2 + 1
     int shk;          // log2 of the element stride between outputs k1, k1 + 1
     int shc;          // final pass: log2 of the source stride between column groups (c >> log_rho)
+    int shcd;         // log2 of the output stride between columns (0 except in a single-pass transform, whose columns are rows)
 };
 
 // does the pass qualify?  On success *n1_valid = how many of a thread's sixteen stage-1 inputs exist (the first
@@ -161,6 +162,12 @@ inline bool pass_uniform(const PassArgs &A, int *n1_valid) {
         *n1_valid = (int)(A.src_width >> sh1);
         return true;
     }
+    if (A.ndig == 0) {
+        // a single-pass transform of contiguous rows: a tile is 2^lt whole rows = TILE consecutive words, in and out
+        if (A.pre || A.log_rho != 0 || A.B != 0 || A.logR != 0 || A.a != A.logn) return false;
+        if (A.src_width != n || A.src_row_stride != n || A.dst_row_stride != n) return false;
+        return (A.n_rows & (((i64)1 << lt) - 1)) == 0;
+    }
     const int lc = A.B + A.log_rho;
     if (A.pre || A.ndig < 1 || lc < lt || lt < A.log_rho || lt - A.log_rho > A.dig[0]) return false;
     if (A.src_width != n || A.logn + A.log_rho > 28) return false;
@@ -179,7 +186,7 @@ template <int A2>
 VI_HD TileU tile_uniform(const PassArgs &A, i64 tile) {
     TileU U;
     U.src_u = U.dst_u = U.pre_u = U.tw_u = 0;
-    U.sh1 = U.sh2 = U.shk = U.shc = 0;
+    U.sh1 = U.sh2 = U.shk = U.shc = U.shcd = 0;
     const int lt = logT(A);
     if (!A.is_final) {
         const int lc = A.B + A.logR;
@@ -194,6 +201,15 @@ VI_HD TileU tile_uniform(const PassArgs &A, i64 tile) {
         U.sh1 = A2 + A.logR;
         U.sh2 = 4 + A.logR;
         U.shk = A.logR;
+    } else if (A.ndig == 0) {
+        // single-pass transform: column c of the tile is row (tile << lt) + c, point l of it word (c << a) + l of the tile
+        U.src_u = (tile << lt) * A.src_row_stride;
+        U.dst_u = (tile << lt) * A.dst_row_stride;
+        U.sh1 = A2;
+        U.sh2 = 4;
+        U.shk = 0;
+        U.shc = A.a;
+        U.shcd = A.a;
     } else {
         const int lc = A.B + A.log_rho;
         const i64 row = tile >> (lc - lt);
@@ -405,7 +421,7 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
 #pragma unroll
         for (int i = 0; i < 16 / E2; ++i) {
             const int k1 = (tid + i * NTHREADS) >> lt;
-            const u32 off = (u32)c + ((u32)k1 << U.shk);
+            const u32 off = ((u32)c << U.shcd) + ((u32)k1 << U.shk);
             u64 x[E2], tw[E2];
             if (!A.is_final) {
 #pragma unroll
@@ -467,14 +483,15 @@ VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u
 // x[j] + x[j + 16] and gets the even outputs from a 16-point transform, thread h = 1 forms the differences times
 // w_32^j (shifts) and gets the odd outputs -- no exchange between the two.  h is the top bit of the thread id, so a
 // wavefront is all sums or all differences.  Per-element addressing (a single pass is never a uniform pass).
-template <bool INV>
+template <bool INV, bool UNI = false>
 VI_HD void fast_stage2_512(const PassArgs &A, i64 tile, int tid, const u64 *lds) {
     constexpr int A2 = 5;
     const int lt = logT(A);                                // 3: eight columns per tile
     const int st = (1 << lt) + 1;
     const int c = tid & ((1 << lt) - 1);
     const int k1 = (tid >> lt) & 15, h = tid >> (lt + 4);
-    const ColRef R = col_ref(A, tile, c);
+    ColRef R{};
+    if (!UNI) R = col_ref(A, tile, c);
     const int lc = A.B + A.log_rho;
     u64 x[32], y[16];
 #pragma unroll
@@ -495,6 +512,18 @@ VI_HD void fast_stage2_512(const PassArgs &A, i64 tile, int tid, const u64 *lds)
     VI_SCHED_FENCE();
     dft_reg<4, INV>(y);
     VI_SCHED_FENCE();
+    if constexpr (UNI) {                                   // contiguous rows (pass_uniform): output k of column c is word (c << 9) + k of the tile
+        const TileU U = tile_uniform<A2>(A, tile);
+        const URun dst = urun(A.dst + U.dst_u);
+        const u32 off = ((u32)c << U.shcd) + (u32)k1 + 16u * (u32)h;
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            u64 v = y[m];
+            if (A.scale != 1) v = gl::mul(v, A.scale);
+            ustore_stream(dst, 32u * (u32)m, off, v);
+        }
+        return;
+    }
     if (!R.valid) return;
 #pragma unroll
     for (int m = 0; m < 16; ++m) {
