@@ -373,7 +373,7 @@ def bench_ntt(torch, steps=20):
     2^8 ... 2^20: in place, round trip checked."""
     from verinf_amd.prover import cuda_primitives as cp
     res = {}
-    for logn in (8, 9, 12, 16, 20):
+    for logn in (8, 9, 10, 11, 12, 16, 20):
         rows = rand_field(torch, (1 << (26 - logn), 1 << logn), 40 + logn)
         keep = rows.clone()
         for _ in range(steps):
