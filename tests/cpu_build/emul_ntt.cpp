@@ -35,10 +35,10 @@ Owned *make_owned(int logn, int inv, bool row = false) {
 
 int g_use_fast = 1;
 
-template <int A2, bool INV, bool UNI, bool HALF = false>
+template <int A2, bool INV, bool UNI, bool HALF = false, bool SGL = false>
 void run_fast_u(const PassArgs &A) {
     i64 tiles = pass_tiles(A);
-    std::vector<u64> lds(fast_lds_words(A.a));
+    std::vector<u64> lds(SGL ? SglLds<A2>::WORDS : fast_lds_words(A.a));
     std::vector<u64> regs((size_t)NTHREADS * 16);
     std::vector<u32> oks(NTHREADS);
     int n_loop = (!A.is_final && A.loop_cosets) ? (1 << A.log_rho) : 1;
@@ -50,10 +50,10 @@ void run_fast_u(const PassArgs &A) {
             {
                 u64 pw[16] = {};
                 if (A.pre) fast_pre_load<A2, UNI>(A, tile, tid, t, pw);
-                fast_stage1<A2, INV, HALF>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
-                                           pw, A.twi, lds.data());
+                fast_stage1<A2, INV, HALF, false, SGL>(A, tile, tid, t, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]),
+                                                       pw, A.twi, lds.data());
             }
-            for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds.data());
+            for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2<A2, INV, UNI, SGL>(A, tile, tid, t, lds.data());
         }
     }
 }
@@ -70,7 +70,11 @@ template <int A2, bool INV>
 void run_fast(const PassArgs &A_in) {
     PassArgs A = A_in;
     A.uniform = (g_allow_uniform && pass_uniform(A, &A.n1_valid)) ? 1 : 0;
-    if (A.uniform && A.is_final && A.ndig == 0) ++g_single_uniform_runs;
+    if (A.uniform && A.is_final && A.ndig == 0) {          // the launcher's choice of the whole-tile form
+        ++g_single_uniform_runs;
+        run_fast_u<A2, INV, true, false, true>(A);
+        return;
+    }
     if (INV && A.uniform && g_allow_half && upper_half_zero(A)) { ++g_half_runs; run_fast_u<A2, INV, true, true>(A); }
     else if (A.uniform) run_fast_u<A2, INV, true>(A);
     else run_fast_u<A2, INV, false>(A);
@@ -140,7 +144,7 @@ int run_passes_at(const std::vector<PassArgs> &passes, size_t q);
 template <bool INV, bool UNI>
 void run_512_u(const PassArgs &A) {
     i64 tiles = pass_tiles(A);
-    std::vector<u64> lds(fast_lds_words(A.a));
+    std::vector<u64> lds(UNI ? SglLds<5>::WORDS : fast_lds_words(A.a));
     std::vector<u64> regs((size_t)NTHREADS * 16);
     std::vector<u32> oks(NTHREADS);
     for (i64 tile = 0; tile < tiles; ++tile) {
@@ -149,8 +153,8 @@ void run_512_u(const PassArgs &A) {
         for (int tid = 0; tid < NTHREADS; ++tid) {
             u64 pw[16] = {};
             if (A.pre) fast_pre_load<5, false>(A, tile, tid, 0, pw);
-            fast_stage1<5, INV>(A, tile, tid, 0, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]), pw,
-                                A.twi, lds.data());
+            fast_stage1<5, INV, false, false, UNI>(A, tile, tid, 0, oks[tid], *reinterpret_cast<const u64(*)[16]>(&regs[(size_t)tid * 16]), pw,
+                                                   A.twi, lds.data());
         }
         for (int tid = 0; tid < NTHREADS; ++tid) fast_stage2_512<INV, UNI>(A, tile, tid, lds.data());
     }

@@ -52,11 +52,13 @@ __global__ __launch_bounds__(NTHREADS) void k_ntt_pass(const PassArgs A) {
 // UNI: compiled for passes whose tiles are all addressed by scalar bases plus 32-bit thread offsets (pass_uniform).
 // HALF: the first pass over source rows at most half as wide as the transform (upper_half_zero): eight of a thread's
 // sixteen inputs are zero, so they are not loaded and the first butterfly level of stage 1 is skipped.
-template <int A2, bool INV, bool FIN, bool UNI, bool HALF = false>
+// SGL: a single-pass transform over whole tiles of contiguous rows (pass_uniform): stage 2 stores along output rows.
+template <int A2, bool INV, bool FIN, bool UNI, bool HALF = false, bool SGL = false>
 __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     PassArgs A = A_in;
     if (FIN) A.is_final = 1;
-    __shared__ u64 lds[TILE + (16 << A2)];
+    static_assert(!SGL || (FIN && UNI && !HALF), "whole-tile single-pass transforms are uniform final passes");
+    __shared__ u64 lds[SGL ? SglLds<A2>::WORDS : TILE + (16 << A2)];
     __shared__ u64 twi[16 << A2];
     const int tid = threadIdx.x;
     // A pass that expands one source tile into rho cosets runs rho workgroups per tile, the coset being the low
@@ -102,9 +104,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
             if (tid + i * NTHREADS < (16 << A2)) twi[twi_slot<A2, FIN>((tid + i * NTHREADS) >> 4, (tid + i * NTHREADS) & 15)] = tw_mine[i];
         __syncthreads();
     }
-    fast_stage1<A2, INV, HALF, FIN>(A, tile, tid, t, ok, reg, pw, twi, lds);
+    fast_stage1<A2, INV, HALF, FIN, SGL>(A, tile, tid, t, ok, reg, pw, twi, lds);
     __syncthreads();
-    fast_stage2<A2, INV, UNI>(A, tile, tid, t, lds);
+    fast_stage2<A2, INV, UNI, SGL>(A, tile, tid, t, lds);
 }
 
 
@@ -114,7 +116,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
     PassArgs A = A_in;
     A.is_final = 1;
     constexpr int A2 = 5;
-    __shared__ u64 lds[TILE + (16 << A2)];
+    __shared__ u64 lds[UNI ? SglLds<A2>::WORDS : TILE + (16 << A2)];
     __shared__ u64 twi[16 << A2];
     const int tid = threadIdx.x;
     const i64 tile = blockIdx.x;
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_512(const PassArgs A_in) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) twi[twi_slot<A2, true>((tid + i * NTHREADS) >> 4, (tid + i * NTHREADS) & 15)] = tw_mine[i];
     __syncthreads();
-    fast_stage1<A2, INV, false, true>(A, tile, tid, 0, ok, reg, pw, twi, lds);
+    fast_stage1<A2, INV, false, true, UNI>(A, tile, tid, 0, ok, reg, pw, twi, lds);
     __syncthreads();
     fast_stage2_512<INV, UNI>(A, tile, tid, lds);
 }
@@ -351,7 +353,10 @@ void launch_fast_a(const PassArgs &A_in, dim3 grid, dim3 block, hipStream_t s) {
     A.uniform = pass_uniform(A, &A.n1_valid) ? 1 : 0;
     if (A.uniform && A.inverse && upper_half_zero(A))
         hipLaunchKernelGGL((k_ntt_fast<A2, true, false, true, true>), grid, block, 0, s, A);
-    else if (A.uniform) launch_fast_u<A2, true>(A, grid, block, s);
+    else if (A.uniform && A.is_final && A.ndig == 0) {     // single-pass transform over whole tiles
+        if (A.inverse) hipLaunchKernelGGL((k_ntt_fast<A2, true, true, true, false, true>), grid, block, 0, s, A);
+        else hipLaunchKernelGGL((k_ntt_fast<A2, false, true, true, false, true>), grid, block, 0, s, A);
+    } else if (A.uniform) launch_fast_u<A2, true>(A, grid, block, s);
     else launch_fast_u<A2, false>(A, grid, block, s);
 }
 

@@ -350,6 +350,26 @@ VI_HD void fast_fix(const PassArgs &A, u32 ok, u64 (&reg)[16]) {
 template <int A2, bool TWT>
 VI_HD constexpr int twi_slot(int n2, int k1) { return TWT ? (k1 << A2) + n2 : n2 * 16 + k1; }
 
+// Where (k1, n2, column c) sits in LDS between the two stages: [k1][n2][c] with one word of padding per (k1, n2) row.
+// SGL (a single-pass transform over whole tiles, pass_uniform): stage 2 runs k1 along the lanes there, so that a
+// wavefront's stores are 128-byte runs of output rows (with the columns along the lanes, as in the other passes,
+// consecutive lanes would store whole rows apart: the columns of such a tile ARE its rows); the k1 pitch is then
+// padded to 4 mod 8 words, which puts the sixteen k1 of a wavefront on different banks.
+// The 512-point kernel has no LDS to spare (with any padding of the k1 pitch a fourth workgroup no longer fits a CU):
+// there the n2 rows of a k1 block are rotated by 2 k1 instead, which spreads the sixteen k1 over the even banks.
+template <int A2>
+struct SglLds {
+    static constexpr int E2 = 1 << A2, T = TILE >> (4 + A2), ST = T + 1, RAW = E2 * ST;
+    static constexpr int S1 = A2 == 5 ? RAW : RAW + ((4 - RAW % 8) + 8) % 8;
+    static constexpr int WORDS = 16 * S1;
+};
+template <int A2, bool SGL>
+VI_HD int lds_slot(int st, int k1, int n2, int c) {
+    if constexpr (SGL && A2 == 5) return k1 * SglLds<A2>::S1 + ((n2 + 2 * k1) & 31) * SglLds<A2>::ST + c;
+    if constexpr (SGL) return k1 * SglLds<A2>::S1 + n2 * SglLds<A2>::ST + c;
+    return ((k1 << A2) + n2) * st + c;
+}
+
 // phase 2: optional coset pre-multiplier, 16-point transform, w_L^(n2 k1), into LDS
 // twi: w_L^(n2 k1) at [n2 * 16 + k1]
 // the coset pre-multipliers of this thread's sixteen inputs (a column that does not exist takes those of
@@ -374,7 +394,7 @@ VI_HD void fast_pre_load(const PassArgs &A, i64 tile, int tid, int t_loop, u64 (
     for (int n1 = 0; n1 < 16; ++n1) pw[n1] = pre[R.valid ? (i64)((n1 << A2) + n2) << sh : 0];
 }
 
-template <int A2, bool INV, bool HALF = false, bool TWT = false>
+template <int A2, bool INV, bool HALF = false, bool TWT = false, bool SGL = false>
 VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok, const u64 (&reg)[16],
                        const u64 (&pw)[16], const u64 *twi, u64 *lds) {
     int c, n2;
@@ -401,19 +421,46 @@ VI_HD void fast_stage1(const PassArgs &A, i64 tile, int tid, int t_loop, u32 ok,
         for (int k1 = g; k1 < g + 4; ++k1) {
             u64 v = x[k1];
             if (k1 > 0) v = gl::mul(v, twi[twi_slot<A2, TWT>(n2, k1)]);
-            lds[((k1 << A2) + n2) * st + c] = v;
+            lds[lds_slot<A2, SGL>(st, k1, n2, c)] = v;
         }
         VI_SCHED_FENCE();
     }
 }
 
 // phase 3: 16/E2 stage-2 transforms, inter-pass twiddle (or final scale), scatter
-template <int A2, bool INV, bool UNI>
+template <int A2, bool INV, bool UNI, bool SGL = false>
 VI_HD void fast_stage2(const PassArgs &A, i64 tile, int tid, int t_loop, const u64 *lds) {
     constexpr int E2 = 1 << A2;
     const int lt = logT(A);
     const int st = (1 << lt) + 1;
     const int c = tid & ((1 << lt) - 1);
+    if constexpr (SGL) {
+        // whole tiles of a single-pass transform: thread (k1 = low four bits, sixteen columns per trip), outputs
+        // k1 + 16 k2 of row c at word (c << a) + k1 + 16 k2 of the tile
+        static_assert(UNI, "whole tiles are addressed through scalar bases");
+        const TileU U = tile_uniform<A2>(A, tile);
+        const URun dst = urun(A.dst + U.dst_u);
+        const int k1 = tid & 15;
+#pragma unroll
+        for (int i = 0; i < 16 / E2; ++i) {
+            const int cc = (tid >> 4) + 16 * i;
+            const u32 off = ((u32)cc << U.shcd) + (u32)k1;
+            u64 x[E2];
+#pragma unroll
+            for (int n2 = 0; n2 < E2; ++n2) x[n2] = lds[lds_slot<A2, true>(st, k1, n2, cc)];
+            VI_SCHED_FENCE();
+            dft_reg<A2, INV>(x);
+            VI_SCHED_FENCE();
+#pragma unroll
+            for (int k2 = 0; k2 < E2; ++k2) {
+                u64 v = x[k2];
+                if (A.scale != 1) v = gl::mul(v, A.scale);
+                ustore_stream(dst, (u32)k2 << 4, off, v);
+                if ((k2 & 3) == 3) VI_SCHED_FENCE();
+            }
+        }
+        return;
+    }
     if constexpr (UNI) {
         const TileU U = tile_uniform<A2>(A, tile);
         const URun dst = urun(A.dst + U.dst_u + (A.is_final ? 0 : (i64)t_loop * A.dst_coset_stride));
@@ -488,14 +535,15 @@ VI_HD void fast_stage2_512(const PassArgs &A, i64 tile, int tid, const u64 *lds)
     constexpr int A2 = 5;
     const int lt = logT(A);                                // 3: eight columns per tile
     const int st = (1 << lt) + 1;
-    const int c = tid & ((1 << lt) - 1);
-    const int k1 = (tid >> lt) & 15, h = tid >> (lt + 4);
+    // UNI (whole tiles of contiguous rows): k1 along the lanes, see lds_slot
+    const int c = UNI ? (tid >> 4) & ((1 << lt) - 1) : tid & ((1 << lt) - 1);
+    const int k1 = UNI ? tid & 15 : (tid >> lt) & 15, h = tid >> (lt + 4);
     ColRef R{};
     if (!UNI) R = col_ref(A, tile, c);
     const int lc = A.B + A.log_rho;
     u64 x[32], y[16];
 #pragma unroll
-    for (int n2 = 0; n2 < 32; ++n2) x[n2] = lds[((k1 << A2) + n2) * st + c];
+    for (int n2 = 0; n2 < 32; ++n2) x[n2] = lds[lds_slot<A2, UNI>(st, k1, n2, c)];
     if (h == 0) {
 #pragma unroll
         for (int j = 0; j < 16; ++j) y[j] = gl::addc(x[j], x[j + 16]);
