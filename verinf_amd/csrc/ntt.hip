@@ -94,7 +94,15 @@ __global__ __launch_bounds__(NTHREADS, 4) void k_ntt_fast(const PassArgs A_in) {
     u64 reg[16], pw[16];
     u32 ok;
     if (A.pre) fast_pre_load<A2, UNI>(A, tile, tid, t, pw);
-    fast_load<A2, UNI, HALF>(A, tile, tid, reg, ok);
+    // A tile that only this workgroup reads is fetched with the streaming hint, like the stores: in a strided pass
+    // (except the one whose rho workgroups per tile share it through the L2), and in the final pass over 256-point
+    // digits.  Measured per kind of pass on two boxes: strided passes 0 to -0.2 % on the 2^16 -> 2^18 extension and
+    // -2.5 % on transforms of 2^20 points; final passes -0.3 to -1 % on the 2^16 -> 2^18 extension and -0.6 % on
+    // transforms of 2^16 points, but +1 % on the 2^14 -> 2^16 extension (128-point digits) and +6 % on transforms of
+    // 2^20 points (64-point digits).
+    constexpr bool STREAM = UNI && (!FIN || A2 == 4);
+    if (STREAM && !expand) fast_load<A2, UNI, HALF, STREAM>(A, tile, tid, reg, ok);
+    else fast_load<A2, UNI, HALF>(A, tile, tid, reg, ok);
     if (!A.is_final) {
         if (lane < count) twi[first + lane] = tw_wave;
         __builtin_amdgcn_wave_barrier();
@@ -189,7 +197,7 @@ __global__ __launch_bounds__(NTHREADS, VI_MID_MIN_WG) void k_lde_mid(const PassA
     }
     u64 reg[16], coef[16];
     u32 ok;
-    fast_load<A2, true>(Ai, tile, tid, reg, ok);
+    fast_load<A2, true, false, A2 == 4>(Ai, tile, tid, reg, ok);      // streaming where it measured faster, see k_ntt_fast
 #pragma unroll
     for (int i = 0; i < PER; ++i)
         if (tid + i * NTHREADS < (16 << A2)) {

@@ -240,6 +240,11 @@ __device__ __forceinline__ u64 uload(const URun &b, u32 uni, u32 off) {
     const vi_u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(b.r, off * 8u, uni * 8u, 0);
     return ((u64)v[1] << 32) | v[0];
 }
+// read once by this launch and by no later one
+__device__ __forceinline__ u64 uload_stream(const URun &b, u32 uni, u32 off) {
+    const vi_u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(b.r, off * 8u, uni * 8u, 2);
+    return ((u64)v[1] << 32) | v[0];
+}
 __device__ __forceinline__ void ustore(const URun &b, u32 uni, u32 off, u64 x) {
     const vi_u32x2 v = {(u32)x, (u32)(x >> 32)};
     __builtin_amdgcn_raw_buffer_store_b64(v, b.r, off * 8u, uni * 8u, 0);
@@ -257,6 +262,7 @@ __device__ __forceinline__ void ustore_stream(const URun &b, u32 uni, u32 off, u
 struct URun { u64 *p; };
 inline URun urun(const u64 *base) { return URun{const_cast<u64 *>(base)}; }
 inline u64 uload(const URun &b, u32 uni, u32 off) { return b.p[(size_t)uni + off]; }
+inline u64 uload_stream(const URun &b, u32 uni, u32 off) { return b.p[(size_t)uni + off]; }
 inline void ustore(const URun &b, u32 uni, u32 off, u64 x) { b.p[(size_t)uni + off] = x; }
 inline void ustore_stream(const URun &b, u32 uni, u32 off, u64 x) { b.p[(size_t)uni + off] = x; }
 #endif
@@ -288,7 +294,7 @@ VI_HD void s1_coords(const PassArgs &A, int tid, int &c, int &n2) {
 // before -- eight memory round trips per tile instead of one.
 // HALF (uniform passes whose source rows end within the first eight planes, upper_half_zero()): inputs 8 .. 15 are
 // not loaded.
-template <int A2, bool UNI, bool HALF = false>
+template <int A2, bool UNI, bool HALF = false, bool STREAM = false>
 VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &ok) {
     int c, n2;
     s1_coords<A2>(A, tid, c, n2);
@@ -300,7 +306,9 @@ VI_HD void fast_load(const PassArgs &A, i64 tile, int tid, u64 (&reg)[16], u32 &
         // for every thread, so it is made on the scalar base
         const URun src = urun(A.src + U.src_u);
 #pragma unroll
-        for (int n1 = 0; n1 < NL; ++n1) reg[n1] = uload(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off);
+        for (int n1 = 0; n1 < NL; ++n1)
+            reg[n1] = STREAM ? uload_stream(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off)
+                             : uload(src, (u32)(n1 < A.n1_valid ? n1 : 0) << U.sh1, off);
 #pragma unroll
         for (int n1 = NL; n1 < 16; ++n1) reg[n1] = 0;
         ok = A.n1_valid >= 16 ? 0xFFFFu : ((1u << A.n1_valid) - 1u);
