@@ -181,7 +181,7 @@ __global__ __launch_bounds__(BLOCK) void k_sum_partial(const u64 *a, i64 n, u64 
     for (; i + 3 * stride < n; i += 4 * stride) {     // four loads in flight
         u64 v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = a[i + u * stride];
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(&a[i + u * stride]);     // read once: streaming
 #pragma unroll
         for (int u = 0; u < 4; ++u) acc = gl::add(acc, v[u] >= gl::P ? v[u] - gl::P : v[u]);
     }
