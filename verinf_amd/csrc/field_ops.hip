@@ -25,7 +25,8 @@ __device__ __forceinline__ u64 apply(u64 a, u64 b) {
 template <int OP>
 __global__ __launch_bounds__(BLOCK) void k_binop(const u64 *a, const u64 *b, u64 *out, i64 n) {
     i64 stride = (i64)gridDim.x * BLOCK;
-    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride) out[i] = apply<OP>(a[i], b[i]);
+    for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n; i += stride)
+        __builtin_nontemporal_store(apply<OP>(__builtin_nontemporal_load(a + i), __builtin_nontemporal_load(b + i)), out + i);
 }
 
 // two elements per lane through 16-byte accesses (operands 16-byte aligned, n even)
@@ -33,10 +34,15 @@ template <int OP>
 __global__ __launch_bounds__(BLOCK) void k_binop_v2(const ulonglong2 *a, const ulonglong2 *b, ulonglong2 *out, i64 n2) {
     i64 stride = (i64)gridDim.x * BLOCK;
     for (i64 i = (i64)blockIdx.x * BLOCK + threadIdx.x; i < n2; i += stride) {
-        ulonglong2 x = a[i], y = b[i], r;
-        r.x = apply<OP>(x.x, y.x);
-        r.y = apply<OP>(x.y, y.y);
-        out[i] = r;
+        // operands read once, result not read back by this launch: streaming hints (2^24 elements 5.1 -> 5.9 TB/s,
+        // 2^27 4.40 -> 4.50 TB/s)
+        typedef u64 v2 __attribute__((ext_vector_type(2)));
+        const v2 xv = __builtin_nontemporal_load(reinterpret_cast<const v2 *>(a + i));
+        const v2 yv = __builtin_nontemporal_load(reinterpret_cast<const v2 *>(b + i));
+        v2 rv;
+        rv.x = apply<OP>(xv.x, yv.x);
+        rv.y = apply<OP>(xv.y, yv.y);
+        __builtin_nontemporal_store(rv, reinterpret_cast<v2 *>(out + i));
     }
 }
 
