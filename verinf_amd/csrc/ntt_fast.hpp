@@ -24,8 +24,10 @@
 // from displacing the source lines that the coset workgroups of a tile share in the L2.
 #if defined(__HIP_DEVICE_COMPILE__) && !defined(VI_PLAIN_STORES)
 #define VI_STREAM_STORE(p, v) __builtin_nontemporal_store((v), (p))
+#define VI_STREAM_LOAD(p) __builtin_nontemporal_load(p)
 #else
 #define VI_STREAM_STORE(p, v) (*(p) = (v))
+#define VI_STREAM_LOAD(p) (*(p))
 #endif
 
 namespace ntt {
@@ -767,7 +769,7 @@ VI_HD void row_stage0(const PassArgs &A, i64 tile, int tid, u64 *lds) {
             const i64 idx = ((i64)n1 << 8) + tid;
             const bool there = row < A.n_rows && idx < A.src_width;
             ok |= there ? (1u << (j * E0 + n1)) : 0u;
-            x[j * E0 + n1] = A.src[there ? row * A.src_row_stride + idx : 0];
+            x[j * E0 + n1] = VI_STREAM_LOAD(&A.src[there ? row * A.src_row_stride + idx : 0]);     // read once
         }
     }
     // w_n^(k r), the same for every row; row 0 of the table is 1 forward and 1/n inverse
