@@ -40,7 +40,7 @@ LDE_TRAFFIC_BYTES_PER_STEP = 8.06e9
 # 1024 SIMDs issue the instruction classes these kernels consist of (carry, multiply, three-operand and shift
 # instructions: one per 4.16 cycles per SIMD, measured by `bench.py --valu-probe`,
 # profiles/valu_issue_rates__probe.md) at the 2.4 GHz peak clock
-LDE_VALU_INSTS_PER_STEP = 2 * (58_687_488 + 290_062_336 + 188_088_320)
+LDE_VALU_INSTS_PER_STEP = 2 * (58_785_792 + 290_095_104 + 188_481_536)
 VALU_ISSUE_CYCLES_PER_INSTR = 4.16
 VALU_ISSUE_PEAK_PER_S = 256 * 4 * 2.4e9 / VALU_ISSUE_CYCLES_PER_INSTR
 
